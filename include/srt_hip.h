@@ -1,0 +1,231 @@
+/*
+ * srt_hip.h -- C ABI of the SwiftRTHip native module (MI355X / gfx950).
+ *
+ * This module fills, for the matmul / Dense path, the role that Sources/CCUDA (the clang
+ * module exposing the CUDA runtime) and Modules/SwiftRTCuda (the extern "C" srt* functions)
+ * fill in the reference.  A Swift `HipQueue` imports this header through a module map and
+ * calls it exactly where `CudaQueue` calls the CUDA runtime and the srt* functions.
+ *
+ * Conventions (same as the reference's native module):
+ *   - every function returns a status; srtSuccess == 0.
+ *   - srtErrorNotSupported means "caller, run your CPU fallback"
+ *     (role of cudaErrorNotSupported in cpuFallback,
+ *     Sources/SwiftRTCore/platform/cuda/device/CudaPlatform.swift:122-144).
+ *     Any other non-zero status is a hard error (the reference's cudaCheck resets the device
+ *     and traps, CudaPlatform.swift:180-193).
+ *   - the native side never throws, aborts or logs; it never retains tensor memory or
+ *     descriptor memory after a call returns (descriptors live on the caller's stack,
+ *     CudaExtensions.swift:24-84), and kernels are launched asynchronously on `stream`.
+ *   - data pointers are already offset to the first element of the view
+ *     (Tensor.deviceRead, Sources/SwiftRTCore/tensor/Tensor.swift:558-582); extents and
+ *     strides are 64-bit counts of elements.
+ *   - plain C types only: no C++ and no framework types cross this boundary.
+ */
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* every declaration below is exported from the shared library (it is built with hidden
+ * default visibility) */
+#pragma GCC visibility push(default)
+
+/* ---- status ---------------------------------------------------------------------------- */
+typedef int32_t srtStatus;
+enum {
+  srtSuccess = 0,
+  srtErrorInvalidValue = 1,      /* null pointer, rank/extent mismatch, bad enum value        */
+  srtErrorOutOfMemory = 2,       /* device or pinned-host allocation failed                   */
+  srtErrorNotReady = 600,        /* srtEventQuery: work not finished (not an error)           */
+  srtErrorNotSupported = 801,    /* run the CPU fallback (same value as cudaErrorNotSupported) */
+  srtErrorLaunchFailure = 719,   /* a launch or an asynchronous error was reported by HIP     */
+  srtErrorNoDevice = 100,        /* no gfx950 device visible / HIP runtime failed to start    */
+  srtErrorUnknown = 999
+};
+
+/* Human-readable name of a status; never NULL; storage is static. */
+const char* srtGetStatusString(srtStatus status);
+
+/* ---- element types ----------------------------------------------------------------------
+ * Replaces srtDataType, Modules/SwiftRTCuda/tensor_api.h:28-65.  The values the path uses keep
+ * the reference's numeric ids (they are the cudaDataType values) so `E.type` in
+ * StorageElement.swift:123-129 ports unchanged. */
+typedef enum {
+  srtUnknownType = -1,
+  srtReal32F = 0,
+  srtReal64F = 1,   /* declared for completeness; matmul returns srtErrorNotSupported */
+  srtReal16F = 2,
+  srtReal16BF = 14
+} srtDataType;
+
+/* Storage order.  Replaces the cublasLtOrder_t field of srtTensorDescriptor
+ * (tensor_api.h:76); same numeric values as CUBLASLT_ORDER_COL / CUBLASLT_ORDER_ROW, which is
+ * what `order.cublas` yields (CudaPlatform.swift:297-311).  Strides are authoritative; order
+ * is checked only to reject tiled layouts (anything else -> srtErrorNotSupported). */
+typedef enum { srtOrderCol = 0, srtOrderRow = 1 } srtOrder;
+
+/* Tensor descriptor.  Replaces srtTensorDescriptor, tensor_api.h:70-87, field for field, so
+ * Tensor.withTensor (CudaExtensions.swift:24-84) builds it the same way.  shape / strides /
+ * logicalStrides point at `rank` values on the caller's stack; they are read during the call
+ * only. */
+typedef struct {
+  srtDataType type;             /* element type                                              */
+  uint32_t rank;                /* number of dimensions                                      */
+  srtOrder order;               /* storage order                                             */
+  size_t count;                 /* number of logical elements                                */
+  size_t spanCount;             /* number of storage elements spanned                        */
+  const size_t* shape;          /* extent of each dimension                                  */
+  const size_t* strides;        /* storage stride of each dimension, in elements             */
+  const size_t* logicalStrides; /* dense logical strides (unused by matmul, may be NULL)     */
+} srtTensorDescriptor;
+
+/* Epilogue activation.  Case order and values follow ActivationType,
+ * Sources/SwiftRTCore/platform/common/FunctionProperties.swift:44-51 (rawValue ports 1:1). */
+typedef enum {
+  srtActivationSigmoid = 0,     /* 1 / (1 + exp(-x))                                         */
+  srtActivationRelu = 1,        /* max(x, 0)                                                 */
+  srtActivationTanh = 2,
+  srtActivationClippedRelu = 3, /* min(max(x, 0), coef)   coef = activationReluCeiling       */
+  srtActivationElu = 4,         /* x > 0 ? x : coef * (exp(x) - 1)                           */
+  srtActivationIdentity = 5
+} srtActivation;
+
+/* Opaque handles.  A stream is a HIP stream; an event a HIP event. */
+typedef struct srtStream_st* srtStream;
+typedef struct srtEvent_st* srtEvent;
+
+/* ---- device ------------------------------------------------------------------------------ */
+/* Replaces cudaGetDeviceCount (CudaPlatform.swift:89). */
+srtStatus srtGetDeviceCount(int32_t* count);
+/* Replaces cudaSetDevice (CudaQueue.swift:62,78; CudaDevice.swift:70). */
+srtStatus srtSetDevice(int32_t device);
+srtStatus srtGetDevice(int32_t* device);
+
+typedef struct {
+  char name[256];
+  char archName[64];           /* e.g. "gfx950:sramecc+:xnack-"                               */
+  size_t totalGlobalMem;       /* bytes                                                       */
+  int32_t multiProcessorCount; /* compute units                                               */
+  int32_t clockRateKHz;        /* peak engine clock                                           */
+  int32_t memoryClockRateKHz;
+  int32_t memoryBusWidthBits;
+  int32_t l2CacheBytes;
+  int32_t sharedMemPerBlockBytes; /* LDS available to one workgroup                           */
+  int32_t warpSize;            /* 64                                                          */
+} srtDeviceProperties;
+/* Replaces cudaGetDeviceProperties (CudaDevice.swift:88). */
+srtStatus srtGetDeviceProperties(srtDeviceProperties* props, int32_t device);
+/* Blocks until every stream of the current device is idle (cudaDeviceSynchronize role). */
+srtStatus srtDeviceSynchronize(void);
+
+/* ---- streams ----------------------------------------------------------------------------- */
+/* Replaces cudaStreamCreateWithFlags(.., cudaStreamNonBlocking) (CudaQueue.swift:65-68).
+ * Streams are created at default priority on the current device. */
+srtStatus srtStreamCreate(srtStream* stream);
+srtStatus srtStreamDestroy(srtStream stream);
+/* Replaces cudaStreamSynchronize (CudaQueue.swift:193). */
+srtStatus srtStreamSynchronize(srtStream stream);
+
+/* ---- events ------------------------------------------------------------------------------ */
+/* Replaces cudaEventCreateWithFlags (CudaEvent.swift:48-50).  enableTiming != 0 makes the
+ * event usable with srtEventElapsedTime. */
+srtStatus srtEventCreate(srtEvent* event, int32_t enableTiming);
+/* Replaces cudaEventDestroy (CudaEvent.swift:55). */
+srtStatus srtEventDestroy(srtEvent event);
+/* Replaces cudaEventRecord (CudaQueue.swift:159). */
+srtStatus srtEventRecord(srtEvent event, srtStream stream);
+/* Replaces cudaStreamWaitEvent (CudaQueue.swift:175). */
+srtStatus srtStreamWaitEvent(srtStream stream, srtEvent event);
+/* Replaces cudaEventSynchronize (CudaEvent.swift:62,70). */
+srtStatus srtEventSynchronize(srtEvent event);
+/* srtSuccess when complete, srtErrorNotReady otherwise (cudaEventQuery role). */
+srtStatus srtEventQuery(srtEvent event);
+srtStatus srtEventElapsedTime(float* milliseconds, srtEvent start, srtEvent stop);
+
+/* ---- memory ------------------------------------------------------------------------------ */
+/* Replace srtDeviceAllocate / srtDeviceFree, Modules/SwiftRTCuda/memory_api.h:26-27 (called
+ * from CudaDeviceMemory, CudaDevice.swift:147,159).  Stream-ordered caching allocator: a
+ * freed block is reused at once on the stream it was last used on, and on other streams once
+ * the work queued on that stream at the time of the free has finished.  Thread safe.  The
+ * caller owns the pointer; the library keeps no reference to tensor memory. */
+srtStatus srtDeviceAllocate(void** devPtr, size_t size, srtStream stream);
+srtStatus srtDeviceFree(void* devPtr);
+/* Returns every cached (free) block of every device to the driver. */
+srtStatus srtDeviceEmptyCache(void);
+/* Pinned host staging memory (newly allocated, never registered in place). */
+srtStatus srtHostAllocate(void** hostPtr, size_t size);
+srtStatus srtHostFree(void* hostPtr);
+
+typedef enum {
+  srtMemcpyHostToDevice = 1,
+  srtMemcpyDeviceToHost = 2,
+  srtMemcpyDeviceToDevice = 3
+} srtMemcpyKind;
+/* Replaces cudaMemcpyAsync (CudaQueue.swift:125-151): ordered on `stream`; host buffers may
+ * be pageable. */
+srtStatus srtMemcpyAsync(void* dst, const void* src, size_t byteCount, srtMemcpyKind kind,
+                         srtStream stream);
+/* Fills byteCount bytes with `value` on `stream` using a fill kernel (safe to capture). */
+srtStatus srtMemsetAsync(void* dst, int32_t value, size_t byteCount, srtStream stream);
+
+/* ---- matmul ------------------------------------------------------------------------------
+ * out = op(a) . op(b), op = optional swap of the last two dimensions (`Tensor.t`,
+ * Sources/SwiftRTCore/tensor/TensorInit.swift:844-890).  Rank 2, or rank 3 with a leading
+ * batch dimension (batch stride taken from strides[0]; 0 broadcasts an operand).
+ *
+ * This is the entry point HipQueue.matmul calls, for both overloads, in place of the
+ * cpuFallback in CudaQueue.matmul (Sources/SwiftRTCore/platform/cuda/functions/
+ * CudaMatmul.swift:25-42 and :44-61); the arithmetic it replaces is cpu_matmul
+ * (Sources/SwiftRTCore/platform/cpu/functions/CpuMath.swift:1141-1161, :1164-1186).
+ * Elements: srtReal32F, srtReal16F, srtReal16BF, all three tensors the same type.  Products
+ * are accumulated in fp32 and rounded once (nearest even) to the element type.
+ * Operands may be any strided view; `out` may have any strides that do not alias.
+ *
+ * Returns srtErrorNotSupported (caller falls back to the CPU) for other element types,
+ * orders other than row/col, or rank other than 2/3; srtErrorInvalidValue when extents do not
+ * agree; srtSuccess with no launch when any extent is zero. */
+srtStatus srtMatmul(const void* a, const srtTensorDescriptor* aDesc, int32_t transposeA,
+                    const void* b, const srtTensorDescriptor* bDesc, int32_t transposeB,
+                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+
+/* out = activation(op(a) . op(b) + bias), bias broadcast over rows, bias and activation applied
+ * to the fp32 accumulators in registers before the single rounding to the element type.
+ * This is the Dense forward: it implements what matmul(_:transposed:_:transposed:bias:)
+ * (Sources/SwiftRTCore/operators/Matmul.swift:57-72, which drops its bias) and
+ * Dense.callAsFunction (Sources/SwiftRTLayers/Dense.swift:36-39, a stub) are meant to compute,
+ * and what the recurrent cells compute today as three ops
+ * (Sources/SwiftRTLayers/Recurrent.swift:157-161, :255-266).
+ * bias: rank-1 tensor of N elements of the same type (bias == NULL: no bias add).
+ * coef: ceiling for srtActivationClippedRelu, alpha for srtActivationElu, ignored otherwise.
+ * Rank 2 or 3 as srtMatmul (the same bias is applied to every batch). */
+srtStatus srtMatmulBiasActivation(const void* a, const srtTensorDescriptor* aDesc, int32_t transposeA,
+                                  const void* b, const srtTensorDescriptor* bDesc, int32_t transposeB,
+                                  const void* bias, const srtTensorDescriptor* biasDesc,
+                                  srtActivation activation, double coef,
+                                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+
+/* Name of the kernel family the dispatcher selects for this problem ("mfma_256x256",
+ * "skinny", "generic", ...), written into `name`; nothing is launched.  Diagnostic only
+ * (the reference's matmul diagnostic line, CudaMatmul.swift:34-37, has no counterpart for
+ * kernel choice). */
+srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transposeA,
+                               const srtTensorDescriptor* bDesc, int32_t transposeB,
+                               const srtTensorDescriptor* oDesc, const void* a, const void* b,
+                               const void* out, char* name, size_t nameCapacity);
+
+/* ---- test helper ------------------------------------------------------------------------- */
+/* Replaces srtDelayStream, Modules/SwiftRTCuda/utilities_api.h:28: occupies `stream` for about
+ * `seconds` (bounded spin on the device clock; at most 10 s). */
+srtStatus srtDelayStream(double seconds, srtStream stream);
+
+/* Library version: major * 10000 + minor * 100 + patch. */
+int32_t srtGetVersion(void);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif

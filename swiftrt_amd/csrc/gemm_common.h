@@ -1,0 +1,122 @@
+// Shared definitions for the matmul kernels: the normalized problem, element codecs and
+// the fused bias + activation epilogue.  gfx950 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/srt_hip.h"
+
+namespace srt {
+
+// A matmul after the caller's transposes, orders and views have been folded into strides.
+// op(A)[m,k] = A[m*sam + k*sak], op(B)[k,n] = B[k*sbk + n*sbn], C[m,n] = C[m*scm + n*scn];
+// batch b adds b*sab / b*sbb / b*scb.  All strides are in elements.
+struct GemmProblem {
+  int dtype;  // srtDataType
+  int M, N, K, batch;
+  const void* A;
+  const void* B;
+  void* C;
+  const void* bias;  // may be null
+  long long sam, sak, sab;
+  long long sbk, sbn, sbb;
+  long long scm, scn, scb;
+  long long sbias;  // stride between bias elements
+  int bias_per_row;  // 0: bias indexed by column n (the Dense case); 1: by row m (after a C^T flip)
+  int activation;    // srtActivation
+  float coef;
+};
+
+// ---- element codecs ---------------------------------------------------------------------
+struct BF16 {
+  using storage = uint16_t;
+  static constexpr int dtype = srtReal16BF;
+  static __device__ __forceinline__ float to_float(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+  // round to nearest even; NaN -> 0x7FFF.  Same rule as BFloat16.float2bfloat16_rn in the
+  // reference (platform/common/BFloat16.swift:53-80).
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return 0x7fff;
+    return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+  }
+};
+
+struct F16 {
+  using storage = uint16_t;
+  static constexpr int dtype = srtReal16F;
+  static __device__ __forceinline__ float to_float(uint16_t h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+  }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    _Float16 v = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+  }
+};
+
+struct F32 {
+  using storage = float;
+  static constexpr int dtype = srtReal32F;
+  static __device__ __forceinline__ float to_float(float v) { return v; }
+  static __device__ __forceinline__ float from_float(float v) { return v; }
+};
+
+// ---- epilogue ---------------------------------------------------------------------------
+// Activation on the fp32 accumulator.  Definitions follow the reference where it has one
+// (sigmoid: CpuMath.swift:1369-1377; tanh: libm) and cuDNN's for the rest.
+__device__ __forceinline__ float apply_activation(int activation, float coef, float x) {
+  switch (activation) {
+    case srtActivationSigmoid: return 1.0f / (1.0f + expf(-x));
+    case srtActivationRelu: return x > 0.0f ? x : 0.0f;
+    case srtActivationTanh: return tanhf(x);
+    case srtActivationClippedRelu: {
+      float y = x > 0.0f ? x : 0.0f;
+      return y < coef ? y : coef;
+    }
+    case srtActivationElu: return x > 0.0f ? x : coef * (expf(x) - 1.0f);
+    default: return x;
+  }
+}
+
+// Epilogue state for one output column (or row) set; bias is read as element type T.
+template <typename T>
+struct Epilogue {
+  const typename T::storage* bias;
+  long long sbias;
+  int per_row;
+  int activation;
+  float coef;
+  __device__ __forceinline__ explicit Epilogue(const GemmProblem& p)
+      : bias((const typename T::storage*)p.bias), sbias(p.sbias), per_row(p.bias_per_row),
+        activation(p.activation), coef(p.coef) {}
+  __device__ __forceinline__ float bias_at(int m, int n) const {
+    if (!bias) return 0.0f;
+    return T::to_float(bias[(long long)(per_row ? m : n) * sbias]);
+  }
+  __device__ __forceinline__ typename T::storage finish(float acc, float b) const {
+    float v = acc + b;
+    if (activation != srtActivationIdentity) v = apply_activation(activation, coef, v);
+    return T::from_float(v);
+  }
+};
+
+// ---- launchers (one per kernel family), defined in the .hip files ------------------------
+// Each returns hipSuccess/hip error from the launch; `name` receives the kernel family.
+bool generic_supported(const GemmProblem& p);
+hipError_t launch_generic(const GemmProblem& p, hipStream_t stream);
+
+// Tile configuration chosen for the MFMA family, or 0 if the problem does not qualify.
+int mfma_select(const GemmProblem& p);
+const char* mfma_name(int config);
+hipError_t launch_mfma(const GemmProblem& p, int config, hipStream_t stream);
+
+bool skinny_supported(const GemmProblem& p);
+hipError_t launch_skinny(const GemmProblem& p, hipStream_t stream);
+
+bool f32_mfma_supported(const GemmProblem& p);
+hipError_t launch_f32_mfma(const GemmProblem& p, hipStream_t stream);
+
+}  // namespace srt

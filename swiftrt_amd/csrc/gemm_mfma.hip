@@ -1,0 +1,345 @@
+// bf16 / fp16 matmul on the gfx950 matrix cores: v_mfma_f32_32x32x16 tiles, fp32
+// accumulation in registers, double-buffered LDS staging, fused bias + activation epilogue.
+//
+// Work decomposition
+//   grid    one workgroup per BM x BN tile of C (x batch); workgroup ids are remapped so that
+//           the workgroups resident on one XCD (ids congruent mod 8) cover a compact patch of
+//           tiles and share A row panels / B column panels in that XCD's L2.
+//   block   4 waves in a 2 x 2 arrangement; each wave owns (BM/2) x (BN/2) of the tile as
+//           TM x TN MFMA tiles of 32 x 32, i.e. TM*TN*16 fp32 accumulators per lane.
+//   k loop  BK = 64 per stage; global loads for stage t+1 are issued before the MFMAs of
+//           stage t and written to the other LDS buffer afterwards (one barrier per stage).
+//
+// LDS layout (both operands, all four transpose cases): row r of the tile (an m for A, an n
+// for B) holds its 64 k-values contiguously (128 bytes) as eight 16-byte chunks; chunk c is
+// stored at position c ^ f(r), f(r) = ((r >> 1) ^ (r >> 4)) & 7.  An MFMA operand read is one
+// ds_read_b128 per lane (lane l: row l % 32, chunk 2*kk + l / 32) and the XOR spreads the 16
+// lanes that share an LDS pass over all 64 banks.  What differs per transpose flag is only how
+// the tile gets there:
+//   operand stored k-contiguous  (A not transposed / B transposed): 16-byte global loads along
+//       k, written to LDS as they are;
+//   operand stored mn-contiguous (A transposed / B not transposed): each thread loads an
+//       8(k) x 8(mn) block as eight 16-byte rows (coalesced along mn), transposes it in
+//       registers with 32 v_perm_b32 and writes eight k-contiguous chunks.
+#include "gemm_common.h"
+
+namespace srt {
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int BK = 64;          // k depth of one LDS stage
+constexpr int ROW_BYTES = 128;  // BK * 2 bytes
+constexpr int NT = 256;         // threads per workgroup (4 waves)
+
+template <typename T>
+__device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c);
+
+template <>
+__device__ __forceinline__ f32x16_t mfma32<BF16>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                 c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16_t mfma32<F16>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b),
+                                                c, 0, 0, 0);
+}
+
+__device__ __forceinline__ int swz(int row) { return ((row >> 1) ^ (row >> 4)) & 7; }
+
+__device__ __forceinline__ uint32_t lds_off(int row, int chunk) {
+  return (uint32_t)(row * ROW_BYTES + ((chunk ^ swz(row)) << 4));
+}
+
+// ---- global -> register staging --------------------------------------------------------------
+// K-contiguous operand: R rows x 64 k.  Thread t owns chunk t % 8 of rows t / 8 + 32 i.
+template <int R>
+struct StageK {
+  static constexpr int CH = R * 8 / NT;
+  u32x4_t v[CH];
+
+  __device__ __forceinline__ void load(const uint16_t* base, long long ld, int row0, int rows_total, int k0, int K,
+                                       int tid) {
+    const int chunk = tid & 7;
+    const int k = k0 + chunk * 8;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int row = row0 + (tid >> 3) + 32 * i;
+      u32x4_t x = {0u, 0u, 0u, 0u};
+      if (row < rows_total && k < K) x = *reinterpret_cast<const u32x4_t*>(base + (long long)row * ld + k);
+      v[i] = x;
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned char* lds, int tid) const {
+    const int chunk = tid & 7;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int row = (tid >> 3) + 32 * i;
+      *reinterpret_cast<u32x4_t*>(lds + lds_off(row, chunk)) = v[i];
+    }
+  }
+};
+
+// MN-contiguous operand: 64 k x R mn, element (k, mn) at base[k * ld + mn].  Thread t (< R)
+// owns the 8 x 8 block k-group t / (R/8), mn-group t % (R/8).
+template <int R>
+struct StageMN {
+  static constexpr int GROUPS = R / 8;
+  u32x4_t v[8];
+
+  __device__ __forceinline__ void load(const uint16_t* base, long long ld, int mn0, int mn_total, int k0, int K,
+                                       int tid) {
+    if (R < NT && tid >= R) return;
+    const int mn = mn0 + (tid % GROUPS) * 8;
+    const int kb = k0 + (tid / GROUPS) * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      u32x4_t x = {0u, 0u, 0u, 0u};
+      if (mn < mn_total && kb + j < K) x = *reinterpret_cast<const u32x4_t*>(base + (long long)(kb + j) * ld + mn);
+      v[j] = x;
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned char* lds, int tid) const {
+    if (R < NT && tid >= R) return;
+    const int g = tid % GROUPS;
+    const int kg = tid / GROUPS;
+    // neighbouring lanes start on rows of opposite parity so one LDS pass covers all banks:
+    // at step jj a lane writes row jj ^ (g & 1).  The source dword (jj >> 1) is the same for
+    // both rows of a pair; only the half-word selector depends on the lane.
+    const uint32_t sel_lo = 0x05040100u, sel_hi = 0x07060302u;
+    const uint32_t sel_even = (g & 1) ? sel_hi : sel_lo;  // selector used at even jj
+    const uint32_t sel_odd = (g & 1) ? sel_lo : sel_hi;
+#pragma unroll
+    for (int jj = 0; jj < 8; ++jj) {
+      const int n = jj ^ (g & 1);
+      const uint32_t sel = (jj & 1) ? sel_odd : sel_even;
+      u32x4_t o;
+      // o[d] = { v[2d][n] , v[2d+1][n] } as two 16-bit halves: one byte-permute per dword
+#pragma unroll
+      for (int d = 0; d < 4; ++d) o[d] = __builtin_amdgcn_perm(v[2 * d + 1][jj >> 1], v[2 * d][jj >> 1], sel);
+      const int row = g * 8 + n;
+      *reinterpret_cast<u32x4_t*>(lds + lds_off(row, kg)) = o;
+    }
+  }
+};
+
+template <int R, bool KCONTIG>
+struct Stage;
+template <int R>
+struct Stage<R, true> : StageK<R> {};
+template <int R>
+struct Stage<R, false> : StageMN<R> {};
+
+// XCD-aware remap of the linear workgroup id followed by a grouped tile order.
+// Workgroups are handed to the 8 XCDs round-robin, so ids congruent mod 8 share an L2.  The
+// remap gives each XCD a contiguous range of logical ids; the grouped order walks GROUP_M tile
+// rows at a time so a contiguous range is a compact patch of the tile grid.
+__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int* tm, int* tn) {
+  const int nwg = tiles_m * tiles_n;
+  constexpr int XCDS = 8;
+  int logical = wg;
+  if (nwg >= XCDS * 4) {
+    const int per = (nwg + XCDS - 1) / XCDS;
+    int tall = nwg % XCDS;
+    if (tall == 0) tall = XCDS;
+    const int xcd = wg % XCDS, local = wg / XCDS;
+    logical = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+  }
+  constexpr int GROUP_M = 8;
+  const int per_group = GROUP_M * tiles_n;
+  const int group = logical / per_group;
+  const int first_m = group * GROUP_M;
+  const int gsize = min(tiles_m - first_m, GROUP_M);
+  const int in_group = logical - group * per_group;
+  *tm = first_m + in_group % gsize;
+  *tn = in_group / gsize;
+}
+
+template <typename T, int BM, int BN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
+  constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+  constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, &tm, &tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int bz = blockIdx.y;
+
+  const uint16_t* A = (const uint16_t*)p.A + (long long)bz * p.sab;
+  const uint16_t* B = (const uint16_t*)p.B + (long long)bz * p.sbb;
+  const long long lda = A_KC ? p.sam : p.sak;  // stride of the non-contiguous dimension
+  const long long ldb = B_KC ? p.sbn : p.sbk;
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  Stage<BM, A_KC> sa;
+  Stage<BN, B_KC> sb;
+  const int KT = (p.K + BK - 1) / BK;
+
+  sa.load(A, lda, m0, p.M, 0, p.K, tid);
+  sb.load(B, ldb, n0, p.N, 0, p.K, tid);
+  sa.store(lds, tid);
+  sb.store(lds + A_BYTES, tid);
+  __syncthreads();
+
+  const int frow = lane & 31;
+  const int fch = lane >> 5;
+
+  for (int kt = 0; kt < KT; ++kt) {
+    unsigned char* cur = lds + (kt & 1) * STAGE_BYTES;
+    unsigned char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+    const bool more = kt + 1 < KT;
+    if (more) {
+      sa.load(A, lda, m0, p.M, (kt + 1) * BK, p.K, tid);
+      sb.load(B, ldb, n0, p.N, (kt + 1) * BK, p.K, tid);
+    }
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      u32x4_t af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const u32x4_t*>(cur + lds_off(wm0 + 32 * i + frow, 2 * kk + fch));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bf[j] = *reinterpret_cast<const u32x4_t*>(cur + A_BYTES + lds_off(wn0 + 32 * j + frow, 2 * kk + fch));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
+    }
+    if (more) {
+      sa.store(nxt, tid);
+      sb.store(nxt + A_BYTES, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds column l % 32 and rows 8*(v/4) + 4*(l/32) + v%4 of each 32 x 32 tile
+  Epilogue<T> ep(p);
+  uint16_t* C = (uint16_t*)p.C + (long long)bz * p.scb;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn0 + 32 * j + (lane & 31);
+    if (n >= p.N) continue;
+    const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm0 + 32 * i + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (m >= p.M) continue;
+        const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
+        C[(long long)m * p.scm + n] = ep.finish(acc[i][j][v], bv);
+      }
+    }
+  }
+}
+
+// config ids: tile << 2 | a_kc << 1 | b_kc ; tile 1: 256x256, 2: 128x128, 3: 64x64
+template <typename T, int BM, int BN, bool A_KC, bool B_KC>
+hipError_t launch_one(const GemmProblem& p, hipStream_t stream) {
+  constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROW_BYTES;
+  auto kernel = gemm_mfma_kernel<T, BM, BN, A_KC, B_KC>;
+  if (lds_bytes > 64 * 1024) {
+    static bool configured = false;  // benign race: the attribute is idempotent
+    if (!configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+      if (e != hipSuccess) return e;
+      configured = true;
+    }
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);
+  return hipGetLastError();
+}
+
+template <typename T, int BM, int BN>
+hipError_t launch_layout(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_one<T, BM, BN, true, true>(p, stream);
+  if (a_kc && !b_kc) return launch_one<T, BM, BN, true, false>(p, stream);
+  if (!a_kc && b_kc) return launch_one<T, BM, BN, false, true>(p, stream);
+  return launch_one<T, BM, BN, false, false>(p, stream);
+}
+
+template <typename T>
+hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hipStream_t stream) {
+  switch (tile) {
+    case 1: return launch_layout<T, 256, 256>(p, a_kc, b_kc, stream);
+    case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
+    default: return launch_layout<T, 64, 64>(p, a_kc, b_kc, stream);
+  }
+}
+
+inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+}  // namespace
+
+// The MFMA family needs: a 16-bit element type, C rows contiguous, each operand contiguous
+// along k or along its other dimension with 16-byte aligned rows, and extents along the
+// contiguous dimensions that are multiples of 8 (so every 16-byte load is whole).
+int mfma_select(const GemmProblem& p) {
+  if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
+  if (p.scn != 1 || p.K < 1) return 0;
+  if (p.batch > 65535) return 0;
+  bool a_kc, b_kc;
+  if (p.sak == 1 && (p.K % 8) == 0) a_kc = true;
+  else if (p.sam == 1 && (p.M % 8) == 0) a_kc = false;
+  else return 0;
+  if (p.sbk == 1 && (p.K % 8) == 0) b_kc = true;
+  else if (p.sbn == 1 && (p.N % 8) == 0) b_kc = false;
+  else return 0;
+  const long long lda = a_kc ? p.sam : p.sak, ldb = b_kc ? p.sbn : p.sbk;
+  // a single row/column operand may carry any leading stride; otherwise rows must stay aligned
+  if ((lda % 8) != 0 || (ldb % 8) != 0) return 0;
+  if ((p.sab % 8) != 0 || (p.sbb % 8) != 0) return 0;
+  if (!aligned16(p.A) || !aligned16(p.B)) return 0;
+  if (p.sam < 0 || p.sak < 0 || p.sbk < 0 || p.sbn < 0 || p.scm < 0) return 0;
+
+  auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
+  int tile;
+  if (tiles(256) >= 192) tile = 1;
+  else if (tiles(128) >= 192) tile = 2;
+  else if (p.M > 64 && p.N > 64 && tiles(128) * 4 >= tiles(64)) tile = tiles(128) >= 64 ? 2 : 3;
+  else tile = 3;
+  return (tile << 2) | (a_kc ? 2 : 0) | (b_kc ? 1 : 0);
+}
+
+const char* mfma_name(int config) {
+  switch (config >> 2) {
+    case 1: return "mfma_256x256";
+    case 2: return "mfma_128x128";
+    default: return "mfma_64x64";
+  }
+}
+
+hipError_t launch_mfma(const GemmProblem& p, int config, hipStream_t stream) {
+  const int tile = config >> 2;
+  const bool a_kc = (config & 2) != 0, b_kc = (config & 1) != 0;
+  if (p.dtype == srtReal16BF) return launch_tile<BF16>(p, tile, a_kc, b_kc, stream);
+  return launch_tile<F16>(p, tile, a_kc, b_kc, stream);
+}
+
+}  // namespace srt

@@ -1,0 +1,241 @@
+"""HIP platform: device, queue, event and device-memory types above the C ABI.
+
+Python mirror of the roles the reference's CUDA platform fills
+(Sources/SwiftRTCore/platform/cuda/device/CudaPlatform.swift, CudaDevice.swift,
+CudaQueue.swift, CudaEvent.swift), used by the tests and the benchmark to drive the C ABI
+the way a Swift `HipQueue` would.  It holds no arithmetic: every operation is a native call.
+"""
+import ctypes
+import itertools
+import threading
+
+from . import native
+from .native import check
+
+_queue_ids = itertools.count(1)
+
+
+class HipEvent:
+    """Role of CudaEvent (CudaEvent.swift:43-75): owns a native event, destroyed with the object."""
+
+    def __init__(self, timing=False):
+        h = ctypes.c_void_p()
+        check(native.lib().srtEventCreate(ctypes.byref(h), 1 if timing else 0), "srtEventCreate")
+        self.handle = h
+        self.recorded = False
+
+    def wait(self):
+        if self.recorded:
+            check(native.lib().srtEventSynchronize(self.handle), "srtEventSynchronize")
+
+    @property
+    def occurred(self):
+        if not self.recorded:
+            return True
+        st = native.lib().srtEventQuery(self.handle)
+        if st == native.ERROR_NOT_READY:
+            return False
+        check(st, "srtEventQuery")
+        return True
+
+    def elapsed_ms_since(self, start):
+        ms = ctypes.c_float()
+        check(native.lib().srtEventElapsedTime(ctypes.byref(ms), start.handle, self.handle), "srtEventElapsedTime")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.handle:
+                native.lib().srtEventDestroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class HipDeviceMemory:
+    """Role of CudaDeviceMemory (CudaDevice.swift:96-162): the host object owns the pointer and
+    frees it when released; byte count padded to a multiple of 32 as the reference does."""
+
+    def __init__(self, device_index, byte_count, queue):
+        self.device_index = device_index
+        self.byte_count = int(byte_count)
+        padded = (self.byte_count + 31) // 32 * 32
+        p = ctypes.c_void_p()
+        check(native.lib().srtDeviceAllocate(ctypes.byref(p), max(padded, 32), queue.stream), "srtDeviceAllocate")
+        self.pointer = p.value
+        self.version = -1
+        self.name = None
+
+    def __del__(self):
+        try:
+            if self.pointer:
+                native.lib().srtDeviceFree(ctypes.c_void_p(self.pointer))
+                self.pointer = None
+        except Exception:
+            pass
+
+
+class HipQueue:
+    """Role of CudaQueue (CudaQueue.swift:22-196): one non-blocking stream on one device."""
+
+    def __init__(self, device_index, gpu_id, name):
+        self.id = next(_queue_ids)
+        self.device_index = device_index
+        self.gpu_id = gpu_id
+        self.name = name
+        self.creator_thread = threading.get_ident()
+        self.uses_cpu = False
+        self.memory_type = "discrete"
+        self.mode = "async"
+        L = native.lib()
+        check(L.srtSetDevice(gpu_id), "srtSetDevice")
+        s = ctypes.c_void_p()
+        check(L.srtStreamCreate(ctypes.byref(s)), "srtStreamCreate")
+        self.stream = s
+
+    def select(self):
+        check(native.lib().srtSetDevice(self.gpu_id), "srtSetDevice")
+
+    # -- DeviceQueue protocol (platform/common/DeviceQueue.swift:22-82) -----------------------
+    def allocate(self, byte_count, heap_index=0):
+        self.select()
+        return HipDeviceMemory(self.device_index, byte_count, self)
+
+    def copy_to_device(self, host_ptr, dst, byte_count):
+        check(native.lib().srtMemcpyAsync(ctypes.c_void_p(dst.pointer), ctypes.c_void_p(host_ptr), byte_count,
+                                          native.H2D, self.stream), "srtMemcpyAsync(H2D)")
+
+    def copy_to_host(self, src, host_ptr, byte_count):
+        check(native.lib().srtMemcpyAsync(ctypes.c_void_p(host_ptr), ctypes.c_void_p(src.pointer), byte_count,
+                                          native.D2H, self.stream), "srtMemcpyAsync(D2H)")
+
+    def copy_async(self, src, dst):
+        n = min(src.byte_count, dst.byte_count)
+        check(native.lib().srtMemcpyAsync(ctypes.c_void_p(dst.pointer), ctypes.c_void_p(src.pointer), n,
+                                          native.D2D, self.stream), "srtMemcpyAsync(D2D)")
+
+    def record_event(self, timing=False):
+        ev = HipEvent(timing=timing)
+        check(native.lib().srtEventRecord(ev.handle, self.stream), "srtEventRecord")
+        ev.recorded = True
+        return ev
+
+    def wait(self, event):
+        if event.recorded:
+            check(native.lib().srtStreamWaitEvent(self.stream, event.handle), "srtStreamWaitEvent")
+
+    def wait_for_completion(self):
+        check(native.lib().srtStreamSynchronize(self.stream), "srtStreamSynchronize")
+
+    def delay(self, seconds):
+        check(native.lib().srtDelayStream(float(seconds), self.stream), "srtDelayStream")
+
+    # -- the matmul path ---------------------------------------------------------------------
+    def matmul(self, lhs, transpose_lhs, rhs, transpose_rhs, result, bias=None, activation=None, coef=0.0):
+        """Role of CudaQueue.matmul (platform/cuda/functions/CudaMatmul.swift:25-61), rank 2 and 3.
+
+        Operands are moved to this queue's device if stale (Tensor.device_read, the role of
+        Tensor.deviceRead), descriptors are built per call and the native entry point is invoked
+        on this queue's stream.  srtErrorNotSupported surfaces as NotSupportedError: a Swift
+        caller would run its own cpu_matmul there; this module has no CPU arithmetic."""
+        from .tensor import ActivationType
+        self.select()
+        a_ptr = lhs.device_read(self)
+        b_ptr = rhs.device_read(self)
+        bias_ptr = bias.device_read(self) if bias is not None else None
+        o_ptr = result.device_read_write(self)
+        ad, ka = lhs.descriptor()
+        bd, kb = rhs.descriptor()
+        od, ko = result.descriptor()
+        L = native.lib()
+        if bias is None and activation in (None, ActivationType.identity):
+            st = L.srtMatmul(a_ptr, ctypes.byref(ad), int(transpose_lhs), b_ptr, ctypes.byref(bd), int(transpose_rhs),
+                             o_ptr, ctypes.byref(od), self.stream)
+        else:
+            act = ActivationType.identity if activation is None else activation
+            if bias is not None:
+                biasd, kbias = bias.descriptor()
+                biasd_ref = ctypes.byref(biasd)
+            else:
+                biasd_ref, kbias = None, None
+            st = L.srtMatmulBiasActivation(a_ptr, ctypes.byref(ad), int(transpose_lhs), b_ptr, ctypes.byref(bd),
+                                           int(transpose_rhs), bias_ptr, biasd_ref, int(act), float(coef),
+                                           o_ptr, ctypes.byref(od), self.stream)
+            del kbias
+        del ka, kb, ko
+        check(st, "srtMatmul")
+
+    def __del__(self):
+        try:
+            if self.stream:
+                native.lib().srtStreamDestroy(self.stream)
+                self.stream = None
+        except Exception:
+            pass
+
+
+class HipDevice:
+    """Role of CudaDevice (CudaDevice.swift:22-94).  Index 0 is reserved for the CPU in the
+    reference's numbering; GPU i is device i + 1."""
+
+    def __init__(self, index, queue_count):
+        self.index = index
+        self.gpu_id = index - 1
+        props = native.DeviceProperties()
+        check(native.lib().srtGetDeviceProperties(ctypes.byref(props), self.gpu_id), "srtGetDeviceProperties")
+        self.properties = props
+        self.name = f"gpu:{self.gpu_id}"
+        self.memory_type = "discrete"
+        self.queues = [HipQueue(index, self.gpu_id, f"{self.name}_q{i}") for i in range(queue_count)]
+
+    def describe(self):
+        p = self.properties
+        return (f"[type: {p.name.decode()}, arch: {p.archName.decode()}, multiprocessors: {p.multiProcessorCount}, "
+                f"memory: {p.totalGlobalMem >> 30} GB, clock: {p.clockRateKHz / 1e6:.2f} GHz]")
+
+
+class HipPlatform:
+    """Role of CudaPlatform (CudaPlatform.swift:22-115): enumerates devices, owns the queue stack."""
+
+    accelerator_queue_count = 2   # CudaPlatform.acceleratorQueueCount, CudaPlatform.swift:39
+    _local = None
+    _lock = threading.Lock()
+
+    def __init__(self):
+        n = ctypes.c_int32()
+        check(native.lib().srtGetDeviceCount(ctypes.byref(n)), "srtGetDeviceCount")
+        if n.value < 1:
+            raise native.SrtError(native.ERROR_NO_DEVICE, "HipPlatform: no GPU visible")
+        self.devices = [None] + [HipDevice(i + 1, self.accelerator_queue_count) for i in range(n.value)]
+        self.queue_stack = [self.devices[1].queues[0]]   # default queue, CudaPlatform.swift:103-104
+
+    @classmethod
+    def local(cls):
+        with cls._lock:
+            if cls._local is None:
+                cls._local = HipPlatform()
+            return cls._local
+
+    @property
+    def current_queue(self):
+        return self.queue_stack[-1]
+
+
+def current_queue():
+    """`currentQueue` (platform/common/Platform.swift:78-80)."""
+    return HipPlatform.local().current_queue
+
+
+class using:
+    """`using(queue:)` scope: pushes a queue on the stack for the duration of a with-block."""
+
+    def __init__(self, queue):
+        self.queue = queue
+
+    def __enter__(self):
+        HipPlatform.local().queue_stack.append(self.queue)
+        return self.queue
+
+    def __exit__(self, *exc):
+        HipPlatform.local().queue_stack.pop()
+        return False

@@ -1,0 +1,147 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares,
+descriptor marshalling, host-side shape logic.  No compute calls (no GPU here)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import swiftrt_amd as srt
+from swiftrt_amd import native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "srt_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(srt[A-Z]\w*)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 28
+    L = ctypes.CDLL(native.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in srt_hip.h but not exported"
+    # and the binding table covers the header exactly
+    assert sorted(native.SIGNATURES) == names
+
+
+def test_status_strings_and_version():
+    L = native.lib()
+    assert L.srtGetVersion() >= 100
+    assert L.srtGetStatusString(0) == b"srtSuccess"
+    assert L.srtGetStatusString(801) == b"srtErrorNotSupported"
+    assert L.srtGetStatusString(12345) == b"srtErrorUnknown"
+
+
+def test_status_mapping_to_exceptions():
+    native.check(0)
+    with pytest.raises(srt.NotSupportedError):
+        native.check(native.ERROR_NOT_SUPPORTED, "x")
+    with pytest.raises(srt.SrtError) as e:
+        native.check(native.ERROR_INVALID_VALUE, "x")
+    assert not isinstance(e.value, srt.NotSupportedError)
+
+
+def test_descriptor_marshalling():
+    d, keep = native.make_descriptor(native.REAL16BF, (4, 6), (12, 2), native.ORDER_ROW)
+    assert d.rank == 2 and d.count == 24 and d.spanCount == 3 * 12 + 5 * 2 + 1
+    assert [d.shape[i] for i in range(2)] == [4, 6] and [d.strides[i] for i in range(2)] == [12, 2]
+    assert [d.logicalStrides[i] for i in range(2)] == [6, 1]
+    assert ctypes.sizeof(native.TensorDescriptor) == 56   # 3 x int32 + pad, 2 x size_t, 3 pointers
+
+
+def test_descriptor_validation_without_gpu():
+    # argument checks run before any device work, so they are observable on a CPU-only host
+    L = native.lib()
+    ad, k1 = native.make_descriptor(native.REAL32F, (3, 2), (2, 1), native.ORDER_ROW)
+    bd, k2 = native.make_descriptor(native.REAL32F, (3, 4), (4, 1), native.ORDER_ROW)   # inner dims differ
+    od, k3 = native.make_descriptor(native.REAL32F, (3, 4), (4, 1), native.ORDER_ROW)
+    dummy = ctypes.c_void_p(256)
+    assert L.srtMatmul(dummy, ctypes.byref(ad), 0, dummy, ctypes.byref(bd), 0, dummy, ctypes.byref(od), None) \
+        == native.ERROR_INVALID_VALUE
+    # double precision is not part of the path -> caller falls back
+    a64, k4 = native.make_descriptor(native.REAL64F, (3, 2), (2, 1), native.ORDER_ROW)
+    b64, k5 = native.make_descriptor(native.REAL64F, (2, 4), (4, 1), native.ORDER_ROW)
+    o64, k6 = native.make_descriptor(native.REAL64F, (3, 4), (4, 1), native.ORDER_ROW)
+    assert L.srtMatmul(dummy, ctypes.byref(a64), 0, dummy, ctypes.byref(b64), 0, dummy, ctypes.byref(o64), None) \
+        == native.ERROR_NOT_SUPPORTED
+    # tiled order -> not supported
+    at, k7 = native.make_descriptor(native.REAL32F, (3, 2), (2, 1), 2)
+    b2, k8 = native.make_descriptor(native.REAL32F, (2, 4), (4, 1), native.ORDER_ROW)
+    assert L.srtMatmul(dummy, ctypes.byref(at), 0, dummy, ctypes.byref(b2), 0, dummy, ctypes.byref(od), None) \
+        == native.ERROR_NOT_SUPPORTED
+    # empty result: success, nothing launched
+    ae, k9 = native.make_descriptor(native.REAL32F, (0, 2), (2, 1), native.ORDER_ROW)
+    oe, k10 = native.make_descriptor(native.REAL32F, (0, 4), (4, 1), native.ORDER_ROW)
+    assert L.srtMatmul(None, ctypes.byref(ae), 0, dummy, ctypes.byref(b2), 0, None, ctypes.byref(oe), None) == 0
+    # null descriptor
+    assert L.srtMatmul(dummy, None, 0, dummy, ctypes.byref(b2), 0, dummy, ctypes.byref(od), None) \
+        == native.ERROR_INVALID_VALUE
+
+
+def test_kernel_selection_is_queryable_without_gpu():
+    L = native.lib()
+
+    def query(dt, M, N, K, ta=False, tb=False, align=256):
+        ashape = (K, M) if ta else (M, K)
+        bshape = (N, K) if tb else (K, N)
+        ad, k1 = native.make_descriptor(dt, ashape, (ashape[1], 1), native.ORDER_ROW)
+        bd, k2 = native.make_descriptor(dt, bshape, (bshape[1], 1), native.ORDER_ROW)
+        od, k3 = native.make_descriptor(dt, (M, N), (N, 1), native.ORDER_ROW)
+        buf = ctypes.create_string_buffer(64)
+        p = ctypes.c_void_p(align)
+        st = L.srtMatmulQueryKernel(ctypes.byref(ad), int(ta), ctypes.byref(bd), int(tb), ctypes.byref(od),
+                                    p, p, p, buf, 64)
+        assert st == 0
+        return buf.value.decode()
+
+    assert query(native.REAL16BF, 8192, 8192, 8192) == "mfma_256x256"
+    assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256"
+    assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256"
+    assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
+    assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"
+    assert query(native.REAL16BF, 33, 33, 33) == "generic"
+    assert query(native.REAL16BF, 64, 64, 64, align=2) == "generic"      # misaligned view
+    assert query(native.REAL32F, 512, 512, 512) in ("generic", "f32_mfma")
+
+
+def test_tensor_layout_and_views():
+    t = srt.Tensor(np.arange(12, dtype=np.float32).reshape(3, 4))
+    assert t.shape == (3, 4) and t.strides == (4, 1)
+    assert t.t.shape == (4, 3) and t.t.strides == (1, 4)          # .t swaps extents and strides, zero copy
+    assert np.array_equal(t.t.array(), np.arange(12, dtype=np.float32).reshape(3, 4).T)
+    v = t[1:3, 1:4:2]
+    assert v.shape == (2, 2) and v.strides == (4, 2) and v.offset == 5
+    assert np.array_equal(v.array(), [[5, 7], [9, 11]])
+    c = srt.Tensor(np.arange(6, dtype=np.float32).reshape(3, 2), order=srt.Order.col)
+    assert c.strides == (1, 3)
+    assert np.array_equal(c.array(), np.arange(6, dtype=np.float32).reshape(3, 2))
+    t3 = srt.Tensor(np.zeros((2, 3, 4), np.float16))
+    assert t3.t.shape == (2, 4, 3) and t3.t.strides == (12, 1, 4)  # only the last two dims swap
+
+
+def test_matmul_shape_rules_raise_before_any_native_call():
+    a = srt.Tensor(np.zeros((3, 2), np.float32))
+    b = srt.Tensor(np.zeros((3, 4), np.float32))
+    with pytest.raises(ValueError):
+        srt.matmul(a, b)
+    with pytest.raises(ValueError):
+        srt.Dense(srt.Tensor(np.zeros((2, 4), np.float32)), bias=srt.Tensor(np.zeros(3, np.float32)))
+
+
+def test_activation_enum_matches_reference_case_order():
+    assert [a.name for a in srt.ActivationType] == ["sigmoid", "relu", "tanh", "clippedRelu", "elu", "identity"]
+    assert [int(a) for a in srt.ActivationType] == list(range(6))
+
+
+def test_bf16_fast_encoder_matches_oracle_codec():
+    from oracle import srt_oracle as ora
+    from tests import helpers
+    r = np.random.default_rng(0)
+    x = np.concatenate([r.standard_normal(100000).astype(np.float32),
+                        np.array([0, -0.0, np.inf, -np.inf, np.nan, 1 + 2 ** -8, 1 + 3 * 2 ** -8, 3.4e38], np.float32)])
+    assert np.array_equal(helpers.bf16_encode_fast(x), ora.encode(x, ora.BF16))

@@ -1,0 +1,96 @@
+"""GPU tests of the device / stream / event / memory entry points of the C ABI."""
+import ctypes
+import time
+
+import numpy as np
+import pytest
+
+import swiftrt_amd as srt
+from swiftrt_amd import native
+
+pytestmark = pytest.mark.gpu
+
+
+def test_platform_enumerates_gfx950():
+    p = srt.HipPlatform.local()
+    assert len(p.devices) >= 2 and p.devices[0] is None          # device 0 is the CPU slot
+    d = p.devices[1]
+    assert b"gfx950" in d.properties.archName
+    assert d.properties.warpSize == 64 and d.properties.multiProcessorCount >= 200
+    assert len(d.queues) == srt.HipPlatform.accelerator_queue_count
+    assert srt.current_queue() is d.queues[0]
+
+
+def test_memcpy_round_trip_and_memset():
+    q = srt.current_queue()
+    src = np.arange(100003, dtype=np.uint8)
+    mem = q.allocate(src.nbytes)
+    q.copy_to_device(src.ctypes.data, mem, src.nbytes)
+    dst = np.zeros_like(src)
+    q.copy_to_host(mem, dst.ctypes.data, src.nbytes)
+    q.wait_for_completion()
+    assert np.array_equal(src, dst)
+    L = native.lib()
+    native.check(L.srtMemsetAsync(ctypes.c_void_p(mem.pointer), 0xAB, 1000, q.stream))
+    native.check(L.srtMemsetAsync(ctypes.c_void_p(mem.pointer + 1001), 0x11, 7, q.stream))
+    q.copy_to_host(mem, dst.ctypes.data, src.nbytes)
+    q.wait_for_completion()
+    assert np.all(dst[:1000] == 0xAB) and dst[1000] == src[1000] and np.all(dst[1001:1008] == 0x11)
+    assert np.array_equal(dst[1008:], src[1008:])
+
+
+def test_caching_allocator_reuses_blocks_per_stream():
+    q = srt.current_queue()
+    m = q.allocate(5000)
+    p0 = m.pointer
+    del m
+    m2 = q.allocate(6000)          # same 8 KiB bin, same stream: handed back at once
+    assert m2.pointer == p0
+    m3 = q.allocate(6000)
+    assert m3.pointer != p0
+    assert m2.pointer % 256 == 0 and m3.pointer % 256 == 0
+    native.check(native.lib().srtDeviceFree(None))
+    assert native.lib().srtDeviceFree(ctypes.c_void_p(12345)) == native.ERROR_INVALID_VALUE
+    del m2, m3
+    native.check(native.lib().srtDeviceEmptyCache())
+
+
+def test_events_delay_and_cross_queue_wait():
+    p = srt.HipPlatform.local()
+    q0, q1 = p.devices[1].queues[0], p.devices[1].queues[1]
+    start = q0.record_event(timing=True)
+    q0.delay(0.05)
+    done = q0.record_event(timing=True)
+    assert not done.occurred                      # srtEventQuery -> not ready while the delay spins
+    q1.wait(done)                                 # q1 now ordered after q0's delay
+    t0 = time.time()
+    q1.wait_for_completion()
+    assert done.occurred
+    assert done.elapsed_ms_since(start) >= 45.0
+    assert time.time() - t0 < 5.0
+
+
+def test_storage_migration_flags():
+    # DiscreteStorage's lazy replica movement: first device read copies host->device, a second does not;
+    # reading on the host after a device write copies back once
+    a = srt.Tensor(np.ones((4, 4), np.float32))
+    q = srt.current_queue()
+    a.device_read(q)
+    assert a.storage.last_copy == "h2d"
+    a.device_read(q)
+    assert a.storage.last_copy is None
+    c = srt.matmul(a, a)
+    assert np.array_equal(c.array(), np.full((4, 4), 4, np.float32)) and c.storage.last_copy == "d2h"
+    c.array()
+    assert c.storage.last_copy is None
+
+
+def test_using_queue_scope_and_two_queues():
+    p = srt.HipPlatform.local()
+    q1 = p.devices[1].queues[1]
+    a = srt.Tensor(np.full((8, 8), 2, np.float32))
+    with srt.using(q1):
+        assert srt.current_queue() is q1
+        b = srt.matmul(a, a)
+    c = srt.matmul(b, a)           # consumed on queue 0: ordered after queue 1 through an event
+    assert np.array_equal(c.array(), np.full((8, 8), 2 * 2 * 8 * 2 * 8, np.float32))
