@@ -22,6 +22,7 @@
 //       8(k) x 8(mn) block as eight 16-byte rows (coalesced along mn), transposes it in
 //       registers with 32 v_perm_b32 and writes eight k-contiguous chunks.
 #include "gemm_common.h"
+#include "gemm_mfma_dtl.h"
 
 namespace srt {
 
@@ -284,10 +285,21 @@ hipError_t launch_layout(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t
   return launch_one<T, BM, BN, false, false>(p, stream);
 }
 
+// 256 x 256 tiles: the direct-to-LDS kernel whenever 32-bit buffer offsets reach every operand
+template <typename T>
+hipError_t launch_dtl(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return dtl::launch<T, true, true>(p, stream);
+  if (a_kc && !b_kc) return dtl::launch<T, true, false>(p, stream);
+  if (!a_kc && b_kc) return dtl::launch<T, false, true>(p, stream);
+  return dtl::launch<T, false, false>(p, stream);
+}
+
 template <typename T>
 hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hipStream_t stream) {
   switch (tile) {
-    case 1: return launch_layout<T, 256, 256>(p, a_kc, b_kc, stream);
+    case 1:
+      if (dtl::dtl_fits(p, a_kc, b_kc)) return launch_dtl<T>(p, a_kc, b_kc, stream);
+      return launch_layout<T, 256, 256>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     default: return launch_layout<T, 64, 64>(p, a_kc, b_kc, stream);
   }

@@ -41,6 +41,7 @@ def test_memcpy_round_trip_and_memset():
 
 def test_caching_allocator_reuses_blocks_per_stream():
     q = srt.current_queue()
+    native.check(native.lib().srtDeviceEmptyCache())     # start from an empty cache
     m = q.allocate(5000)
     p0 = m.pointer
     del m
