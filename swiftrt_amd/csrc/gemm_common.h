@@ -39,6 +39,18 @@ struct BF16 {
     if ((x & 0x7fffffffu) > 0x7f800000u) return 0x7fff;
     return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
   }
+  // Two values -> one dword (a in the low half).  EXACT = false uses the hardware converter
+  // (round to nearest even, one instruction) and is only valid when neither input is a NaN;
+  // EXACT = true is the scalar encoder (NaN -> 0x7FFF).  Callers test a whole tile for NaNs once
+  // and pick the variant.
+  template <bool EXACT>
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    if (EXACT) return (uint32_t)from_float(a) | ((uint32_t)from_float(b) << 16);
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  }
 };
 
 struct F16 {
@@ -54,6 +66,10 @@ struct F16 {
     uint16_t h;
     __builtin_memcpy(&h, &v, 2);
     return h;
+  }
+  template <bool EXACT>
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    return (uint32_t)from_float(a) | ((uint32_t)from_float(b) << 16);
   }
 };
 
@@ -79,6 +95,22 @@ __device__ __forceinline__ float apply_activation(int activation, float coef, fl
     case srtActivationElu: return x > 0.0f ? x : coef * (expf(x) - 1.0f);
     default: return x;
   }
+}
+
+// Same with the activation fixed at compile time: kernels switch on the activation once per
+// workgroup and run an epilogue specialised for it, so the unrolled store code of the common
+// cases (identity, relu) carries no transcendental code and no per-element branches.
+template <int ACT>
+__device__ __forceinline__ float activation_ct(float coef, float x) {
+  if (ACT == srtActivationSigmoid) return 1.0f / (1.0f + expf(-x));
+  if (ACT == srtActivationRelu) return x > 0.0f ? x : 0.0f;
+  if (ACT == srtActivationTanh) return tanhf(x);
+  if (ACT == srtActivationClippedRelu) {
+    float y = x > 0.0f ? x : 0.0f;
+    return y < coef ? y : coef;
+  }
+  if (ACT == srtActivationElu) return x > 0.0f ? x : coef * (expf(x) - 1.0f);
+  return x;
 }
 
 // Epilogue state for one output column (or row) set; bias is read as element type T.

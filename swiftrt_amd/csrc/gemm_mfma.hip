@@ -22,9 +22,19 @@
 //       8(k) x 8(mn) block as eight 16-byte rows (coalesced along mn), transposes it in
 //       registers with 32 v_perm_b32 and writes eight k-contiguous chunks.
 #include "gemm_common.h"
-#include "gemm_mfma_dtl.h"
 
 namespace srt {
+
+// 256 x 256 ring kernels, one translation unit per (type, layout): gemm_ring_inst.hip
+bool ring_fits_problem(const GemmProblem& p, bool a_kc, bool b_kc);
+#define SRT_RING_DECL(T) \
+  hipError_t launch_ring_##T##_00(const GemmProblem&, hipStream_t); \
+  hipError_t launch_ring_##T##_01(const GemmProblem&, hipStream_t); \
+  hipError_t launch_ring_##T##_10(const GemmProblem&, hipStream_t); \
+  hipError_t launch_ring_##T##_11(const GemmProblem&, hipStream_t);
+SRT_RING_DECL(BF16)
+SRT_RING_DECL(F16)
+#undef SRT_RING_DECL
 
 namespace {
 
@@ -285,21 +295,28 @@ hipError_t launch_layout(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t
   return launch_one<T, BM, BN, false, false>(p, stream);
 }
 
-// 256 x 256 tiles: the direct-to-LDS kernel whenever 32-bit buffer offsets reach every operand
 template <typename T>
-hipError_t launch_dtl(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
-  if (a_kc && b_kc) return dtl::launch<T, true, true>(p, stream);
-  if (a_kc && !b_kc) return dtl::launch<T, true, false>(p, stream);
-  if (!a_kc && b_kc) return dtl::launch<T, false, true>(p, stream);
-  return dtl::launch<T, false, false>(p, stream);
+hipError_t launch_ring(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream);
+template <>
+hipError_t launch_ring<BF16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_ring_BF16_11(p, stream);
+  if (a_kc) return launch_ring_BF16_10(p, stream);
+  if (b_kc) return launch_ring_BF16_01(p, stream);
+  return launch_ring_BF16_00(p, stream);
+}
+template <>
+hipError_t launch_ring<F16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_ring_F16_11(p, stream);
+  if (a_kc) return launch_ring_F16_10(p, stream);
+  if (b_kc) return launch_ring_F16_01(p, stream);
+  return launch_ring_F16_00(p, stream);
 }
 
+// tile 1 (256 x 256) is the ring kernel; tiles 2 and 3 are the register-staged kernels above
 template <typename T>
 hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hipStream_t stream) {
   switch (tile) {
-    case 1:
-      if (dtl::dtl_fits(p, a_kc, b_kc)) return launch_dtl<T>(p, a_kc, b_kc, stream);
-      return launch_layout<T, 256, 256>(p, a_kc, b_kc, stream);
+    case 1: return launch_ring<T>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     default: return launch_layout<T, 64, 64>(p, a_kc, b_kc, stream);
   }
@@ -332,7 +349,7 @@ int mfma_select(const GemmProblem& p) {
 
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
   int tile;
-  if (tiles(256) >= 192) tile = 1;
+  if (tiles(256) >= 192 && ring_fits_problem(p, a_kc, b_kc)) tile = 1;
   else if (tiles(128) >= 192) tile = 2;
   else if (p.M > 64 && p.N > 64 && tiles(128) * 4 >= tiles(64)) tile = tiles(128) >= 64 ? 2 : 3;
   else tile = 3;

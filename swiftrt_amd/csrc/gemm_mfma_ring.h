@@ -1,0 +1,601 @@
+// 256 x 256 bf16 / fp16 matmul tile kernel for gfx950: direct-to-LDS operand staging through a
+// ring of NS k-stages of depth 32, v_mfma_f32_32x32x16 with fp32 accumulators in registers,
+// fused bias + activation epilogue staged through LDS into 16-byte row stores.
+//
+// Why a ring of shallow stages: a global load takes on the order of a microsecond to land, i.e.
+// longer than the 64 MFMAs of a 64-deep k tile take to issue.  What bounds the prefetch distance
+// is LDS capacity, so the 160 KiB are cut into NS = 5 stages of 32 KiB (k depth 32): a stage is
+// requested (NS - 1) iterations -- about 4 x 1024 MFMA cycles -- before it is consumed.
+//
+// Global memory -> LDS goes through `buffer_load_dwordx4 ... lds`: no staging registers, no LDS
+// write instructions, out-of-range addresses return zero (the buffer descriptor bounds every
+// operand), and the XOR swizzles are applied on the *global* side -- lane l of a load always
+// lands at LDS byte M0 + 16 l, so each lane fetches the 16-byte chunk that belongs at its
+// landing position.
+//
+// LDS layouts per operand (one stage = A region 16 KiB + B region 16 KiB):
+//   stored k-contiguous  (A not transposed / B transposed):
+//       [256 rows][4 chunks of 16 B]; chunk c of row r sits at position c ^ ((r >> 2) & 3).
+//       MFMA operand = one ds_read_b128 (lane l: row l % 32, chunk 2 kk + l / 32).
+//   stored mn-contiguous (A transposed / B not transposed):
+//       [32 k][32 chunks of 16 B] (a k-row is 256 m or n = 512 B); chunk c of k-row k sits at
+//       position c ^ ((k & 3) << 2).  MFMA operand = two ds_read_b64_tr_b16: within each group
+//       of 16 lanes the instruction transposes a 4(k) x 16(mn) block, so every lane ends up with
+//       4 consecutive k of its own m / n without any VALU work.
+//   Both layouts hand lane l the k values kk*16 + 8*(l/32) + 0..7, so any pairing is valid, and
+//   both are free of LDS bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
+//
+// Pipeline, per stage s (two phases of 16 MFMAs per wave):
+//   phase 0   MFMAs of k slice 0 (registers); the LDS reads of slice 1 ride on the first eight
+//             MFMAs, the four B loads of stage s-1+NS on the last eight
+//   sync      s_waitcnt vmcnt(8 (NS-2)) lgkmcnt(0); s_barrier -- stage s+1 has landed for every
+//             wave, and every wave holds all of stage s in registers, so slot s % NS is free
+//   phase 1   MFMAs of slice 1, interleaved with the four A loads of stage s+NS (into the slot
+//             just freed) and the LDS reads of slice 0 of stage s+1
+// The interleave is fixed in the source with scheduling fences so that every memory instruction
+// issues in the shadow of an MFMA.
+//
+// The MFMA is issued with the B fragment as its first operand, so each 32 x 32 accumulator tile
+// is C^T: a lane owns one row m and, per group of four registers, four consecutive columns n --
+// the epilogue rounds them, packs 8 bytes per group into an LDS staging area and writes C from
+// there in whole 256-byte row segments.
+#pragma once
+#include "gemm_common.h"
+
+namespace srt {
+namespace ring {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+#define SRT_LDS __attribute__((address_space(3)))
+
+constexpr int BM = 256, BN = 256, BK = 32;
+constexpr int NT = 256;                    // 4 waves, 2 x 2, each 128 x 128
+constexpr int REGION = 256 * BK * 2;       // bytes of one operand stage (16 KiB)
+constexpr int STAGE = 2 * REGION;          // 32 KiB
+constexpr uint32_t OOB = 0x80000000u;      // byte offset beyond any supported operand: reads 0, stores dropped
+
+template <typename T>
+__device__ __forceinline__ f32x16_t mfma(u32x4_t a, u32x4_t b, f32x16_t c);
+template <>
+__device__ __forceinline__ f32x16_t mfma<BF16>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                 c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x16_t mfma<F16>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b),
+                                                c, 0, 0, 0);
+}
+
+// Raw buffer descriptor: base, stride 0, num_records in bytes, 32-bit untyped data format.
+__device__ __forceinline__ u32x4_t make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t p = reinterpret_cast<uint64_t>(base);
+  u32x4_t r = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, bytes, 0x00020000u};
+  return r;
+}
+
+// One 16-byte-per-lane load straight into LDS: lane l's data lands at lds_addr + 16 l.
+// Written as inline assembly so that no automatic wait on the vector-memory counter is placed
+// in front of unrelated LDS reads; completion is awaited explicitly before the barrier.
+__device__ __forceinline__ void load_to_lds(u32x4_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
+// The same load in two halves, for the main loop: the LDS landing address goes into M0 first,
+// an MFMA is issued in between (it also provides the wait state M0 needs before the load reads
+// it), then the load itself.  Nothing else may touch M0 between the two.
+template <int IMM>
+__device__ __forceinline__ void set_lds_target(uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_base), "n"(IMM) : "scc");
+}
+__device__ __forceinline__ void load_to_lds_at_m0(u32x4_t rsrc, uint32_t voff, uint32_t soff) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+
+// ---- global -> LDS ---------------------------------------------------------------------------
+// Per-lane byte offsets (into the operand's buffer) of the 4 loads a wave issues per stage for
+// one operand; the k advance goes through the scalar offset.
+template <bool KC>
+struct Loader {
+  uint32_t voff[4];
+  uint32_t kstep;   // bytes per k stage
+
+  // tile_row0: first m (or n) of the tile.  ld: elements between rows (KC) or between k (MN).
+  __device__ __forceinline__ void init(int wave, int lane, int tile_row0, long long ld) {
+    if (KC) {
+      // load i of this wave covers tile rows (wave*4 + i)*16 .. +15, 4 lanes per 64-byte row
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = (wave * 4 + i) * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+        voff[i] = (uint32_t)(((long long)(tile_row0 + row) * ld + chunk * 8) * 2);
+      }
+      kstep = BK * 2;
+    } else {
+      // load i covers k rows (wave*4 + i)*2 .. +1, 32 lanes per 512-byte k row
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int krow = (wave * 4 + i) * 2 + (lane >> 5);
+        const int chunk = (lane & 31) ^ ((krow & 3) << 2);
+        voff[i] = (uint32_t)(((long long)krow * ld + tile_row0 + chunk * 8) * 2);
+      }
+      kstep = (uint32_t)(BK * ld * 2);
+    }
+  }
+
+  // Load i of this wave for the k stage at scalar byte offset `soff` (stage * kstep, or OOB to
+  // make the whole load read zeros without touching memory), into the operand region at LDS
+  // address `region`.  `tail`: this is a ragged last stage; for a k-contiguous operand the
+  // logical chunks >= mask_from lie at or beyond K and must read as zero (an mn-contiguous
+  // operand gets that from the bounds check, its k rows >= K being past the end of the view).
+  __device__ __forceinline__ void issue_one(u32x4_t rsrc, uint32_t region, int wave, int lane, uint32_t soff, int i,
+                                            bool tail, int mask_from) const {
+    uint32_t v = voff[i];
+    if (KC) {
+      // (row >> 2) & 3 of the row this lane fetches does not depend on i or the wave
+      const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+      v = (tail && chunk >= mask_from) ? OOB : v;
+    }
+    load_to_lds(rsrc, region + (uint32_t)(wave * 4 + i) * 1024u, v, soff);
+  }
+
+  // Permanently aim the chunks at or beyond K out of range (called once, just before the loads
+  // of a ragged last stage are issued; every later load is out of range as a whole anyway).
+  __device__ __forceinline__ void mask_tail(int lane, int mask_from) {
+    if (KC) {
+      const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+      if (chunk >= mask_from) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) voff[i] = OOB;
+      }
+    }
+  }
+};
+
+// ---- LDS -> MFMA operands ----------------------------------------------------------------------
+template <bool KC>
+struct FragReader {
+  uint32_t base[4];   // KC: [0..1] one address per k slice; MN: one address per 32-wide tile index
+
+  // wave_row0: first m (n) of the wave's 128-wide slice inside the tile
+  __device__ __forceinline__ void init(int lane, int wave_row0) {
+    if (KC) {
+      const int r = lane & 31, h = lane >> 5;
+      const int f = (r >> 2) & 3;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) base[kk] = (uint32_t)((wave_row0 + r) * 64 + (((2 * kk + h) ^ f) << 4));
+      base[2] = base[3] = 0;
+    } else {
+      const int g = lane >> 4, jn = lane & 15, e = jn >> 2, q = jn & 3;
+      // lane supplies the address of T[k = 8*(g>>1) + e (+ 16 kk + 4 r)][mn = wave_row0 + 32 t + 16*(g&1) + 4 q]
+      const int krow = 8 * (g >> 1) + e;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int mn = wave_row0 + 32 * t + 16 * (g & 1) + 4 * q;
+        const int chunk = (mn >> 3) ^ (e << 2);
+        base[t] = (uint32_t)(krow * 512 + chunk * 16 + ((mn >> 2) & 1) * 8);
+      }
+    }
+  }
+
+  // operand for 32-wide tile t (0..3) and k slice kk (0..1) of the region at LDS address `region`
+  __device__ __forceinline__ u32x4_t read(uint32_t region, int t, int kk) const {
+    if (KC) {
+      return *reinterpret_cast<const SRT_LDS u32x4_t*>(region + base[kk] + t * 2048);
+    } else {
+      const uint32_t a = region + base[t] + kk * 8192;
+      const u32x2_t lo =
+          __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a)));
+      const u32x2_t hi = __builtin_bit_cast(
+          u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a + 2048)));
+      u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+      return v;
+    }
+  }
+};
+
+// XCD-aware remap of the linear workgroup id followed by a grouped tile order.
+// Workgroups are handed to the 8 XCDs round-robin, so ids congruent mod 8 share an L2.  The
+// remap gives each XCD a contiguous range of logical ids; the grouped order walks GROUP_M tile
+// rows at a time so a contiguous range is a compact patch of the tile grid.
+__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int* tm, int* tn) {
+  const int nwg = tiles_m * tiles_n;
+  constexpr int XCDS = 8;
+  int logical = wg;
+  if (nwg >= XCDS * 4) {
+    const int per = (nwg + XCDS - 1) / XCDS;
+    int tall = nwg % XCDS;
+    if (tall == 0) tall = XCDS;
+    const int xcd = wg % XCDS, local = wg / XCDS;
+    logical = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+  }
+  constexpr int GROUP_M = 8;
+  const int per_group = GROUP_M * tiles_n;
+  const int group = logical / per_group;
+  const int first_m = group * GROUP_M;
+  const int gsize = min(tiles_m - first_m, GROUP_M);
+  const int in_group = logical - group * per_group;
+  *tm = first_m + in_group % gsize;
+  *tn = in_group / gsize;
+}
+
+#define SRT_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Epilogue of one wave.
+// acc[i][j] is a transposed 32 x 32 tile: lane l owns row m = wave_m0 + 32 i + l % 32 and, in
+// registers 4 g .. 4 g + 3, the columns n = wave_n0 + 32 j + 8 g + 4 (l / 32) + 0..3.
+//
+// Step 1 for identity / relu / clippedRelu (apply_linear_epilogue): bias, then the activation
+// as two branch-free selects driven by uniform parameters, in place and in straight-line code
+// (the accumulators never cross a branch).  Returns whether any lane of the wave holds a NaN,
+// so the rounding step can use the one-instruction hardware converter when there is none.
+template <typename T>
+__device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x16_t (&acc)[4][4], int wave_m0,
+                                                      int wave_n0, int lane) {
+  using S = typename T::storage;
+  const S* bias = (const S*)p.bias;
+  const bool per_row = p.bias_per_row != 0;
+  const bool clamp_low = p.activation == srtActivationRelu || p.activation == srtActivationClippedRelu;
+  const float ceiling = p.activation == srtActivationClippedRelu ? p.coef : __builtin_inff();
+  const int r = lane & 31, h = lane >> 5;
+  float brow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = wave_m0 + 32 * i + r;
+    brow[i] = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+  }
+  bool nan = false;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float bcol[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
+        bcol[e] = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float x = acc[i][j][4 * g + e] + (per_row ? brow[i] : bcol[e]);
+          x = (clamp_low && !(x > 0.0f)) ? 0.0f : x;   // relu: x > 0 ? x : 0 (a NaN becomes 0, as max(x, 0) gives)
+          x = x > ceiling ? ceiling : x;               // identity: ceiling = +inf keeps x, NaN included
+          acc[i][j][4 * g + e] = x;
+        }
+        nan |= __builtin_isunordered(acc[i][j][4 * g], acc[i][j][4 * g + 1]);
+        nan |= __builtin_isunordered(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+      }
+    }
+  return __builtin_amdgcn_ballot_w64(nan) != 0;
+}
+
+// Step 2 (store_tile): one rounding to the element type, then a trip through LDS so that global
+// stores are whole 16-byte chunks of C rows (a store instruction writes four 256-byte row
+// segments instead of 64 scattered pieces).  The wave's 128 x 128 result goes in two halves of
+// 64 rows through its private 16 KiB staging area at LDS address `stage`: [64 rows][16 chunks of
+// 16 B], chunk c of row r at position c ^ (r & 15) (reads of a row are conflict-free, writes of
+// a column 2-way).  Global stores go through a bounds-checked buffer; chunks outside M x N aim
+// out of range.
+template <typename T, bool EXACT>
+__device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t (&acc)[4][4], int wave_m0, int wave_n0,
+                                           int bz, int lane, uint32_t stage) {
+  using S = typename T::storage;
+  S* C = (S*)p.C + (long long)bz * p.scb;
+  const long long c_last = (long long)(p.M - 1) * p.scm + p.N;   // elements spanned by C (< 2^30, checked on the host)
+  const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
+  const int ldc2 = (int)(p.scm * 2);
+  const int r = lane & 31, h = lane >> 5;
+  // read side: lane covers chunk (lane & 15) of rows (lane >> 4) + 4 it
+  const int rd_chunk = lane & 15, rd_row = lane >> 4;
+  const int n_rd = wave_n0 + 8 * rd_chunk;
+  const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8 (checked on the host): the chunk is whole
+
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    // ---- registers -> staging ----
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const int i = 2 * half + ii;
+      const int row = 32 * ii + r;
+      const uint32_t row_addr = stage + (uint32_t)row * 256u + (uint32_t)h * 8u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x2_t w = {T::template pack2<EXACT>(acc[i][j][4 * g], acc[i][j][4 * g + 1]),
+                             T::template pack2<EXACT>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
+          const int c = 4 * j + g;
+          *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
+        }
+      }
+    }
+    // ---- staging -> global: 16 instructions of 4 rows x 256 bytes ----
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const int row = rd_row + 4 * it;
+      const u32x4_t v =
+          *reinterpret_cast<const SRT_LDS u32x4_t*>(stage + (uint32_t)row * 256u + (uint32_t)((rd_chunk ^ (row & 15)) << 4));
+      const int m = wave_m0 + 64 * half + row;
+      const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc2 + n_rd * 2) : OOB;
+      __builtin_amdgcn_raw_buffer_store_b128(v, rc, (int)off, 0, 0);
+    }
+  }
+}
+
+// Epilogue for sigmoid / tanh / elu: acc + bias goes to the staging area as fp32, and the
+// activation, the rounding and the store run in a rolled loop over the staged rows, so the
+// transcendental code exists once instead of once per accumulator register.
+// Four passes of 32 rows: staging is [32 rows][32 chunks of 16 B], chunk c of row r at c ^ r.
+template <typename T>
+__device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, const f32x16_t (&acc)[4][4],
+                                                          int wave_m0, int wave_n0, int bz, int lane, uint32_t stage) {
+  using S = typename T::storage;
+  S* C = (S*)p.C + (long long)bz * p.scb;
+  const S* bias = (const S*)p.bias;
+  const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
+  const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
+  const int ldc2 = (int)(p.scm * 2);
+  const bool per_row = p.bias_per_row != 0;
+  const int r = lane & 31, h = lane >> 5;
+  const int rd_chunk = lane & 31, rd_row = lane >> 5;   // read side: 4 columns of rows rd_row + 2 it
+  const int n_rd = wave_n0 + 4 * rd_chunk;
+  const bool n_rd_ok = n_rd < p.N;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = wave_m0 + 32 * i + r;
+    const float brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4_t x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
+          const float bcol = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+          x[e] = acc[i][j][4 * g + e] + (per_row ? brow : bcol);
+        }
+        const int c = 8 * j + 2 * g + h;
+        *reinterpret_cast<SRT_LDS f32x4_t*>(stage + (uint32_t)r * 512u + (uint32_t)((c ^ r) << 4)) = x;
+      }
+#pragma unroll 1
+    for (int it = 0; it < 16; ++it) {
+      const int row = rd_row + 2 * it;
+      const f32x4_t x =
+          *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u + (uint32_t)((rd_chunk ^ row) << 4));
+      uint32_t lo = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[0])) |
+                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[1])) << 16);
+      uint32_t hi = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[2])) |
+                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[3])) << 16);
+      const u32x2_t w = {lo, hi};
+      const int mm = wave_m0 + 32 * i + row;
+      const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
+      __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, 0);
+    }
+  }
+}
+
+template <typename T, bool A_KC, bool B_KC, bool TRANS_ACT, int NS>
+__global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
+  static_assert(NS >= 3 && NS <= 5, "ring depth");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
+  const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  int tm, tn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, &tm, &tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int bz = blockIdx.y;
+
+  const uint16_t* A = (const uint16_t*)p.A + (long long)bz * p.sab;
+  const uint16_t* B = (const uint16_t*)p.B + (long long)bz * p.sbb;
+  const long long lda = A_KC ? p.sam : p.sak;
+  const long long ldb = B_KC ? p.sbn : p.sbk;
+  // bytes spanned by each operand view: anything beyond reads as zero
+  const uint32_t a_bytes = (uint32_t)((A_KC ? (long long)(p.M - 1) * lda + p.K : (long long)(p.K - 1) * lda + p.M) * 2);
+  const uint32_t b_bytes = (uint32_t)((B_KC ? (long long)(p.N - 1) * ldb + p.K : (long long)(p.K - 1) * ldb + p.N) * 2);
+  const u32x4_t ra = make_rsrc(A, a_bytes);
+  const u32x4_t rb = make_rsrc(B, b_bytes);
+
+  Loader<A_KC> la;
+  Loader<B_KC> lb;
+  la.init(wave, lane, m0, lda);
+  lb.init(wave, lane, n0, ldb);
+  FragReader<A_KC> fa;
+  FragReader<B_KC> fb;
+  fa.init(lane, wm0);
+  fb.init(lane, wn0);
+
+  // acc[i][j] is the transposed 32 x 32 tile: m = 32 i + lane % 32, n = 32 j + 8 (v/4) + 4 (lane/32) + v % 4
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int KT = (p.K + BK - 1) / BK;
+  // first logical 16-byte chunk of the last k stage that lies at or beyond K (4 = stage is whole)
+  const int tail_mask = (p.K % BK) ? ((p.K % BK) + 7) / 8 : 4;
+
+  // ---- prologue: fill the ring (stages 0 .. NS-2 and the A part of stage NS-1; its B part is
+  //      the first thing the loop requests), wait for stage 0 only ----
+#pragma unroll
+  for (int t = 0; t < NS; ++t) {
+    const uint32_t slot = lds + (uint32_t)t * STAGE;
+    const bool tail = (t == KT - 1) && tail_mask < 4;
+    const uint32_t soa = t < KT ? (uint32_t)t * la.kstep : OOB;
+    const uint32_t sob = t < KT ? (uint32_t)t * lb.kstep : OOB;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) la.issue_one(ra, slot, wave, lane, soa, i, tail, tail_mask);
+    if (t < NS - 1) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lb.issue_one(rb, slot + REGION, wave, lane, sob, i, tail, tail_mask);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(8 * (NS - 2) + 4) : "memory");
+  SRT_FENCE();
+
+  u32x4_t af[2][4], bf[2][4];   // [k slice][32-wide tile]
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    af[0][t] = fa.read(lds, t, 0);
+    bf[0][t] = fb.read(lds + REGION, t, 0);
+  }
+
+  // The loop body is branch-free: loads past the last stage are aimed out of range (they return
+  // zeros without touching memory and land in a slot nobody reads again), and the reads of
+  // "stage KT" in the last trip fetch LDS contents that are never used.
+  // Loop-carried scalars: LDS slots of stage kt-1 (prv) and kt (cur), and the byte offsets of
+  // the stages being requested.  Loads of one stage are split over two phases: its A part in
+  // phase 1 of iteration kt (stage kt+NS into slot cur), its B part in phase 0 of iteration
+  // kt+1 (same stage, same slot, by then called prv).
+  uint32_t cur = lds, prv = lds + (NS - 1) * STAGE;
+  const bool ragged = tail_mask < 4;
+  const uint32_t wave_lds = (uint32_t)wave * 4096u;   // this wave's 4 KiB share of an operand region
+  for (int kt = 0; kt < KT; ++kt) {
+    uint32_t nxt = cur + STAGE;
+    if (nxt == lds + NS * STAGE) nxt = lds;
+
+    // ---- phase 0: MFMAs of slice 0.  The eight fragment reads of slice 1 ride on the first
+    //      eight MFMAs so that they have returned by the time the barrier is reached; the B part
+    //      of stage kt-1+NS rides on the second eight. ----
+    const int kb = kt - 1 + NS;
+    const uint32_t sob = kb < KT ? (uint32_t)kb * lb.kstep : OOB;
+    if (ragged && kb == KT - 1) lb.mask_tail(lane, tail_mask);
+    const uint32_t b_target = prv + REGION + wave_lds;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int u = i * 4 + j;   // 0..15
+        if (u == 8) set_lds_target<0>(b_target);
+        if (u == 10) set_lds_target<1024>(b_target);
+        if (u == 12) set_lds_target<2048>(b_target);
+        if (u == 14) set_lds_target<3072>(b_target);
+        if (u >= 8 && (u & 1) == 0) SRT_FENCE();
+        acc[i][j] = mfma<T>(bf[0][j], af[0][i], acc[i][j]);
+        if (u >= 8 && (u & 1) == 0) {
+          SRT_FENCE();
+          load_to_lds_at_m0(rb, lb.voff[(u - 8) >> 1], sob);
+        }
+        // order of first use in phase 1: a0 b0 b1 b2 b3 a1 a2 a3
+        if (u == 0) af[1][0] = fa.read(cur, 0, 1);
+        else if (u >= 1 && u <= 4) bf[1][u - 1] = fb.read(cur + REGION, u - 1, 1);
+        else if (u >= 5 && u <= 7) af[1][u - 4] = fa.read(cur, u - 4, 1);
+        SRT_FENCE();
+      }
+    }
+
+    // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(8 * (NS - 2)) : "memory");
+    SRT_FENCE();
+
+    // ---- phase 1: MFMAs of slice 1; the A part of stage kt+NS goes into the slot just vacated
+    //      (even MFMAs 0..6), the reads of slice 0 of stage kt+1 ride on the odd MFMAs ----
+    const int ka = kt + NS;
+    const uint32_t soa = ka < KT ? (uint32_t)ka * la.kstep : OOB;
+    if (ragged && ka == KT - 1) la.mask_tail(lane, tail_mask);
+    const uint32_t a_target = cur + wave_lds;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int u = i * 4 + j;   // 0..15
+        if (u == 0) set_lds_target<0>(a_target);
+        if (u == 2) set_lds_target<1024>(a_target);
+        if (u == 4) set_lds_target<2048>(a_target);
+        if (u == 6) set_lds_target<3072>(a_target);
+        if (u < 8 && (u & 1) == 0) SRT_FENCE();
+        acc[i][j] = mfma<T>(bf[1][j], af[1][i], acc[i][j]);
+        if (u < 8 && (u & 1) == 0) {
+          SRT_FENCE();
+          load_to_lds_at_m0(ra, la.voff[u >> 1], soa);
+        }
+        if (u & 1) {
+          const int r = u >> 1;   // 0..7, same first-use order as above
+          if (r == 0) af[0][0] = fa.read(nxt, 0, 0);
+          else if (r <= 4) bf[0][r - 1] = fb.read(nxt + REGION, r - 1, 0);
+          else af[0][r - 4] = fa.read(nxt, r - 4, 0);
+        }
+        SRT_FENCE();
+      }
+    }
+    prv = cur;
+    cur = nxt;
+  }
+  // every load still in flight (all out of range by now, but still writing zeros into LDS) must
+  // retire, in every wave, before the LDS is reused as the epilogue's staging area
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  const uint32_t stage = lds + (uint32_t)wave * 16384u;
+
+  // ---- epilogue ----
+  if (TRANS_ACT) {
+    store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+  } else {
+    const bool any_nan = apply_linear_epilogue<T>(p, acc, m0 + wm0, n0 + wn0, lane);
+    if (any_nan) store_tile<T, true>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+    else store_tile<T, false>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+  }
+}
+
+#undef SRT_FENCE
+
+// Host-side preconditions beyond those of the MFMA family: every view must span less than 1 Gi
+// elements so 32-bit byte offsets reach it (including the rows of a partial last tile), and C
+// must take aligned 16-byte stores of eight whole columns.
+inline bool ring_fits(const GemmProblem& p, bool a_kc, bool b_kc) {
+  const long long lda = a_kc ? p.sam : p.sak, ldb = b_kc ? p.sbn : p.sbk;
+  const long long a_reach = a_kc ? ((long long)p.M + BM) * lda + p.K : ((long long)p.K + BK) * lda + p.M + BM;
+  const long long b_reach = b_kc ? ((long long)p.N + BN) * ldb + p.K : ((long long)p.K + BK) * ldb + p.N + BN;
+  const long long c_reach = ((long long)p.M + BM) * p.scm + p.N + BN;
+  const long long lim = 0x7fffffffLL / 2 - 4096;   // in elements: byte offsets stay below 2^31
+  if (!(a_reach < lim && b_reach < lim && c_reach < lim)) return false;
+  if ((p.N % 8) != 0 || (p.scm % 8) != 0 || (p.scb % 8) != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(p.C) & 15u) != 0) return false;
+  return true;
+}
+
+template <typename T, bool A_KC, bool B_KC, bool TRANS_ACT, int NS>
+hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_ring_kernel<T, A_KC, B_KC, TRANS_ACT, NS>;
+  constexpr int lds_bytes = NS * STAGE;
+  static bool configured = false;   // benign race: setting the attribute twice is harmless
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);
+  return hipGetLastError();
+}
+
+template <typename T, bool A_KC, bool B_KC, int NS = 5>
+hipError_t launch(const GemmProblem& p, hipStream_t stream) {
+  const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
+                     p.activation == srtActivationElu;
+  if (trans) return launch_kernel<T, A_KC, B_KC, true, NS>(p, stream);
+  return launch_kernel<T, A_KC, B_KC, false, NS>(p, stream);
+}
+
+}  // namespace ring
+}  // namespace srt
