@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+
+A step is one bf16 GEMM C = A.B with M = N = K = 8192 (row-major, no transposes, fp32
+accumulation, bf16 output) -- the configuration the headline metric is quoted on -- launched
+through the C ABI (srtMatmul) on the library's own stream, inputs resident in HBM.
+Inputs: A, B ~ N(0,1)/sqrt(K), seed 2 (Philox), rounded once to bf16.
+
+Prints ONE JSON line on stdout.  `value` is TFLOP/s over the K timed steps (wall clock between
+two stream synchronisations); `roofline.achieved` uses the average kernel duration measured
+with events recorded on the stream the kernel runs on.  `cpu_baseline` times the CPU oracle
+(the restated reference cpu_matmul, one thread) on a slab of rows of the same problem.
+--all additionally reports the other configurations (transposed lhs, Dense, skinny, batched
+fp16, fp32) on stderr.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0
+# HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/gemm_ring_bf16_8192_counters.txt); None until measured for the current kernel.
+TRAFFIC_BYTES_8192 = None
+
+
+def rng(seed):
+    return np.random.Generator(np.random.Philox(seed))
+
+
+def bf16_encode(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    r = ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    r[(u & 0x7FFFFFFF) > 0x7F800000] = 0x7FFF
+    return r
+
+
+def bf16_decode(h):
+    return (h.astype(np.uint32) << 16).view(np.float32)
+
+
+class Timer:
+    """Event pair on a queue's stream."""
+
+    def __init__(self, queue):
+        self.q = queue
+
+    def run(self, fn, steps):
+        start = self.q.record_event(timing=True)
+        for i in range(steps):
+            fn(i)
+        stop = self.q.record_event(timing=True)
+        stop.wait()
+        return stop.elapsed_ms_since(start)
+
+
+def time_steps(queue, fn, steps, warmup):
+    for i in range(warmup):
+        fn(i)
+    queue.wait_for_completion()
+    t0 = time.perf_counter()
+    ev_ms = Timer(queue).run(fn, steps)
+    queue.wait_for_completion()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms, ev_ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--all", action="store_true", help="also report the other configurations on stderr")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures the single-GPU matmul path; run it with --gpus 1 "
+                 "(the path shards over M or N with no exchange step, see DESIGN.md)")
+
+    import swiftrt_amd as srt
+    from swiftrt_amd import native
+
+    q = srt.current_queue()
+    props = srt.HipPlatform.local().devices[1].properties
+    n = 8192
+
+    g = rng(2)
+    a_st = bf16_encode(g.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n)))
+    b_st = bf16_encode(g.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n)))
+    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+    c = srt.Tensor(shape=[n, n], dtype=np.uint16)
+    a.device_read(q), b.device_read(q), c.device_read_write(q)
+
+    def step(_i):
+        q.matmul(a, False, b, False, c)
+
+    wall_ms, ev_ms = time_steps(q, step, args.steps, args.warmup)
+    flops = 2.0 * n * n * n
+    ms_per_step = wall_ms / args.steps
+    kernel_ms = ev_ms / args.steps
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+
+    # parity spot check of what was just timed: sampled rows against the fp64 GEMM
+    got = c.array()
+    rows = np.arange(0, n, 1024)
+    c64 = bf16_decode(a_st[rows]).astype(np.float64) @ bf16_decode(b_st).astype(np.float64)
+    max_rel = float(np.max(np.abs(bf16_decode(got[rows]).astype(np.float64) - c64)) / np.max(np.abs(c64)))
+    if not max_rel <= 2e-2:
+        sys.exit(f"parity check failed: max-norm relative error {max_rel} > 2e-2")
+
+    result = {
+        "metric": "bf16 GEMM TFLOP/s (8192^3, 1 MI355X)", "value": round(value, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "bf16 GEMM M=N=K=8192, row-major, no transposes, fp32 accumulate, bf16 out; "
+                               "A,B ~ N(0,1)/sqrt(K) seed 2; inputs resident in HBM",
+                   "entry_point": "srtMatmul", "kernel": "gemm_ring_kernel<BF16> 256x256x32, 5-stage LDS ring"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": TRAFFIC_BYTES_8192},
+        "max_rel_err_vs_fp64": max_rel,
+        "device": {"name": props.name.decode(), "arch": props.archName.decode(), "cus": props.multiProcessorCount,
+                   "peak_clock_mhz": props.clockRateKHz // 1000},
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(a_st, b_st, n)
+
+    if args.all:
+        report_other_configs(srt, q, a_st, b_st, n, args)
+
+    print(json.dumps(result), flush=True)
+
+
+def cpu_baseline(a_st, b_st, n):
+    """The CPU oracle (restated reference cpu_matmul: sequential k, fp32 multiply-then-add, one
+    thread, as the reference runs it) on a slab of rows of the same GEMM; also the host's
+    multi-core fp32 BLAS figure for the 'speedup vs host CPU' part of the metric."""
+    from oracle import srt_oracle as ora
+    rows = 24
+    t0 = time.perf_counter()
+    ora.matmul(a_st[:rows], b_st, acc=ora.ACC_VALUE)
+    dt = time.perf_counter() - t0
+    slab_flops = 2.0 * rows * n * n
+    out = {"value": round(slab_flops / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+           "sample": f"{rows} of {n} rows of C of the same bf16 GEMM ({dt:.1f} s), extrapolates linearly; the "
+                     "restatement omits the reference's per-element tensor-subscript overhead, so it is an upper "
+                     "bound on the reference's speed",
+           "host_cores": os.cpu_count()}
+    # all-core fp32 BLAS on a 2048-row slab (not the reference's algorithm; reported for scale only)
+    m = 2048
+    af = bf16_decode(a_st[:m])
+    bf = bf16_decode(b_st)
+    t0 = time.perf_counter()
+    af @ bf
+    dt2 = time.perf_counter() - t0
+    out["host_blas_fp32_tflops"] = round(2.0 * m * n * n / dt2 / 1e12, 4)
+    return out
+
+
+def report_other_configs(srt, q, a_st, b_st, n, args):
+    """Secondary configurations, human-readable on stderr."""
+    from swiftrt_amd import native
+
+    def line(name, ms, flops, nbytes, peak_key):
+        tf = flops / (ms * 1e-3) / 1e12
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        print(f"[bench] {name}: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s ({100 * tf / PEAK_TFLOPS[peak_key]:.1f}% of "
+              f"{peak_key} MFMA peak)  {gbs:.0f} GB/s algorithmic ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM peak)",
+              file=sys.stderr, flush=True)
+
+    def timed(fn, steps=args.steps, warmup=args.warmup):
+        _, ev = time_steps(q, fn, steps, warmup)
+        return ev / steps
+
+    # cfg3 with transposeLhs: A stored K x M
+    at = srt.Tensor(np.ascontiguousarray(a_st.T))
+    b = srt.Tensor(b_st)
+    c = srt.Tensor(shape=[n, n], dtype=np.uint16)
+    at.device_read(q), b.device_read(q), c.device_read_write(q)
+    line("cfg3 bf16 8192^3 transposeLhs", timed(lambda i: q.matmul(at, True, b, False, c)), 2.0 * n ** 3, 3 * n * n * 2, "bf16")
+    del at, c
+
+    # cfg4 Dense
+    g = rng(3)
+    x = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))
+    w = srt.Tensor(bf16_encode(g.standard_normal((4096, 11008), dtype=np.float32) / np.float32(64)))
+    bias = srt.Tensor(bf16_encode(g.uniform(-0.1, 0.1, 11008).astype(np.float32)))
+    y = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+    for t in (x, w, bias):
+        t.device_read(q)
+    y.device_read_write(q)
+    line("cfg4 Dense bf16 4096x4096x11008 +bias +relu",
+         timed(lambda i: q.matmul(x, False, w, False, y, bias=bias, activation=srt.ActivationType.relu)),
+         2.0 * 4096 * 4096 * 11008, (4096 * 4096 + 4096 * 11008 * 2 + 11008) * 2, "bf16")
+    del x, w, y
+
+    # cfg5 skinny: rotate 4 weight buffers so the weight is not served from the last-level cache
+    g = rng(4)
+    wbase = bf16_encode(g.standard_normal((14336, 4096), dtype=np.float32) / np.float32(64))
+    ws = [srt.Tensor(wbase.copy()) for _ in range(4)]
+    for t in ws:
+        t.device_read(q)
+    for m in (1, 8, 32):
+        xs = srt.Tensor(bf16_encode(g.standard_normal((m, 4096), dtype=np.float32)))
+        o = srt.Tensor(shape=[m, 14336], dtype=np.uint16)
+        xs.device_read(q), o.device_read_write(q)
+        line(f"cfg5 skinny bf16 M={m} K=4096 N=14336 transposeRhs",
+             timed(lambda i: q.matmul(xs, False, ws[i % 4], True, o), steps=200, warmup=20),
+             2.0 * m * 4096 * 14336, 2 * (m * 4096 + 14336 * 4096 + m * 14336), "bf16")
+    del ws
+
+    # cfg2 batched fp16
+    g = rng(1)
+    a2 = srt.Tensor((g.standard_normal((32, 256, 256)) * 0.1).astype(np.float16))
+    b2 = srt.Tensor((g.standard_normal((32, 256, 256)) * 0.1).astype(np.float16))
+    c2 = srt.Tensor(shape=[32, 256, 256], dtype=np.float16)
+    a2.device_read(q), b2.device_read(q), c2.device_read_write(q)
+    line("cfg2 fp16 batch 32 x 256^3 transposeRhs", timed(lambda i: q.matmul(a2, False, b2, True, c2), steps=200, warmup=20),
+         2.0 * 32 * 256 ** 3, 32 * 3 * 256 * 256 * 2, "f16")
+
+    # cfg1 fp32
+    g = rng(0)
+    a1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
+    b1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
+    c1 = srt.Tensor(shape=[512, 512], dtype=np.float32)
+    a1.device_read(q), b1.device_read(q), c1.device_read_write(q)
+    line("cfg1 fp32 512^3", timed(lambda i: q.matmul(a1, False, b1, False, c1), steps=200, warmup=20),
+         2.0 * 512 ** 3, 3 * 512 * 512 * 4, "f32")
+
+
+if __name__ == "__main__":
+    main()

@@ -313,6 +313,49 @@ def test_every_activation_vs_oracle(act, dt):
     assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1.0))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("act", list(srt.ActivationType))
+def test_ring_kernel_epilogues_vs_oracle(act, dt):
+    """Every activation (+ bias) through the 256 x 256 ring kernel, ragged M / N / K edges."""
+    r = H.rng(16)
+    M, N, K = 3600, 3592, 72
+    x = H.encode(r.standard_normal((M, K)).astype(np.float32), dt)
+    w = H.encode((r.standard_normal((K, N)) / 8).astype(np.float32), dt)
+    b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
+    coef = 0.75
+    xt, wt = srt.Tensor(x), srt.Tensor(w)
+    out = srt.Tensor(shape=[M, N], dtype=x.dtype)
+    assert query_kernel(xt, False, wt, False, out) == "mfma_256x256"
+    layer = srt.Dense(wt, srt.Tensor(b), act, relu_ceiling=coef, elu_alpha=coef)
+    got = H.decode(layer(xt).array())
+    rows = np.concatenate([np.arange(0, M, 211), [M - 1]])
+    want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, acc=ora.ACC_F32, fused=True))
+    tol = {H.F16: 2.0 ** -10, H.BF16: 2.0 ** -7}[dt]
+    assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
+
+
+def test_ring_kernel_nan_and_inf_encode_like_the_reference():
+    """A NaN anywhere in a tile switches the wave to the exact encoder: NaN -> 0x7FFF, inf stays inf."""
+    M = N = 3584
+    K = 64
+    a = np.zeros((M, K), np.float32)
+    b = np.zeros((K, N), np.float32)
+    a[:, 0] = 1.0
+    b[0, :] = 2.0
+    a[5, 1] = np.nan       # row 5 of C becomes NaN
+    a[300, 2] = np.inf     # row 300 becomes inf (inf * 0 products avoided: only column k=2 of b is nonzero below)
+    b[2, :] = 1.0
+    b[1, :] = 1.0
+    got = gpu_matmul(H.encode(a, H.BF16), H.encode(b, H.BF16), want_kernel="mfma_256x256")
+    assert np.all(got[5] == 0x7FFF)
+    assert np.all(got[300] == 0x7F80)
+    assert np.all(got[6] == H.encode(np.array([2.0], np.float32), H.BF16)[0])
+    # relu maps the NaN row to 0 (x > 0 ? x : 0), identity keeps it
+    layer = srt.Dense(srt.Tensor(H.encode(b, H.BF16)), None, srt.ActivationType.relu)
+    y = layer(srt.Tensor(H.encode(a, H.BF16))).array()
+    assert np.all(y[5] == 0) and np.all(y[300] == 0x7F80)
+
+
 # ---- error behaviour -----------------------------------------------------------------------------
 def test_not_supported_and_invalid_value_surface_as_in_the_reference():
     q = srt.current_queue()
