@@ -82,6 +82,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--all", action="store_true", help="also report the other configurations on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run three 256 MiB device-to-device copies (known traffic, for scaling the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the single-GPU matmul path; run it with --gpus 1 "
@@ -91,6 +94,15 @@ def main():
     from swiftrt_amd import native
 
     q = srt.current_queue()
+    if args.copy_calibration:
+        nbytes = 256 << 20
+        src, dst = q.allocate(nbytes), q.allocate(nbytes)
+        native.check(native.lib().srtMemsetAsync(ctypes.c_void_p(src.pointer), 1, nbytes, q.stream))
+        for _ in range(3):
+            q.copy_async(src, dst)
+        q.wait_for_completion()
+        print(json.dumps({"copy_calibration_bytes": nbytes, "copies": 3}))
+        return
     props = srt.HipPlatform.local().devices[1].properties
     n = 8192
 
