@@ -30,8 +30,8 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/gemm_ring_bf16_8192_counters.txt); None until measured for the current kernel.
-TRAFFIC_BYTES_8192 = None
+# and scaled by a 256 MiB device copy (profiles/gemm_ring_bf16_8192_counters.txt).
+TRAFFIC_BYTES_8192 = 1.749e9   # 2.000 x FETCH_SIZE (788 266 KiB) + 1.000 x WRITE_SIZE (131 072 KiB)
 
 
 def rng(seed):
@@ -159,7 +159,7 @@ def cpu_baseline(a_st, b_st, n):
     thread, as the reference runs it) on a slab of rows of the same GEMM; also the host's
     multi-core fp32 BLAS figure for the 'speedup vs host CPU' part of the metric."""
     from oracle import srt_oracle as ora
-    rows = 24
+    rows = 64
     t0 = time.perf_counter()
     ora.matmul(a_st[:rows], b_st, acc=ora.ACC_VALUE)
     dt = time.perf_counter() - t0

@@ -95,3 +95,15 @@ def test_using_queue_scope_and_two_queues():
         b = srt.matmul(a, a)
     c = srt.matmul(b, a)           # consumed on queue 0: ordered after queue 1 through an event
     assert np.array_equal(c.array(), np.full((8, 8), 2 * 2 * 8 * 2 * 8, np.float32))
+
+
+def test_cpp_host_mirror_runs_the_reference_kats():
+    """The C++ mirror of the Swift host types (swiftrt_amd/host/srt_host.hpp) over the C ABI."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "host_mirror_test")
+    assert os.path.exists(exe), "tests/host_mirror_test is built by __graft_entry__.build()"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "all checks passed" in out.stdout
