@@ -280,6 +280,18 @@ __device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x
   return __builtin_amdgcn_ballot_w64(nan) != 0;
 }
 
+// NaN test alone, for the plain matmul case.
+__device__ __forceinline__ bool any_nan_in_tile(const f32x16_t (&acc)[4][4]) {
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; v += 2) nan |= __builtin_isunordered(acc[i][j][v], acc[i][j][v + 1]);
+  return __builtin_amdgcn_ballot_w64(nan) != 0;
+}
+
 // Step 2 (store_tile): one rounding to the element type, then a trip through LDS so that global
 // stores are whole 16-byte chunks of C rows (a store instruction writes four 256-byte row
 // segments instead of 64 scattered pieces).  The wave's 128 x 128 result goes in two halves of
@@ -386,7 +398,12 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
   }
 }
 
-template <typename T, bool A_KC, bool B_KC, bool TRANS_ACT, int NS>
+// EPI selects the epilogue the kernel is compiled with (the accumulators never cross a branch).
+constexpr int EPI_PLAIN = 0;    // matmul: no bias, identity
+constexpr int EPI_LINEAR = 1;   // bias and/or relu / clippedRelu
+constexpr int EPI_TRANS = 2;    // sigmoid / tanh / elu (+ bias)
+
+template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
   static_assert(NS >= 3 && NS <= 5, "ring depth");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
@@ -547,10 +564,11 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
   const uint32_t stage = lds + (uint32_t)wave * 16384u;
 
   // ---- epilogue ----
-  if (TRANS_ACT) {
+  if (EPI == EPI_TRANS) {
     store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   } else {
-    const bool any_nan = apply_linear_epilogue<T>(p, acc, m0 + wm0, n0 + wn0, lane);
+    // EPI_PLAIN (no bias, identity): the accumulators are final as they are
+    const bool any_nan = EPI == EPI_PLAIN ? any_nan_in_tile(acc) : apply_linear_epilogue<T>(p, acc, m0 + wm0, n0 + wn0, lane);
     if (any_nan) store_tile<T, true>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
     else store_tile<T, false>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   }
@@ -573,9 +591,9 @@ inline bool ring_fits(const GemmProblem& p, bool a_kc, bool b_kc) {
   return true;
 }
 
-template <typename T, bool A_KC, bool B_KC, bool TRANS_ACT, int NS>
+template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
-  auto kernel = gemm_ring_kernel<T, A_KC, B_KC, TRANS_ACT, NS>;
+  auto kernel = gemm_ring_kernel<T, A_KC, B_KC, EPI, NS>;
   constexpr int lds_bytes = NS * STAGE;
   static bool configured = false;   // benign race: setting the attribute twice is harmless
   if (!configured) {
@@ -593,8 +611,9 @@ template <typename T, bool A_KC, bool B_KC, int NS = 5>
 hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
                      p.activation == srtActivationElu;
-  if (trans) return launch_kernel<T, A_KC, B_KC, true, NS>(p, stream);
-  return launch_kernel<T, A_KC, B_KC, false, NS>(p, stream);
+  if (trans) return launch_kernel<T, A_KC, B_KC, EPI_TRANS, NS>(p, stream);
+  if (p.bias == nullptr && p.activation == srtActivationIdentity) return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS>(p, stream);
+  return launch_kernel<T, A_KC, B_KC, EPI_LINEAR, NS>(p, stream);
 }
 
 }  // namespace ring

@@ -1,16 +1,21 @@
 // Small-M matmul (M <= 32) against a k-contiguous weight: out[m, n] = sum_k x[m, k] * W[n, k].
 // The shape of single-token / small-batch inference; bound by streaming W from HBM once.
 //
-// No LDS staging and no barrier in the k loop: the MFMA B-operand layout (lane l holds 8
-// consecutive k of column l % 32) is exactly a 16-byte global load of row n of W, so each lane
-// loads its operand straight from memory.  The order of k inside one MFMA is free as long as
-// both operands agree, so lane (n, h) reads the 64 contiguous bytes k0 + 32 h .. k0 + 32 h + 31
-// (four 16-byte loads, one per MFMA step) and a wave consumes whole 128-byte lines of each row.
-//   block   4 waves share 32 rows of W (one 32 x 32 output tile, rows m >= M are zero);
-//           wave w takes the 64-wide k blocks w, w + 4, ...; partial tiles are summed through
+//   block   4 waves share 32 rows of W (one 32 x 32 output tile; rows m >= M are zero).  Wave w
+//           takes the 64-wide k blocks w, w + 4, ...; the four partial tiles are summed through
 //           LDS once at the end, then bias + activation + store.
-//   grid    ceil(N / 32) x batch workgroups, all resident at once: the HBM pipe sees
-//           every row's stream concurrently.
+//   W       streams HBM -> LDS with `buffer_load_dwordx4 ... lds`, fully coalesced: one load
+//           instruction fetches 8 rows x 128 contiguous bytes (whole cache lines), four per k
+//           block.  Each wave owns a private ring of DEPTH k blocks in LDS (no workgroup barrier
+//           in the k loop, only s_waitcnt on the wave's own loads), so DEPTH (2-3) x 4 KiB per wave
+//           are in flight at any time.  LDS layout per block: [32 rows][8 chunks of 16 B], chunk c
+//           of row r at c ^ ((r >> 1) & 7): the MFMA B-operand read (lane l: row l % 32, chunk
+//           2 s + l / 32) is one conflict-free ds_read_b128.
+//   x       is tiny and hits in L2; its rows for the same k block ride in the same ring slot
+//           (8, 16 or 32 staged rows, one load instruction per 8), so the k loop's only
+//           vector-memory instructions are global->LDS loads and its only register-producing
+//           loads are LDS reads.
+//   grid    ceil(N / 32) x batch workgroups of 60-72 KiB LDS: two per CU, all resident at once.
 #include "gemm_common.h"
 
 namespace srt {
@@ -21,6 +26,7 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+#define SRT_LDS __attribute__((address_space(3)))
 
 template <typename T>
 __device__ __forceinline__ f32x16_t mfma32s(u32x4_t a, u32x4_t b, f32x16_t c);
@@ -36,29 +42,40 @@ __device__ __forceinline__ f32x16_t mfma32s<F16>(u32x4_t a, u32x4_t b, f32x16_t 
 }
 
 constexpr int SK_WAVES = 4;
-constexpr int SK_KB = 64;  // k per block step
+constexpr int SK_KB = 64;          // k per block step (128 bytes per row)
+constexpr int SK_WBYTES = 32 * 128;   // W part of a ring slot: 32 rows x 128 B
+constexpr uint32_t SK_OOB = 0x80000000u;
 
-struct Frag4 {
-  u32x4_t c[4];
+// ring depth per x-row capacity: two workgroups per CU must fit in 160 KiB of LDS
+template <int XR>
+struct SkinnyShape {
+  static constexpr int DEPTH = XR == 32 ? 2 : 3;           // k blocks in flight per wave
+  static constexpr int SLOT = SK_WBYTES + XR * 128;         // W rows + x rows of one k block
+  static constexpr int LOADS = 4 + XR / 8;                  // load instructions per k block
+  static constexpr int LDS = SK_WAVES * DEPTH * SLOT;       // 60 / 72 / 64 KiB
 };
 
-// four 16-byte chunks at row_ptr + k0 + 32 h + 8 s, zero beyond K
-__device__ __forceinline__ void load_frag(Frag4& f, const uint16_t* row_ptr, int k0, int h, int K, bool row_ok) {
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int k = k0 + 32 * h + 8 * s;
-    u32x4_t x = {0u, 0u, 0u, 0u};
-    if (row_ok && k < K) x = *reinterpret_cast<const u32x4_t*>(row_ptr + k);
-    f.c[s] = x;
-  }
+__device__ __forceinline__ void sk_load_to_lds(u32x4_t rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
 }
 
-template <typename T>
+// XR = number of x rows staged per k block (8, 16 or 32 >= M).
+// Every vector-memory instruction in the k loop is a global->LDS load issued from inline assembly
+// and awaited with explicit s_waitcnt vmcnt; everything that produces registers is an LDS read,
+// which the compiler tracks on its own counter.
+template <typename T, int XR>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem p) {
-  __shared__ float red[SK_WAVES][16][64];
+  using Shape = SkinnyShape<XR>;
+  constexpr int DEPTH = Shape::DEPTH;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char sk_lds_raw[];
+  const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)sk_lds_raw;
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
   const int n0 = blockIdx.x * 32;
   const int bz = blockIdx.y;
@@ -66,50 +83,105 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   const uint16_t* X = (const uint16_t*)p.A + (long long)bz * p.sab;
   const uint16_t* W = (const uint16_t*)p.B + (long long)bz * p.sbb;
 
-  const int n = n0 + r;
-  const bool n_ok = n < p.N;
-  const bool m_ok = r < p.M;
-  const uint16_t* wrow = W + (long long)(n_ok ? n : 0) * p.sbn;
-  const uint16_t* xrow = X + (long long)(m_ok ? r : 0) * p.sam;
+  // both operands through bounds-checked buffers: rows >= N (>= M) and k >= K read zero
+  const uint32_t w_bytes = (uint32_t)(((long long)(p.N - 1) * p.sbn + p.K) * 2);
+  const uint64_t wp = reinterpret_cast<uint64_t>(W);
+  const u32x4_t rw = {(uint32_t)wp, (uint32_t)(wp >> 32) & 0xffffu, w_bytes, 0x00020000u};
+  const uint32_t x_bytes = (uint32_t)(((long long)(p.M - 1) * p.sam + p.K) * 2);
+  const uint64_t xp = reinterpret_cast<uint64_t>(X);
+  const u32x4_t rx = {(uint32_t)xp, (uint32_t)(xp >> 32) & 0xffffu, x_bytes, 0x00020000u};
+
+  // A load instruction covers 8 rows x 128 contiguous bytes (8 lanes per row); the lane fetches
+  // the 16-byte chunk that belongs at its landing position (chunk c of row r sits at
+  // c ^ ((r >> 1) & 7)).  (row >> 1) & 7 only depends on the lane, not on which group of 8 rows.
+  const int lrow = lane >> 3;
+  const int lchunk = (lane & 7) ^ ((lrow >> 1) & 3) ^ 0;   // rows 8 i + lrow: ((8 i + lrow) >> 1) & 7 = 4 (i & 1) + (lrow >> 1)
+  uint32_t wvoff[4], xvoff[XR / 8];
+  int wchunk[4], xchunk[XR / 8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 8 * i + lrow;
+    wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
+    const int n = n0 + row;
+    wvoff[i] = n < p.N ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * 8) * 2) : SK_OOB;
+  }
+#pragma unroll
+  for (int i = 0; i < XR / 8; ++i) {
+    const int row = 8 * i + lrow;
+    xchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
+    xvoff[i] = row < p.M ? (uint32_t)(((long long)row * p.sam + xchunk[i] * 8) * 2) : SK_OOB;
+  }
+  (void)lchunk;
+  const uint32_t my_ring = lds + (uint32_t)wave * (DEPTH * Shape::SLOT);
+
+  // fragment read address inside a region: row r, chunk 2 s + h, swizzled
+  uint32_t rd[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) rd[s] = (uint32_t)(r * 128 + (((2 * s + h) ^ ((r >> 1) & 7)) << 4));
+  const bool x_lane = r < XR;   // lanes of rows that are not staged hold zero operands
+
+  const int KB = (p.K + SK_KB - 1) / SK_KB;   // k blocks in total; this wave takes wave, wave + 4, ...
+  const int k_chunks = p.K / 8;                // valid 16-byte chunks per row
+
+  auto issue = [&](int kb, int slot) {
+    const bool live = kb < KB;
+    const uint32_t base = my_ring + (uint32_t)slot * Shape::SLOT;
+    const uint32_t soff = (uint32_t)kb * (SK_KB * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool in_k = live && (kb * 8 + wchunk[i]) < k_chunks;
+      sk_load_to_lds(rw, base + (uint32_t)i * 1024u, in_k ? wvoff[i] : SK_OOB, soff);
+    }
+#pragma unroll
+    for (int i = 0; i < XR / 8; ++i) {
+      const bool in_k = live && (kb * 8 + xchunk[i]) < k_chunks;
+      sk_load_to_lds(rx, base + SK_WBYTES + (uint32_t)i * 1024u, in_k ? xvoff[i] : SK_OOB, soff);
+    }
+  };
 
   f32x16_t acc;
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
 
-  const int KB = (p.K + SK_KB - 1) / SK_KB;
-  Frag4 w0, x0, w1, x1;
-  int kb = wave;
-  if (kb < KB) {
-    load_frag(w0, wrow, kb * SK_KB, h, p.K, n_ok);
-    load_frag(x0, xrow, kb * SK_KB, h, p.K, m_ok);
-  }
-  // two k blocks per trip: loads for the next pair are in flight while this pair multiplies
-  for (; kb < KB; kb += 2 * SK_WAVES) {
-    const int kb1 = kb + SK_WAVES;
-    const bool has1 = kb1 < KB;
-    if (has1) {
-      load_frag(w1, wrow, kb1 * SK_KB, h, p.K, n_ok);
-      load_frag(x1, xrow, kb1 * SK_KB, h, p.K, m_ok);
-    }
 #pragma unroll
-    for (int s = 0; s < 4; ++s) acc = mfma32s<T>(x0.c[s], w0.c[s], acc);
-    const int kb2 = kb1 + SK_WAVES;
-    if (kb2 < KB) {
-      load_frag(w0, wrow, kb2 * SK_KB, h, p.K, n_ok);
-      load_frag(x0, xrow, kb2 * SK_KB, h, p.K, m_ok);
-    }
-    if (has1) {
-#pragma unroll
-      for (int s = 0; s < 4; ++s) acc = mfma32s<T>(x1.c[s], w1.c[s], acc);
-    }
-  }
+  for (int d = 0; d < DEPTH; ++d) issue(wave + SK_WAVES * d, d);
 
+  // Each trip consumes DEPTH blocks; block d of the trip was issued DEPTH blocks ago.  Loads
+  // retire in order and every block issues exactly LOADS of them (out-of-range ones included),
+  // so a block has landed once at most LOADS (DEPTH - 1) younger loads remain outstanding.
+  for (int kb = wave; kb < KB; kb += SK_WAVES * DEPTH) {
 #pragma unroll
-  for (int v = 0; v < 16; ++v) red[wave][v][lane] = acc[v];
+    for (int d = 0; d < DEPTH; ++d) {
+      const int kcur = kb + SK_WAVES * d;
+      asm volatile("s_waitcnt vmcnt(%0)" : : "i"(Shape::LOADS * (DEPTH - 1)) : "memory");
+      const uint32_t base = my_ring + (uint32_t)d * Shape::SLOT;
+      u32x4_t wf[4], xf[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        wf[s] = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + rd[s]);
+        u32x4_t x = {0u, 0u, 0u, 0u};
+        if (x_lane) x = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + SK_WBYTES + rd[s]);
+        xf[s] = x;
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot is free
+      issue(kcur + SK_WAVES * DEPTH, d);
+      if (kcur < KB) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc = mfma32s<T>(xf[s], wf[s], acc);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();   // every wave's loads have landed and its ring is idle: reuse LDS for the reduction
+
+  float* red = reinterpret_cast<float*>(sk_lds_raw);   // [4 waves][16][64] = 16 KiB
+#pragma unroll
+  for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[v];
   __syncthreads();
 
   // wave w finishes accumulator registers 4w .. 4w+3: rows m = 8 w + 4 h + i, column n
-  if (!n_ok) return;
+  const int n = n0 + r;
+  if (n >= p.N) return;
   Epilogue<T> ep(p);
   uint16_t* C = (uint16_t*)p.C + (long long)bz * p.scb;
   const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
@@ -120,10 +192,32 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     if (m >= p.M) continue;
     float s = 0.0f;
 #pragma unroll
-    for (int w = 0; w < SK_WAVES; ++w) s += red[w][v][lane];
+    for (int w = 0; w < SK_WAVES; ++w) s += red[(w * 16 + v) * 64 + lane];
     const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
     C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, bv);
   }
+}
+
+template <typename T, int XR>
+hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_skinny_kernel<T, XR>;
+  constexpr int lds_bytes = SkinnyShape<XR>::LDS;
+  static bool configured = false;   // benign race: setting the attribute twice is harmless
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3((p.N + 31) / 32, p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
+  if (p.M <= 8) return launch_skinny_shape<T, 8>(p, stream);
+  if (p.M <= 16) return launch_skinny_shape<T, 16>(p, stream);
+  return launch_skinny_shape<T, 32>(p, stream);
 }
 
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
@@ -141,16 +235,15 @@ bool skinny_supported(const GemmProblem& p) {
   if (p.sam < 0 || p.sbn < 0 || p.scm < 0 || p.scn < 0) return false;
   if (!aligned16(p.A) || !aligned16(p.B)) return false;
   if (p.batch > 65535) return false;
+  // 32-bit byte offsets must reach every row of W (and stay below the out-of-range marker)
+  if (((long long)p.N + 32) * p.sbn + p.K >= (0x7fffffffLL / 2 - 4096)) return false;
   // worth it only when the weight dominates the traffic
   return p.N >= 32;
 }
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t stream) {
-  dim3 grid((p.N + 31) / 32, p.batch);
-  dim3 block(SK_WAVES * 64);
-  if (p.dtype == srtReal16BF) hipLaunchKernelGGL(gemm_skinny_kernel<BF16>, grid, block, 0, stream, p);
-  else hipLaunchKernelGGL(gemm_skinny_kernel<F16>, grid, block, 0, stream, p);
-  return hipGetLastError();
+  if (p.dtype == srtReal16BF) return launch_skinny_type<BF16>(p, stream);
+  return launch_skinny_type<F16>(p, stream);
 }
 
 }  // namespace srt
