@@ -143,16 +143,29 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
 
+  // This wave's k blocks are wave, wave + 4, ... (count of them); it walks them in rotated
+  // order, starting at a block that depends on the workgroup, so that the workgroups resident at
+  // one time are spread over different byte offsets of their rows -- with rows a power of two
+  // apart, all workgroups reading the same offset would hammer the same few memory channels.
+  const int count = KB > wave ? (KB - wave + SK_WAVES - 1) / SK_WAVES : 0;
+  const int rot = count > 0 ? (int)((blockIdx.x * 7u) % (unsigned)count) : 0;
+  auto block_at = [&](int j) {   // j-th block of the walk, or KB (= nothing) past the end
+    if (j >= count) return KB;
+    int jj = j + rot;
+    if (jj >= count) jj -= count;
+    return wave + SK_WAVES * jj;
+  };
+
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) issue(wave + SK_WAVES * d, d);
+  for (int d = 0; d < DEPTH; ++d) issue(block_at(d), d);
 
   // Each trip consumes DEPTH blocks; block d of the trip was issued DEPTH blocks ago.  Loads
   // retire in order and every block issues exactly LOADS of them (out-of-range ones included),
   // so a block has landed once at most LOADS (DEPTH - 1) younger loads remain outstanding.
-  for (int kb = wave; kb < KB; kb += SK_WAVES * DEPTH) {
+  for (int j0 = 0; j0 < count; j0 += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      const int kcur = kb + SK_WAVES * d;
+      const int j = j0 + d;
       asm volatile("s_waitcnt vmcnt(%0)" : : "i"(Shape::LOADS * (DEPTH - 1)) : "memory");
       const uint32_t base = my_ring + (uint32_t)d * Shape::SLOT;
       u32x4_t wf[4], xf[4];
@@ -164,8 +177,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
         xf[s] = x;
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot is free
-      issue(kcur + SK_WAVES * DEPTH, d);
-      if (kcur < KB) {
+      issue(block_at(j + DEPTH), d);
+      if (j < count) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) acc = mfma32s<T>(xf[s], wf[s], acc);
       }
