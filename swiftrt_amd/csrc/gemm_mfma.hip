@@ -348,10 +348,11 @@ int mfma_select(const GemmProblem& p) {
   if (p.sam < 0 || p.sak < 0 || p.sbk < 0 || p.sbn < 0 || p.scm < 0) return 0;
 
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
+  // Largest tile that still gives every CU work: 256 x 256 (ring kernel) from 192 tiles up, 128 x 128
+  // from one tile per CU up, otherwise 64 x 64 (measured on batch 32 x 256^3: 7.7 us against 15.0 us).
   int tile;
   if (tiles(256) >= 192 && ring_fits_problem(p, a_kc, b_kc)) tile = 1;
-  else if (tiles(128) >= 192) tile = 2;
-  else if (p.M > 64 && p.N > 64 && tiles(128) * 4 >= tiles(64)) tile = tiles(128) >= 64 ? 2 : 3;
+  else if (tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | (a_kc ? 2 : 0) | (b_kc ? 1 : 0);
 }

@@ -234,43 +234,50 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
 // acc[i][j] is a transposed 32 x 32 tile: lane l owns row m = wave_m0 + 32 i + l % 32 and, in
 // registers 4 g .. 4 g + 3, the columns n = wave_n0 + 32 j + 8 g + 4 (l / 32) + 0..3.
 //
-// Step 1 for identity / relu / clippedRelu (apply_linear_epilogue): bias, then the activation
-// as two branch-free selects driven by uniform parameters, in place and in straight-line code
-// (the accumulators never cross a branch).  Returns whether any lane of the wave holds a NaN,
-// so the rounding step can use the one-instruction hardware converter when there is none.
-template <typename T>
+// Step 1 for identity / relu / clippedRelu (apply_linear_epilogue): bias, then the activation as
+// one or two min/max instructions, in place and in straight-line code (the accumulators never
+// cross a branch); HAS_BIAS and CLAMP are compile-time so each variant carries only the
+// instructions it needs.  CLAMP: 0 none, 1 relu = max(x, 0), 2 clippedRelu = min(max(x, 0), coef).
+// max(NaN, 0) is 0 on this hardware, which is also what x > 0 ? x : 0 gives.
+// Returns whether any lane of the wave holds a NaN, so the rounding step can use the
+// one-instruction hardware converter when there is none.
+template <typename T, bool HAS_BIAS, int CLAMP>
 __device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x16_t (&acc)[4][4], int wave_m0,
                                                       int wave_n0, int lane) {
   using S = typename T::storage;
   const S* bias = (const S*)p.bias;
   const bool per_row = p.bias_per_row != 0;
-  const bool clamp_low = p.activation == srtActivationRelu || p.activation == srtActivationClippedRelu;
-  const float ceiling = p.activation == srtActivationClippedRelu ? p.coef : __builtin_inff();
+  const float ceiling = p.coef;
   const int r = lane & 31, h = lane >> 5;
-  float brow[4];
+  float brow[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (HAS_BIAS) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = wave_m0 + 32 * i + r;
-    brow[i] = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+    for (int i = 0; i < 4; ++i) {
+      const int m = wave_m0 + 32 * i + r;
+      brow[i] = (per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+    }
   }
   bool nan = false;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      float bcol[4];
+      float bcol[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (HAS_BIAS) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
-        bcol[e] = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+        for (int e = 0; e < 4; ++e) {
+          const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
+          bcol[e] = (!per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+        }
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float x = acc[i][j][4 * g + e] + (per_row ? brow[i] : bcol[e]);
-          x = (clamp_low && !(x > 0.0f)) ? 0.0f : x;   // relu: x > 0 ? x : 0 (a NaN becomes 0, as max(x, 0) gives)
-          x = x > ceiling ? ceiling : x;               // identity: ceiling = +inf keeps x, NaN included
+          float x = acc[i][j][4 * g + e];
+          if (HAS_BIAS) x += per_row ? brow[i] : bcol[e];
+          if (CLAMP >= 1) x = __builtin_fmaxf(x, 0.0f);
+          if (CLAMP == 2) x = __builtin_fminf(x, ceiling);
           acc[i][j][4 * g + e] = x;
         }
         nan |= __builtin_isunordered(acc[i][j][4 * g], acc[i][j][4 * g + 1]);
@@ -399,9 +406,12 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
 }
 
 // EPI selects the epilogue the kernel is compiled with (the accumulators never cross a branch).
-constexpr int EPI_PLAIN = 0;    // matmul: no bias, identity
-constexpr int EPI_LINEAR = 1;   // bias and/or relu / clippedRelu
-constexpr int EPI_TRANS = 2;    // sigmoid / tanh / elu (+ bias)
+constexpr int EPI_PLAIN = 0;       // matmul: no bias, identity
+constexpr int EPI_BIAS = 1;        // bias, identity
+constexpr int EPI_RELU = 2;        // relu
+constexpr int EPI_BIAS_RELU = 3;   // bias, relu (the Dense configuration)
+constexpr int EPI_CLIPPED = 4;     // clippedRelu, bias optional (a null bias adds nothing)
+constexpr int EPI_TRANS = 5;       // sigmoid / tanh / elu (+ bias)
 
 template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
@@ -583,8 +593,13 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
   if (EPI == EPI_TRANS) {
     store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   } else {
-    // EPI_PLAIN (no bias, identity): the accumulators are final as they are
-    const bool any_nan = EPI == EPI_PLAIN ? any_nan_in_tile(acc) : apply_linear_epilogue<T>(p, acc, m0 + wm0, n0 + wn0, lane);
+    bool any_nan;
+    if (EPI == EPI_PLAIN) any_nan = any_nan_in_tile(acc);   // the accumulators are final as they are
+    else if (EPI == EPI_BIAS) any_nan = apply_linear_epilogue<T, true, 0>(p, acc, m0 + wm0, n0 + wn0, lane);
+    else if (EPI == EPI_RELU) any_nan = apply_linear_epilogue<T, false, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
+    else if (EPI == EPI_BIAS_RELU) any_nan = apply_linear_epilogue<T, true, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
+    else any_nan = p.bias ? apply_linear_epilogue<T, true, 2>(p, acc, m0 + wm0, n0 + wn0, lane)
+                          : apply_linear_epilogue<T, false, 2>(p, acc, m0 + wm0, n0 + wn0, lane);
     if (any_nan) store_tile<T, true>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
     else store_tile<T, false>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   }
@@ -628,8 +643,13 @@ hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
                      p.activation == srtActivationElu;
   if (trans) return launch_kernel<T, A_KC, B_KC, EPI_TRANS, NS>(p, stream);
-  if (p.bias == nullptr && p.activation == srtActivationIdentity) return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS>(p, stream);
-  return launch_kernel<T, A_KC, B_KC, EPI_LINEAR, NS>(p, stream);
+  if (p.activation == srtActivationClippedRelu) return launch_kernel<T, A_KC, B_KC, EPI_CLIPPED, NS>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS_RELU, NS>(p, stream);
+    return launch_kernel<T, A_KC, B_KC, EPI_RELU, NS>(p, stream);
+  }
+  if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS, NS>(p, stream);
+  return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS>(p, stream);
 }
 
 }  // namespace ring

@@ -140,7 +140,7 @@ def test_integer_inputs_bit_exact_vs_oracle(dt, ta, tb):
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("M,N,K,kernel", [(200, 264, 72, "mfma_64x64"), (1000, 1032, 136, "mfma_128x128"),
+@pytest.mark.parametrize("M,N,K,kernel", [(200, 264, 72, "mfma_64x64"), (2040, 2056, 136, "mfma_128x128"),
                                           (4000, 3976, 200, "mfma_256x256")])
 def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, kernel):
     """Aligned shapes with ragged edges in M, N and K, every tile config and staging layout."""
