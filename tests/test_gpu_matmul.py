@@ -337,6 +337,46 @@ def test_ring_kernel_epilogues_vs_oracle(act, dt):
     assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_ring_kernel_batched_broadcast_and_column_major(dt):
+    """Rank-3 operands through the 256 x 256 ring kernel: strided batch, a broadcast (stride 0) weight,
+    and a column-major problem (computed as C^T, bias then broadcast along the other dimension)."""
+    r = H.rng(17)
+    B_, M, N, K = 3, 2048, 2304, 40
+    a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+    w = r.integers(-3, 4, (K, N)).astype(np.float32)
+    a_st, w_st = H.encode(a, dt), H.encode(w, dt)
+    at = srt.Tensor(a_st)
+    w3 = srt.Tensor(np.broadcast_to(w_st, (B_, K, N)).copy())
+    out = srt.Tensor(shape=[B_, M, N], dtype=a_st.dtype)
+    assert query_kernel(at, False, w3, False, out) == "mfma_256x256"
+    got = srt.matmul(at, w3).array()
+    exact = H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), dt)
+    assert np.array_equal(got.view(np.uint16), exact.view(np.uint16))
+    # broadcast weight: same storage for every batch (batch stride 0), built as a view descriptor by hand
+    q = srt.current_queue()
+    wt = srt.Tensor(w_st)
+    ad, k1 = at.descriptor()
+    bd, k2 = native.make_descriptor(native.REAL16F if dt == H.F16 else native.REAL16BF, (B_, K, N), (0, N, 1), native.ORDER_ROW)
+    od, k3 = out.descriptor()
+    native.check(native.lib().srtMatmul(at.device_read(q), ctypes.byref(ad), 0, wt.device_read(q), ctypes.byref(bd), 0,
+                                        out.device_read_write(q), ctypes.byref(od), q.stream))
+    assert np.array_equal(out.array().view(np.uint16), exact.view(np.uint16))
+    # column-major 2-D problem with bias: result order follows lhs.order; bias still runs along N
+    M2, N2, K2 = 3584, 3840, 48
+    x = r.integers(-3, 4, (M2, K2)).astype(np.float32)
+    w2 = r.integers(-3, 4, (K2, N2)).astype(np.float32)
+    b2 = r.integers(-3, 4, N2).astype(np.float32)
+    xc, wc = srt.Tensor(H.encode(x, dt), order=srt.Order.col), srt.Tensor(H.encode(w2, dt), order=srt.Order.col)
+    yc = srt.matmul(xc, wc, bias=srt.Tensor(H.encode(b2, dt)))
+    assert yc.order == srt.Order.col and query_kernel(xc, False, wc, False, yc) == "mfma_256x256"
+    want = H.encode((x.astype(np.int64) @ w2.astype(np.int64) + b2.astype(np.int64)[None, :]).astype(np.float32), dt)
+    assert np.array_equal(yc.array().view(np.uint16), want.view(np.uint16))
+    # and relu on top (bias per row after the transposition inside the library)
+    layer = srt.Dense(wc, srt.Tensor(H.encode(b2, dt)), srt.ActivationType.relu)
+    assert np.array_equal(layer(xc).array().view(np.uint16), H.encode(np.maximum(H.decode(want), 0), dt).view(np.uint16))
+
+
 def test_ring_kernel_nan_and_inf_encode_like_the_reference():
     """A NaN anywhere in a tile switches the wave to the exact encoder: NaN -> 0x7FFF, inf stays inf."""
     M = N = 3584
