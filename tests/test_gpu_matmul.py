@@ -174,7 +174,7 @@ def test_random_odd_shapes_vs_oracle_and_fp64(dt):
             assert np.all(np.abs(H.decode(got).astype(np.float64) - want) <= tol)
 
 
-# ---- BASELINE configs at full size ------------------------------------------------------------------
+# ---- the benchmark configurations at full size --------------------------------------------------
 def test_cfg1_f32_512_vs_oracle_and_fp64():
     r = H.rng(0)
     a = r.uniform(-1, 1, (512, 512)).astype(np.float32)
