@@ -300,6 +300,33 @@ def report_other_configs(srt, q, a_st, b_st, n, args):
     a1.device_read(q), b1.device_read(q), c1.device_read_write(q)
     line("cfg1 fp32 512^3", timed(prepared(a1, False, b1, False, c1), steps=200, warmup=20),
          2.0 * 512 ** 3, 3 * 512 * 512 * 4, "f32")
+    del a1, b1, c1, a2, b2, c2
+
+    # the neighbours of the Dense layer at its shape (bandwidth-bound: bytes = what each must move once)
+    def bw_line(name, ms, nbytes):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        print(f"[bench] {name}: {ms * 1e3:.1f} us  {gbs:.0f} GB/s algorithmic ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM "
+              f"peak)", file=sys.stderr, flush=True)
+
+    m_, n_ = 4096, 11008
+    g = rng(5)
+    e = m_ * n_ * 2
+    ys = [srt.Tensor(bf16_encode(np.maximum(g.standard_normal((m_, n_), dtype=np.float32), 0))) for _ in range(2)]
+    dys = [srt.Tensor(bf16_encode(g.standard_normal((m_, n_), dtype=np.float32))) for _ in range(2)]
+    outs = [srt.Tensor(shape=[m_, n_], dtype=np.uint16) for _ in range(2)]
+    db = srt.Tensor(shape=[n_], dtype=np.uint16)
+    # two buffer sets in rotation: 3 x 90 MB per call would otherwise partly live in the last-level cache
+    bw_line("Dense backward epilogue bf16 4096x11008: dz = dy*relu'(y), dbias (fused)",
+            timed(lambda i: q.activation_backward(ys[i % 2], dys[i % 2], srt.ActivationType.relu, 0.0, outs[i % 2], db),
+                  steps=40, warmup=6), 3 * e + n_ * 2)
+    bw_line("add bf16 4096x11008 (dense, tensor + tensor)",
+            timed(lambda i: q.add(ys[i % 2], dys[i % 2], outs[i % 2]), steps=40, warmup=6), 3 * e)
+    bias_row = srt.Tensor.repeating(bias, (m_, n_))
+    bw_line("add bf16 4096x11008 + bias[11008] (stride-0 broadcast)",
+            timed(lambda i: q.add(ys[i % 2], bias_row, outs[i % 2]), steps=40, warmup=6), 2 * e + n_ * 2)
+    bw_line("tanh bf16 4096x11008", timed(lambda i: q.tanh(ys[i % 2], outs[i % 2]), steps=40, warmup=6), 2 * e)
+    f32out = srt.Tensor(shape=[m_, n_], dtype=np.float32)
+    bw_line("cast bf16 -> fp32 4096x11008", timed(lambda i: q.copy(ys[i % 2], f32out), steps=40, warmup=6), e + 2 * e)
 
 
 if __name__ == "__main__":

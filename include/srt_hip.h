@@ -216,6 +216,86 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
                                const srtTensorDescriptor* oDesc, const void* a, const void* b,
                                const void* out, char* name, size_t nameCapacity);
 
+/* ---- backward of the Dense epilogue ------------------------------------------------------------
+ * dx = dy * activation'(y) and, when dbias != NULL, dbias[n] = sum over rows of dx[:, n], in one
+ * pass over y and dy.  y is the OUTPUT of the forward activation: the derivative is written in
+ * terms of it (sigmoid y(1-y), tanh 1-y^2, relu y>0, clippedRelu 0<y<coef, elu y>0 ? 1 : y+coef,
+ * identity 1), so the pre-activation need not be kept.
+ *
+ * Fills the role of CudaActivation.backward (cudnnActivationBackward(y, dy, x) -> dx,
+ * Sources/SwiftRTCore/platform/cuda/layers/CudaActivation.swift:101-127) and supplies the bias
+ * term of the pullbacks the reference leaves as fatalError() (_vjpMatmul...bias,
+ * Sources/SwiftRTCore/differentiable/MathDerivatives.swift:520-554).  The remaining two products of
+ * the backward pass are srtMatmul calls with transpose flags (matmulGradients,
+ * MathDerivatives.swift:460-482).
+ * y, dy, dx: rank 2, [M, N], one element type (32F, 16F, 16BF), any strides; dbias: rank 1, N
+ * elements.  Sums are fp32 in a fixed order (results do not vary from run to run).
+ * May allocate a stream-ordered workspace of at most about 4096 x 64 x 16 bytes from the library's
+ * allocator.  srtErrorNotSupported for other ranks or element types. */
+srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yDesc,
+                                    const void* dy, const srtTensorDescriptor* dyDesc,
+                                    srtActivation activation, double coef,
+                                    void* dx, const srtTensorDescriptor* dxDesc,
+                                    void* dbias, const srtTensorDescriptor* dbiasDesc, srtStream stream);
+
+/* ---- element-wise neighbours of the path ---------------------------------------------------------
+ * Same names, argument order and conventions as the reference's native module
+ * (Modules/SwiftRTCuda/math_api.h: srtAdd :75-100, srtDiv :138-148, srtExp :166-170, srtMul
+ * :222-233, srtNeg :268-272, srtSigmoid :285-289, srtSub :315-332, srtTanh :338-342;
+ * compare_api.h: srtMin :139-165, srtMax :170-181; copy_api.h: srtCopy :27-38; fill_api.h:
+ * srtFillFlat :27-33), called from CudaQueue exactly as there
+ * (Sources/SwiftRTCore/platform/cuda/functions/CudaMath.swift:93-150).
+ *
+ * Strided forms: all tensors the same rank and shape; an input broadcasts along a dimension by
+ * giving it stride 0 there (Tensor(repeating:to:)); `out` may be any non-aliasing strided view.
+ * TE forms: `element` points to ONE host-side element of the tensors' type, read during the call.
+ * Flat forms: dense buffers of `count` elements.
+ * Element types 32F, 16F, 16BF (srtCopy / srtCopyFlat also convert between any two of them,
+ * rounding to nearest even); arithmetic is fp32 with one rounding to the element type, i.e. the
+ * reference's CPU definitions evaluated in E.Value (CpuMath.swift:646-662, :1189-1256,
+ * :1369-1377; max is `a >= b ? a : b`, min `a <= b ? a : b`).
+ * Any other element type, or a layout that does not collapse to 4 dimensions: srtErrorNotSupported
+ * (caller falls back to the CPU, the reference's convention for unsupported combinations,
+ * Modules/SwiftRTCuda/op2.h:276-289). */
+srtStatus srtAdd(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtAddTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
+                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtAddFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+srtStatus srtSub(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtSubTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
+                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMul(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMulTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
+                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtDiv(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtDivTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
+                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMax(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMaxTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
+                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMin(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMinTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
+                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtNeg(const void* a, const srtTensorDescriptor* aDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtExp(const void* a, const srtTensorDescriptor* aDesc,
+                 void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtSigmoid(const void* a, const srtTensorDescriptor* aDesc,
+                     void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtTanh(const void* a, const srtTensorDescriptor* aDesc,
+                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtCopy(const void* a, const srtTensorDescriptor* aDesc,
+                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtCopyFlat(srtDataType atype, const void* a, srtDataType otype, void* out, size_t count,
+                      srtStream stream);
+srtStatus srtFillFlat(srtDataType type, void* out, const void* element, size_t count, srtStream stream);
+
 /* ---- test helper ------------------------------------------------------------------------- */
 /* Replaces srtDelayStream, Modules/SwiftRTCuda/utilities_api.h:28: occupies `stream` for about
  * `seconds` (bounded spin on the device clock; at most 10 s). */

@@ -182,3 +182,81 @@ def gemm_f64_rows(lhs, rhs, rows=None, transpose_lhs=False, transpose_rhs=False)
     if rc != 0:
         raise ValueError(f"gemm_f64_rows failed ({rc})")
     return out
+
+
+# ---- element-wise neighbours of the path (numpy restatement) ------------------------------------
+# The reference's CPU definitions, evaluated in E.Value (= float for Float and BFloat16; for
+# Float16 the native half arithmetic of +, -, *, / equals the float operation rounded once, since
+# binary32 carries more than twice binary16's precision) and stored with one rounding:
+#   add/sub/mul/div  mapOp(lhs, rhs, &out, op)        CpuMath.swift:646-662, :1235-1256
+#   max / min        `a >= b ? a : b`, `a <= b ? a : b`   CpuMath.swift:1189-1232
+#   neg, exp         CpuMath.swift:1286-1292, :943-949
+#   sigmoid          `1 / (1 + exp(-x))`               CpuMath.swift:1369-1377
+#   tanh             libm tanh                          CpuMath.swift (cpu_tanh)
+# numpy's float32 +, -, *, / are the correctly rounded IEEE operations, i.e. exactly what the C
+# restatement of these one-line maps would compute; exp/tanh come from the host libm.
+# Pinned by: closed forms on exactly representable inputs, the LSTM fixtures (sigmoid, tanh, mul,
+# add chained, tests/golden/reference_kats.json), numpy.float16 as an independent library oracle
+# for the half results.  Broadcasting follows numpy (stride-0 views), which is what
+# Tensor(repeating:to:) passes to the kernels.
+def _max(a, b):
+    return np.where(a >= b, a, b)
+
+
+def _min(a, b):
+    return np.where(a <= b, a, b)
+
+
+ELEMENTWISE = {
+    "add": lambda a, b: a + b,
+    "sub": lambda a, b: a - b,
+    "mul": lambda a, b: a * b,
+    "div": lambda a, b: a / b,
+    "max": _max,
+    "min": _min,
+    "neg": lambda a, b: -a,
+    "exp": lambda a, b: np.exp(a),
+    "sigmoid": lambda a, b: np.float32(1) / (np.float32(1) + np.exp(-a)),
+    "tanh": lambda a, b: np.tanh(a),
+    "copy": lambda a, b: a,
+}
+
+
+def elementwise(op, a, b=None, out_dtype=None):
+    """a, b: storage arrays (b may be None, a storage array broadcastable to a, or one storage
+    element); returns the storage array of the result (same format as a unless out_dtype)."""
+    dt = dtype_id(a)
+    fa = decode(a)
+    fb = None
+    if b is not None:
+        fb = np.broadcast_to(decode(np.asarray(b)), fa.shape)
+    with np.errstate(all="ignore"):
+        r = ELEMENTWISE[op](fa, fb).astype(np.float32)
+    return encode(r, dt if out_dtype is None else out_dtype)
+
+
+def activation_slope(kind, y, coef=0.0):
+    """Derivative of the activation written through its output y (what cudnnActivationBackward
+    evaluates for these modes): float32 in, float32 out."""
+    y = np.asarray(y, dtype=np.float32)
+    one, zero = np.float32(1), np.float32(0)
+    if kind == SIGMOID:
+        return y * (one - y)
+    if kind == RELU:
+        return np.where(y > 0, one, zero)
+    if kind == TANH:
+        return one - y * y
+    if kind == CLIPPED_RELU:
+        return np.where((y > 0) & (y < np.float32(coef)), one, zero)
+    if kind == ELU:
+        return np.where(y > 0, one, y + np.float32(coef))
+    return np.ones_like(y)
+
+
+def activation_backward_bias(y, dy, kind, coef=0.0):
+    """dx = dy * act'(y) rounded once to the storage type; dbias = column sums of the UNROUNDED
+    products, returned as float64 (the grading value) -- the kernel sums them in fp32 in its own
+    order and rounds once, so it is compared with a tolerance, or exactly on integer data."""
+    dt = dtype_id(y)
+    g = decode(dy) * activation_slope(kind, decode(y), coef)
+    return encode(g, dt), g.astype(np.float64).sum(axis=0)

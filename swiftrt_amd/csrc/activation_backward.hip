@@ -1,0 +1,245 @@
+// Backward of the Dense epilogue: the activation gradient fused with the bias gradient.
+//
+//   dx[m, n]  = dy[m, n] * act'(y[m, n])          (act' written in terms of the OUTPUT y, as
+//                                                  cudnnActivationBackward uses it for these modes)
+//   dbias[n]  = sum_m dx[m, n]                     (fp32 sums, rounded once)
+//
+// The two GEMMs of the backward pass (dX = dZ . W^T, dW = X^T . dZ) are ordinary srtMatmul calls
+// with transpose flags; this kernel produces their common operand dZ in ONE pass over y and dy
+// and gets the bias gradient for free from the values it already holds.  Bandwidth-bound:
+// algorithmic bytes = 3 M N elements (read y, dy; write dx) + N.
+//
+//   grid    x: strips of 64 lanes x V columns, y: row chunks; 4 waves per workgroup, wave w takes
+//           rows w, w + 4, ... of its chunk, so every wave instruction moves one 1 KiB row segment
+//   sums    8 (V) fp32 column sums per lane in registers, waves combined through LDS, one fp32
+//           partial row per chunk in a workspace; a second tiny kernel adds the chunks in a fixed
+//           order (deterministic, no atomics)
+//   V = 1   same structure for layouts the vector path excludes (any strides)
+#include "gemm_common.h"
+#include "status.h"
+
+namespace srt {
+namespace {
+
+// derivative of the activation expressed through its output
+__device__ __forceinline__ float activation_slope(int activation, float coef, float y) {
+  switch (activation) {
+    case srtActivationSigmoid: return y * (1.0f - y);
+    case srtActivationRelu: return y > 0.0f ? 1.0f : 0.0f;
+    case srtActivationTanh: return 1.0f - y * y;
+    case srtActivationClippedRelu: return (y > 0.0f && y < coef) ? 1.0f : 0.0f;
+    case srtActivationElu: return y > 0.0f ? 1.0f : y + coef;
+    default: return 1.0f;
+  }
+}
+
+struct BackwardProblem {
+  int M, N;
+  const void* y;
+  const void* dy;
+  void* dx;
+  long long sym, syn, sdm, sdn, sxm, sxn;   // element strides of y, dy, dx
+  float* partial;                            // [chunks][N] fp32, null when no bias gradient is wanted
+  int rows_per_chunk;
+  int activation;
+  float coef;
+};
+
+template <typename T, int V>
+struct alignas(V * sizeof(typename T::storage)) Pack {
+  typename T::storage v[V];
+};
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void activation_backward_kernel(BackwardProblem p) {
+  using S = typename T::storage;
+  __shared__ float red[4][64 * V];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * 64 + lane) * V;
+  const int m_begin = blockIdx.y * p.rows_per_chunk;
+  const int m_end = min(p.M, m_begin + p.rows_per_chunk);
+  const S* y = (const S*)p.y;
+  const S* dy = (const S*)p.dy;
+  S* dx = (S*)p.dx;
+  float sum[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) sum[i] = 0.0f;
+  if (n0 < p.N) {
+    // two rows per trip (both rows' loads are issued before either is used)
+    for (int m = m_begin + wave; m < m_end; m += 8) {
+      const int m2 = m + 4;
+      const bool second = m2 < m_end;
+      float fy[2][V], fd[2][V];
+      if (V > 1) {
+        const Pack<T, V> py0 = *reinterpret_cast<const Pack<T, V>*>(y + (long long)m * p.sym + n0);
+        const Pack<T, V> pd0 = *reinterpret_cast<const Pack<T, V>*>(dy + (long long)m * p.sdm + n0);
+        Pack<T, V> py1 = py0, pd1 = pd0;
+        if (second) {
+          py1 = *reinterpret_cast<const Pack<T, V>*>(y + (long long)m2 * p.sym + n0);
+          pd1 = *reinterpret_cast<const Pack<T, V>*>(dy + (long long)m2 * p.sdm + n0);
+        }
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          fy[0][i] = T::to_float(py0.v[i]); fd[0][i] = T::to_float(pd0.v[i]);
+          fy[1][i] = T::to_float(py1.v[i]); fd[1][i] = T::to_float(pd1.v[i]);
+        }
+      } else {
+        fy[0][0] = T::to_float(y[(long long)m * p.sym + (long long)n0 * p.syn]);
+        fd[0][0] = T::to_float(dy[(long long)m * p.sdm + (long long)n0 * p.sdn]);
+        fy[1][0] = fy[0][0]; fd[1][0] = fd[0][0];
+        if (second) {
+          fy[1][0] = T::to_float(y[(long long)m2 * p.sym + (long long)n0 * p.syn]);
+          fd[1][0] = T::to_float(dy[(long long)m2 * p.sdm + (long long)n0 * p.sdn]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        if (r == 1 && !second) break;
+        const int row = r ? m2 : m;
+        Pack<T, V> out;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          float g = fd[r][i] * activation_slope(p.activation, p.coef, fy[r][i]);
+          // keep the product as an fp32 value: without this the compiler merges the multiply and
+          // the conversion to half into one mixed-precision instruction that rounds the exact
+          // product once, which differs from "fp32 product, then round" on ties
+          asm volatile("" : "+v"(g));
+          out.v[i] = T::from_float(g);
+          sum[i] += g;
+        }
+        if (V > 1) *reinterpret_cast<Pack<T, V>*>(dx + (long long)row * p.sxm + n0) = out;
+        else dx[(long long)row * p.sxm + (long long)n0 * p.sxn] = out.v[0];
+      }
+    }
+  }
+  if (p.partial == nullptr) return;
+#pragma unroll
+  for (int i = 0; i < V; ++i) red[wave][lane * V + i] = sum[i];
+  __syncthreads();
+  if (wave == 0 && n0 < p.N) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const int c = lane * V + i;
+      p.partial[(long long)blockIdx.y * p.N + n0 + i] = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
+    }
+  }
+}
+
+// Adds the chunks' partial rows: 64 columns per workgroup, the four waves take every fourth chunk
+// (four independent loads in flight per lane) and meet in LDS.  The order of the additions is fixed.
+template <typename T>
+__global__ __launch_bounds__(256) void bias_gradient_finish_kernel(const float* partial, int chunks, int N,
+                                                                   typename T::storage* dbias, long long stride) {
+  __shared__ float red[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * 64 + lane;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  if (n < N) {
+    int c = wave;
+    for (; c + 12 < chunks; c += 16) {
+      s0 += partial[(long long)c * N + n];
+      s1 += partial[(long long)(c + 4) * N + n];
+      s2 += partial[(long long)(c + 8) * N + n];
+      s3 += partial[(long long)(c + 12) * N + n];
+    }
+    for (; c < chunks; c += 4) s0 += partial[(long long)c * N + n];
+  }
+  red[wave][lane] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (wave == 0 && n < N)
+    dbias[(long long)n * stride] = T::from_float((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]));
+}
+
+template <typename T>
+srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_t stream) {
+  constexpr int VEC = 16 / sizeof(typename T::storage);
+  const size_t es = sizeof(typename T::storage);
+  auto vec_ok = [&](const void* ptr, long long sm, long long sn) {
+    return sn == 1 && sm % VEC == 0 && (uintptr_t)ptr % (VEC * es) == 0;
+  };
+  const bool vec = p.N % VEC == 0 && vec_ok(p.y, p.sym, p.syn) && vec_ok(p.dy, p.sdm, p.sdn) && vec_ok(p.dx, p.sxm, p.sxn);
+  const int V = vec ? VEC : 1;
+  const int strips = (p.N + 64 * V - 1) / (64 * V);
+  // enough workgroups to keep every memory channel busy, but at least 16 rows per chunk
+  int chunks = (4096 + strips - 1) / strips;
+  const int max_chunks = (p.M + 15) / 16;
+  if (chunks > max_chunks) chunks = max_chunks;
+  if (chunks > 65535) chunks = 65535;
+  if (chunks < 1) chunks = 1;
+  p.rows_per_chunk = (p.M + chunks - 1) / chunks;
+  chunks = (p.M + p.rows_per_chunk - 1) / p.rows_per_chunk;
+
+  void* workspace = nullptr;
+  if (dbias) {
+    srtStatus s = srtDeviceAllocate(&workspace, (size_t)chunks * p.N * sizeof(float), reinterpret_cast<srtStream>(stream));
+    if (s != srtSuccess) return s;
+  }
+  p.partial = (float*)workspace;
+  const dim3 grid(strips, chunks);
+  if (vec) hipLaunchKernelGGL((activation_backward_kernel<T, VEC>), grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((activation_backward_kernel<T, 1>), grid, dim3(256), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && dbias) {
+    hipLaunchKernelGGL((bias_gradient_finish_kernel<T>), dim3((p.N + 63) / 64), dim3(256), 0, stream,
+                       (const float*)workspace, chunks, p.N, (typename T::storage*)dbias, dbias_stride);
+    e = hipGetLastError();
+  }
+  // stream-ordered: the block becomes reusable for other streams only after the work queued so
+  // far on `stream` has finished
+  if (workspace) (void)srtDeviceFree(workspace);
+  return from_hip(e);
+}
+
+}  // namespace
+}  // namespace srt
+
+extern "C" srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yDesc, const void* dy,
+                                               const srtTensorDescriptor* dyDesc, srtActivation activation,
+                                               double coef, void* dx, const srtTensorDescriptor* dxDesc,
+                                               void* dbias, const srtTensorDescriptor* dbiasDesc,
+                                               srtStream stream) {
+  auto ok = [](const srtTensorDescriptor* d) { return d && d->shape && d->strides; };
+  if (!ok(yDesc) || !ok(dyDesc) || !ok(dxDesc)) return srtErrorInvalidValue;
+  if (dxDesc->rank != 2) return srtErrorNotSupported;
+  if (yDesc->rank != 2 || dyDesc->rank != 2) return srtErrorInvalidValue;
+  const srtDataType t = dxDesc->type;
+  if (t != srtReal32F && t != srtReal16F && t != srtReal16BF) return srtErrorNotSupported;
+  if (yDesc->type != t || dyDesc->type != t) return srtErrorNotSupported;
+  if ((unsigned)activation > (unsigned)srtActivationIdentity) return srtErrorInvalidValue;
+  const size_t M = dxDesc->shape[0], N = dxDesc->shape[1];
+  if (yDesc->shape[0] != M || yDesc->shape[1] != N || dyDesc->shape[0] != M || dyDesc->shape[1] != N)
+    return srtErrorInvalidValue;
+  long long dbias_stride = 0;
+  if (dbias) {
+    if (!ok(dbiasDesc)) return srtErrorInvalidValue;
+    if (dbiasDesc->type != t) return srtErrorNotSupported;
+    if (dbiasDesc->rank != 1 || dbiasDesc->shape[0] != N) return srtErrorInvalidValue;
+    dbias_stride = (long long)dbiasDesc->strides[0];
+  }
+  if (M > 0x7fffffffu || N > 0x7fffffffu) return srtErrorNotSupported;
+  if (N == 0) return srtSuccess;
+  if (M == 0) {
+    // an empty sum: the bias gradient is zero
+    if (dbias) {
+      const uint32_t zero = 0;
+      if (dbias_stride != 1) return srtErrorNotSupported;
+      return srtFillFlat(t, dbias, &zero, N, stream);
+    }
+    return srtSuccess;
+  }
+  if (!y || !dy || !dx) return srtErrorInvalidValue;
+  srt::BackwardProblem p{};
+  p.M = (int)M; p.N = (int)N;
+  p.y = y; p.dy = dy; p.dx = dx;
+  p.sym = (long long)yDesc->strides[0]; p.syn = (long long)yDesc->strides[1];
+  p.sdm = (long long)dyDesc->strides[0]; p.sdn = (long long)dyDesc->strides[1];
+  p.sxm = (long long)dxDesc->strides[0]; p.sxn = (long long)dxDesc->strides[1];
+  p.activation = (int)activation;
+  p.coef = (float)coef;
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  switch (t) {
+    case srtReal32F: return srt::run<srt::F32>(p, dbias, dbias_stride, hs);
+    case srtReal16F: return srt::run<srt::F16>(p, dbias, dbias_stride, hs);
+    default: return srt::run<srt::BF16>(p, dbias, dbias_stride, hs);
+  }
+}

@@ -258,4 +258,73 @@ struct Dense {
   }
 };
 
+// ---- element-wise neighbours (role of CudaQueue.add / mul / max / sigmoid / tanh ...,
+// platform/cuda/functions/CudaMath.swift:93-150) -----------------------------------------------------
+using BinaryFn = srtStatus (*)(const void*, const srtTensorDescriptor*, const void*, const srtTensorDescriptor*,
+                               void*, const srtTensorDescriptor*, srtStream);
+using ElementFn = srtStatus (*)(const void*, const srtTensorDescriptor*, const void*, void*,
+                                const srtTensorDescriptor*, srtStream);
+using UnaryFn = srtStatus (*)(const void*, const srtTensorDescriptor*, void*, const srtTensorDescriptor*, srtStream);
+
+template <typename E>
+Tensor<E> binary(HipQueue& q, BinaryFn fn, const Tensor<E>& lhs, const Tensor<E>& rhs, const char* what) {
+  if (lhs.shape() != rhs.shape()) throw std::invalid_argument("element-wise operands must have one shape");
+  Tensor<E> out(lhs.shape(), lhs.order());
+  const void* a = lhs.device_read(q);
+  const void* b = rhs.device_read(q);
+  void* o = out.device_read_write(q);
+  srtTensorDescriptor ad = lhs.descriptor(), bd = rhs.descriptor(), od = out.descriptor();
+  check(fn(a, &ad, b, &bd, o, &od, q.stream()), what);
+  return out;
+}
+
+template <typename E>
+Tensor<E> binary_element(HipQueue& q, ElementFn fn, const Tensor<E>& lhs, E element, const char* what) {
+  Tensor<E> out(lhs.shape(), lhs.order());
+  const void* a = lhs.device_read(q);
+  void* o = out.device_read_write(q);
+  srtTensorDescriptor ad = lhs.descriptor(), od = out.descriptor();
+  check(fn(a, &ad, &element, o, &od, q.stream()), what);
+  return out;
+}
+
+template <typename E>
+Tensor<E> unary(HipQueue& q, UnaryFn fn, const Tensor<E>& x, const char* what) {
+  Tensor<E> out(x.shape(), x.order());
+  const void* a = x.device_read(q);
+  void* o = out.device_read_write(q);
+  srtTensorDescriptor ad = x.descriptor(), od = out.descriptor();
+  check(fn(a, &ad, o, &od, q.stream()), what);
+  return out;
+}
+
+template <typename E> Tensor<E> add(HipQueue& q, const Tensor<E>& a, const Tensor<E>& b) { return binary(q, srtAdd, a, b, "srtAdd"); }
+template <typename E> Tensor<E> mul(HipQueue& q, const Tensor<E>& a, const Tensor<E>& b) { return binary(q, srtMul, a, b, "srtMul"); }
+template <typename E> Tensor<E> add(HipQueue& q, const Tensor<E>& a, E e) { return binary_element(q, srtAddTE, a, e, "srtAddTE"); }
+template <typename E> Tensor<E> relu(HipQueue& q, const Tensor<E>& a) { return binary_element(q, srtMaxTE, a, E{}, "srtMaxTE"); }
+template <typename E> Tensor<E> sigmoid(HipQueue& q, const Tensor<E>& a) { return unary(q, srtSigmoid, a, "srtSigmoid"); }
+template <typename E> Tensor<E> tanh(HipQueue& q, const Tensor<E>& a) { return unary(q, srtTanh, a, "srtTanh"); }
+
+// ---- backward of Dense: (dx, dweight, dbias) for y = layer(x) and the gradient of y ------------------
+// dz and dbias come from one fused pass (role of CudaActivation.backward,
+// platform/cuda/layers/CudaActivation.swift:101-127, plus the bias pullback the reference leaves as
+// fatalError, MathDerivatives.swift:520-554); dx = dz W^T, dW = x^T dz (matmulGradients :460-482).
+template <typename E>
+struct DenseGradients { Tensor<E> dx, dweight, dbias; };
+
+template <typename E>
+DenseGradients<E> dense_backward(HipQueue& q, const Dense<E>& layer, const Tensor<E>& x, const Tensor<E>& y,
+                                 const Tensor<E>& out_grad) {
+  Tensor<E> dz(y.shape(), y.order()), dbias({y.shape()[1]});
+  const void* yp = y.device_read(q);
+  const void* gp = out_grad.device_read(q);
+  void* zp = dz.device_read_write(q);
+  void* bp = dbias.device_read_write(q);
+  srtTensorDescriptor yd = y.descriptor(), gd = out_grad.descriptor(), zd = dz.descriptor(), bd = dbias.descriptor();
+  check(srtActivationBackwardBias(yp, &yd, gp, &gd, (srtActivation)layer.activation, layer.coef, zp, &zd, bp, &bd,
+                                  q.stream()),
+        "srtActivationBackwardBias");
+  return DenseGradients<E>{matmul(q, dz, false, layer.weight, true), matmul(q, x, true, dz, false), dbias};
+}
+
 }  // namespace srt_host

@@ -89,7 +89,18 @@ SIGNATURES = {
     "srtMatmulQueryKernel": (_i32, [_descp, _i32, _descp, _i32, _descp, _vp, _vp, _vp,
                                      ctypes.c_char_p, ctypes.c_size_t]),
     "srtDelayStream": (_i32, [ctypes.c_double, _vp]),
+    "srtActivationBackwardBias": (_i32, [_vp, _descp, _vp, _descp, _i32, ctypes.c_double, _vp, _descp,
+                                          _vp, _descp, _vp]),
+    "srtAddFlat": (_i32, [_i32, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
+    "srtCopyFlat": (_i32, [_i32, _vp, _i32, _vp, ctypes.c_size_t, _vp]),
+    "srtFillFlat": (_i32, [_i32, _vp, _vp, ctypes.c_size_t, _vp]),
 }
+# element-wise neighbours: tensor-tensor, tensor-element and unary forms share three signatures
+for _name in ("Add", "Sub", "Mul", "Div", "Max", "Min"):
+    SIGNATURES["srt" + _name] = (_i32, [_vp, _descp, _vp, _descp, _vp, _descp, _vp])
+    SIGNATURES["srt" + _name + "TE"] = (_i32, [_vp, _descp, _vp, _vp, _descp, _vp])
+for _name in ("Neg", "Exp", "Sigmoid", "Tanh", "Copy"):
+    SIGNATURES["srt" + _name] = (_i32, [_vp, _descp, _vp, _descp, _vp])
 
 _lib = None
 

@@ -165,6 +165,84 @@ class HipQueue:
         del ka, kb, ko
         check(st, "srtMatmul")
 
+    # -- element-wise neighbours of the path ----------------------------------------------------
+    def _elementwise(self, name, lhs, rhs, out):
+        """Role of CudaQueue.add / mul / max ... (platform/cuda/functions/CudaMath.swift:93-150):
+        tensor-tensor form when `rhs` is a tensor, tensor-element form when it is a scalar, unary
+        form when it is None.  Inputs must already have the shape of `out` (a broadcast operand is
+        a stride-0 view, Tensor.repeating)."""
+        import numpy as np
+        self.select()
+        L = native.lib()
+        a_ptr = lhs.device_read(self)
+        ad, ka = lhs.descriptor()
+        if rhs is None:
+            o_ptr = out.device_read_write(self)
+            od, ko = out.descriptor()
+            st = getattr(L, "srt" + name)(a_ptr, ctypes.byref(ad), o_ptr, ctypes.byref(od), self.stream)
+        elif hasattr(rhs, "device_read"):
+            b_ptr = rhs.device_read(self)
+            o_ptr = out.device_read_write(self)
+            bd, kb = rhs.descriptor()
+            od, ko = out.descriptor()
+            st = getattr(L, "srt" + name)(a_ptr, ctypes.byref(ad), b_ptr, ctypes.byref(bd), o_ptr, ctypes.byref(od),
+                                          self.stream)
+            del kb
+        else:
+            element = lhs.element_storage(rhs)          # one element in the tensor's storage format
+            o_ptr = out.device_read_write(self)
+            od, ko = out.descriptor()
+            st = getattr(L, "srt" + name + "TE")(a_ptr, ctypes.byref(ad), ctypes.c_void_p(element.ctypes.data),
+                                                 o_ptr, ctypes.byref(od), self.stream)
+        del ka, ko
+        check(st, "srt" + name)
+
+    def add(self, lhs, rhs, out): self._elementwise("Add", lhs, rhs, out)
+    def subtract(self, lhs, rhs, out): self._elementwise("Sub", lhs, rhs, out)
+    def mul(self, lhs, rhs, out): self._elementwise("Mul", lhs, rhs, out)
+    def div(self, lhs, rhs, out): self._elementwise("Div", lhs, rhs, out)
+    def max(self, lhs, rhs, out): self._elementwise("Max", lhs, rhs, out)
+    def min(self, lhs, rhs, out): self._elementwise("Min", lhs, rhs, out)
+    def neg(self, x, out): self._elementwise("Neg", x, None, out)
+    def exp(self, x, out): self._elementwise("Exp", x, None, out)
+    def sigmoid(self, x, out): self._elementwise("Sigmoid", x, None, out)
+    def tanh(self, x, out): self._elementwise("Tanh", x, None, out)
+
+    def copy(self, x, out):
+        """Role of CudaQueue.copy / cast: element types may differ (srtCopy converts)."""
+        self._elementwise("Copy", x, None, out)
+
+    def fill(self, out, value):
+        """Role of CudaQueue.fill(_:with:) (platform/cuda/functions/CudaFill.swift): dense `out`."""
+        self.select()
+        element = out.element_storage(value)
+        if not out.is_contiguous:
+            raise native.NotSupportedError(native.ERROR_NOT_SUPPORTED, "fill of a strided view")
+        o_ptr = out.device_read_write(self)
+        check(native.lib().srtFillFlat(out.type_id, o_ptr, ctypes.c_void_p(element.ctypes.data), out.count,
+                                       self.stream), "srtFillFlat")
+
+    def activation_backward(self, y, dy, activation, coef, dx, dbias=None):
+        """Role of CudaActivation.backward (platform/cuda/layers/CudaActivation.swift:101-127) fused
+        with the bias gradient: dx = dy * act'(y), dbias = column sums of dx."""
+        self.select()
+        y_ptr, dy_ptr = y.device_read(self), dy.device_read(self)
+        dx_ptr = dx.device_read_write(self)
+        yd, k1 = y.descriptor()
+        dyd, k2 = dy.descriptor()
+        dxd, k3 = dx.descriptor()
+        if dbias is not None:
+            db_ptr = dbias.device_read_write(self)
+            dbd, k4 = dbias.descriptor()
+            dbd_ref = ctypes.byref(dbd)
+        else:
+            db_ptr, dbd_ref, k4 = None, None, None
+        st = native.lib().srtActivationBackwardBias(y_ptr, ctypes.byref(yd), dy_ptr, ctypes.byref(dyd),
+                                                    int(activation), float(coef), dx_ptr, ctypes.byref(dxd),
+                                                    db_ptr, dbd_ref, self.stream)
+        del k1, k2, k3, k4
+        check(st, "srtActivationBackwardBias")
+
     def __del__(self):
         try:
             if self.stream:

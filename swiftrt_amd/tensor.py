@@ -126,6 +126,66 @@ class Tensor:
     def descriptor(self):
         return native.make_descriptor(_DTYPES[self.dtype], self.shape, self.strides, self.order.value)
 
+    @property
+    def type_id(self):
+        return _DTYPES[self.dtype]
+
+    @property
+    def is_contiguous(self):
+        return tuple(self.strides) == tuple(strides_for(self.shape, self.order))
+
+    def element_storage(self, value):
+        """One scalar in this tensor's storage format (a 1-element array): what
+        `withUnsafePointer(to: element)` hands to the tensor-element entry points."""
+        f = np.array([value], dtype=np.float32)
+        if self.dtype == np.dtype(np.uint16):       # BFloat16: round to nearest even, NaN -> 0x7FFF
+            u = f.view(np.uint32)
+            r = ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+            r[(u & 0x7FFFFFFF) > 0x7F800000] = 0x7FFF
+            return r
+        return f.astype(self.dtype)
+
+    @staticmethod
+    def repeating(other, shape):
+        """Tensor(repeating:to:) (tensor/TensorInit.swift): a zero-copy broadcast view -- `other` is
+        aligned to the trailing dimensions of `shape`, every repeated dimension gets stride 0."""
+        shape = [int(x) for x in shape]
+        lead = len(shape) - other.rank
+        if lead < 0:
+            raise ValueError("cannot repeat to a lower rank")
+        strides = [0] * lead
+        for e, st, target in zip(other.shape, other.strides, shape[lead:]):
+            if e == target:
+                strides.append(st)
+            elif e == 1:
+                strides.append(0)
+            else:
+                raise ValueError("shape is not a repetition of the tensor's shape")
+        return Tensor(shape=shape, order=other.order, _storage=other.storage, _offset=other.offset, _strides=strides)
+
+    # -- operators (operators/Math.swift, AlgebraicField): thin wrappers over the queue functions ----
+    def _binary(self, other, fn_name):
+        out = Tensor(shape=self.shape, dtype=self.dtype, order=self.order)
+        if isinstance(other, Tensor) and other.shape != self.shape:
+            other = Tensor.repeating(other, self.shape)
+        getattr(current_queue(), fn_name)(self, other, out)
+        return out
+
+    def __add__(self, other): return self._binary(other, "add")
+    def __sub__(self, other): return self._binary(other, "subtract")
+    def __mul__(self, other): return self._binary(other, "mul")
+    def __truediv__(self, other): return self._binary(other, "div")
+    __radd__ = __add__
+    __rmul__ = __mul__
+
+    def __rsub__(self, other):          # element - tensor = -(tensor - element)
+        return -(self - other)
+
+    def __neg__(self):
+        out = Tensor(shape=self.shape, dtype=self.dtype, order=self.order)
+        current_queue().neg(self, out)
+        return out
+
     # -- storage migration -------------------------------------------------------------------
     def _ensure_device(self, queue):
         s = self.storage
@@ -213,3 +273,132 @@ class Dense:
         current_queue().matmul(x, False, self.weight, False, result, bias=self.bias,
                                activation=self.activation, coef=self.coef)
         return result
+
+
+# ---- element-wise functions (operators/Math.swift; queue functions in CudaMath.swift) -------------
+def _unary(x, fn_name):
+    out = Tensor(shape=x.shape, dtype=x.dtype, order=x.order)
+    getattr(current_queue(), fn_name)(x, out)
+    return out
+
+
+def sigmoid(x): return _unary(x, "sigmoid")
+def tanh(x): return _unary(x, "tanh")
+def exp(x): return _unary(x, "exp")
+
+
+def maximum(x, other): return x._binary(other, "max")
+def minimum(x, other): return x._binary(other, "min")
+
+
+def relu(x):
+    """max(x, 0) (operators/Math.swift relu): the tensor-element form of max."""
+    return maximum(x, 0.0)
+
+
+def cast(x, dtype):
+    """cast(_:elementsTo:): conversion between Float, Float16 and BFloat16 storage on the device."""
+    out = Tensor(shape=x.shape, dtype=dtype, order=x.order)
+    current_queue().copy(x, out)
+    return out
+
+
+def filled(shape, value, dtype, order=Order.row):
+    out = Tensor(shape=shape, dtype=dtype, order=order)
+    current_queue().fill(out, value)
+    return out
+
+
+def concatenate(a, b, axis):
+    """concatenate(_:_:axis:) of two tensors: two strided device copies into views of the result."""
+    if a.rank != b.rank or a.dtype != b.dtype:
+        raise ValueError("concatenate: rank and element type must agree")
+    shape = list(a.shape)
+    shape[axis] += b.shape[axis]
+    out = Tensor(shape=shape, dtype=a.dtype, order=a.order)
+    lo = [slice(None)] * a.rank
+    hi = [slice(None)] * a.rank
+    lo[axis] = slice(0, a.shape[axis])
+    hi[axis] = slice(a.shape[axis], shape[axis])
+    q = current_queue()
+    q.copy(a, out[tuple(lo)])
+    q.copy(b, out[tuple(hi)])
+    return out
+
+
+# ---- backward of the path ---------------------------------------------------------------------------
+def matmul_gradients(out_grad, lhs, transposed_lhs, rhs, transposed_rhs):
+    """matmulGradients (differentiable/MathDerivatives.swift:460-482): gradients of
+    matmul(lhs, transposed:, rhs, transposed:) as two matmuls with transpose flags, each returned
+    in the layout its operand is STORED in.  The (false, false) case is the reference's; for the
+    transposed cases the reference's table returns some gradients transposed (its shapes only agree
+    for square operands), so the products are written out here:
+        C = A  B   : dA = dC B^T      dB = A^T dC
+        C = A  B^T : dA = dC B        dB = dC^T A
+        C = A^T B  : dA = B dC^T      dB = A dC
+        C = A^T B^T: dA = B^T dC^T    dB = dC^T A^T"""
+    g = out_grad
+    if not transposed_lhs and not transposed_rhs:
+        return matmul(g, rhs, False, True), matmul(lhs, g, True, False)
+    if not transposed_lhs and transposed_rhs:
+        return matmul(g, rhs), matmul(g, lhs, True, False)
+    if transposed_lhs and not transposed_rhs:
+        return matmul(rhs, g, False, True), matmul(lhs, g)
+    return matmul(rhs, g, True, True), matmul(g, lhs, True, True)
+
+
+def dense_backward(layer, x, y, out_grad):
+    """Pullback of Dense.callAsFunction at (x -> y): returns (dx, dweight, dbias).
+    dz = out_grad * act'(y) and dbias = column sums of dz come from ONE fused pass
+    (HipQueue.activation_backward); dx = dz W^T and dW = x^T dz are matmuls with transpose flags
+    (matmulGradients' (false, false) row).  Fills the bias pullbacks the reference leaves as
+    fatalError() (MathDerivatives.swift:520-554)."""
+    dz = Tensor(shape=y.shape, dtype=y.dtype, order=y.order)
+    dbias = Tensor(shape=[y.shape[1]], dtype=y.dtype) if layer.bias is not None else None
+    current_queue().activation_backward(y, out_grad, layer.activation, layer.coef, dz, dbias)
+    dx, dw = matmul_gradients(dz, x, False, layer.weight, False)
+    return dx, dw, dbias
+
+
+# ---- recurrent cells built from the path (SwiftRTLayers/Recurrent.swift) ---------------------------
+class BasicRNNCell:
+    """BasicRNNCell (Recurrent.swift:110-161): state' = tanh(matmul([x, h], W) + b).  `fused`
+    selects one srtMatmulBiasActivation call; otherwise the reference's three queue operations
+    (matmul, add with a broadcast bias, tanh) run unfused on the device."""
+
+    def __init__(self, weight, bias, fused=True):
+        self.weight, self.bias, self.fused = weight, bias, fused
+
+    def __call__(self, x, state):
+        xin = concatenate(x, state, axis=1)
+        if self.fused:
+            out = Tensor(shape=[xin.shape[0], self.weight.shape[1]], dtype=xin.dtype)
+            current_queue().matmul(xin, False, self.weight, False, out, bias=self.bias,
+                                   activation=ActivationType.tanh)
+            return out
+        return tanh(matmul(xin, self.weight) + self.bias)
+
+
+class LSTMCell:
+    """LSTMCell (Recurrent.swift:165-266): gates = matmul([x, h], fusedWeight, bias: fusedBias) cut
+    into input, update, forget, output parts (:176, :190-203); cell' = cell * forget + input *
+    update; hidden' = tanh(cell') * output (:255-266)."""
+
+    def __init__(self, fused_weight, fused_bias):
+        self.fused_weight, self.fused_bias = fused_weight, fused_bias
+        self.hidden_size = fused_weight.shape[1] // 4
+
+    def part(self, i, fused):
+        h = self.hidden_size
+        return fused[:, i * h:(i + 1) * h]
+
+    def __call__(self, x, cell, hidden):
+        gate_input = concatenate(x, hidden, axis=1)
+        fused = matmul(gate_input, self.fused_weight, bias=self.fused_bias)
+        input_gate = sigmoid(self.part(0, fused))
+        update_gate = tanh(self.part(1, fused))
+        forget_gate = sigmoid(self.part(2, fused))
+        output_gate = sigmoid(self.part(3, fused))
+        new_cell = cell * forget_gate + input_gate * update_gate
+        new_hidden = tanh(new_cell) * output_gate
+        return new_cell, new_hidden

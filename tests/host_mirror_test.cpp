@@ -47,6 +47,25 @@ int main() {
   Tensor<float> x({2, 2}, {1, 1, -1, -1});
   EXPECT((layer(q, x).values() == std::vector<float>{3.5f, 0.0f, 0.0f, 3.5f}));
 
+  // its pullback: y = relu(x W + b) = [[3.5, 0], [0, 3.5]], upstream gradient [[1, 2], [3, 4]]
+  //   dz = grad where y > 0 = [[1, 0], [0, 4]]; dbias = [1, 4]; dx = dz W^T; dW = x^T dz
+  auto y = layer(q, x);
+  auto grads = dense_backward(q, layer, x, y, Tensor<float>({2, 2}, {1, 2, 3, 4}));
+  EXPECT((grads.dbias.values() == std::vector<float>{1, 4}));
+  EXPECT((grads.dx.values() == std::vector<float>{1, 2, -4, -8}));
+  EXPECT((grads.dweight.values() == std::vector<float>{1, -4, 1, -4}));
+
+  // element-wise neighbours: add, mul, tensor + element, relu, and the closed forms of sigmoid / tanh at 0
+  Tensor<float> p({2, 3}, {1, -2, 3, -4, 5, -6}), r({2, 3}, {0.5f, 0.5f, 0.5f, 2, 2, 2});
+  EXPECT((add(q, p, r).values() == std::vector<float>{1.5f, -1.5f, 3.5f, -2, 7, -4}));
+  EXPECT((mul(q, p, r).values() == std::vector<float>{0.5f, -1, 1.5f, -8, 10, -12}));
+  EXPECT((add(q, p, 1.0f).values() == std::vector<float>{2, -1, 4, -3, 6, -5}));
+  EXPECT((relu(q, p).values() == std::vector<float>{1, 0, 3, 0, 5, 0}));
+  Tensor<float> zeros({1, 4}, std::vector<float>(4, 0.0f));
+  EXPECT((sigmoid(q, zeros).values() == std::vector<float>(4, 0.5f)));
+  EXPECT((tanh(q, zeros).values() == std::vector<float>(4, 0.0f)));
+  EXPECT((add(q, p.t(), r.t()).values() == std::vector<float>{1.5f, -2, -1.5f, 7, 3.5f, -4}));
+
   // error behaviour: shape mismatch is caught before the call; double precision is NotSupported
   bool threw = false;
   try { matmul(q, a, false, a, false); } catch (const std::invalid_argument&) { threw = true; }

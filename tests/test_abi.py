@@ -83,6 +83,62 @@ def test_descriptor_validation_without_gpu():
         == native.ERROR_INVALID_VALUE
 
 
+def test_elementwise_and_backward_validation_without_gpu():
+    L = native.lib()
+    dummy = ctypes.c_void_p(256)
+    ad, k1 = native.make_descriptor(native.REAL32F, (4, 8), (8, 1), native.ORDER_ROW)
+    bd, k2 = native.make_descriptor(native.REAL32F, (4, 9), (9, 1), native.ORDER_ROW)
+    d64, k3 = native.make_descriptor(native.REAL64F, (4, 8), (8, 1), native.ORDER_ROW)
+    vec, k4 = native.make_descriptor(native.REAL32F, (8,), (1,), native.ORDER_ROW)
+    for name in ("srtAdd", "srtSub", "srtMul", "srtDiv", "srtMax", "srtMin"):
+        f = getattr(L, name)
+        assert f(dummy, ctypes.byref(ad), dummy, ctypes.byref(bd), dummy, ctypes.byref(ad), None) \
+            == native.ERROR_INVALID_VALUE                       # shapes differ
+        assert f(dummy, ctypes.byref(d64), dummy, ctypes.byref(d64), dummy, ctypes.byref(d64), None) \
+            == native.ERROR_NOT_SUPPORTED                       # element type: caller's CPU fallback
+        assert f(dummy, None, dummy, ctypes.byref(ad), dummy, ctypes.byref(ad), None) == native.ERROR_INVALID_VALUE
+        assert getattr(L, name + "TE")(dummy, ctypes.byref(ad), None, dummy, ctypes.byref(ad), None) \
+            == native.ERROR_INVALID_VALUE                       # no element
+    for name in ("srtNeg", "srtExp", "srtSigmoid", "srtTanh"):
+        assert getattr(L, name)(dummy, ctypes.byref(ad), dummy, ctypes.byref(d64), None) == native.ERROR_NOT_SUPPORTED
+        assert getattr(L, name)(dummy, ctypes.byref(ad), dummy, ctypes.byref(vec), None) == native.ERROR_INVALID_VALUE
+    assert L.srtCopy(dummy, ctypes.byref(d64), dummy, ctypes.byref(ad), None) == native.ERROR_NOT_SUPPORTED
+    assert L.srtAddFlat(native.REAL64F, dummy, dummy, dummy, 16, None) == native.ERROR_NOT_SUPPORTED
+    assert L.srtAddFlat(native.REAL32F, dummy, dummy, dummy, 0, None) == native.SUCCESS
+    assert L.srtCopyFlat(native.REAL32F, None, native.REAL16BF, dummy, 16, None) == native.ERROR_INVALID_VALUE
+    assert L.srtFillFlat(native.REAL32F, dummy, None, 16, None) == native.ERROR_INVALID_VALUE
+    # empty tensors: success before any pointer is looked at
+    e, k5 = native.make_descriptor(native.REAL32F, (0, 8), (8, 1), native.ORDER_ROW)
+    assert L.srtAdd(None, ctypes.byref(e), None, ctypes.byref(e), None, ctypes.byref(e), None) == native.SUCCESS
+    # backward: extents, activation code, element type, rank
+    f = L.srtActivationBackwardBias
+    assert f(dummy, ctypes.byref(ad), dummy, ctypes.byref(bd), 1, 0.0, dummy, ctypes.byref(ad), None, None, None) \
+        == native.ERROR_INVALID_VALUE
+    assert f(dummy, ctypes.byref(ad), dummy, ctypes.byref(ad), 6, 0.0, dummy, ctypes.byref(ad), None, None, None) \
+        == native.ERROR_INVALID_VALUE
+    assert f(dummy, ctypes.byref(d64), dummy, ctypes.byref(d64), 1, 0.0, dummy, ctypes.byref(d64), None, None, None) \
+        == native.ERROR_NOT_SUPPORTED
+    assert f(dummy, ctypes.byref(vec), dummy, ctypes.byref(vec), 1, 0.0, dummy, ctypes.byref(vec), None, None, None) \
+        == native.ERROR_NOT_SUPPORTED
+    bad_bias, k6 = native.make_descriptor(native.REAL32F, (9,), (1,), native.ORDER_ROW)
+    assert f(dummy, ctypes.byref(ad), dummy, ctypes.byref(ad), 1, 0.0, dummy, ctypes.byref(ad), dummy,
+             ctypes.byref(bad_bias), None) == native.ERROR_INVALID_VALUE
+
+
+def test_repeating_views_and_gradient_table_shapes():
+    b = srt.Tensor(np.arange(4, dtype=np.float32))
+    r = srt.Tensor.repeating(b, (3, 4))
+    assert r.shape == (3, 4) and r.strides == (0, 1)
+    c = srt.Tensor(np.zeros((3, 1), np.float32))
+    assert srt.Tensor.repeating(c, (3, 5)).strides == (1, 0)
+    with pytest.raises(ValueError):
+        srt.Tensor.repeating(b, (3, 5))
+    assert srt.Tensor(np.zeros((2, 3), np.float32)).is_contiguous
+    assert not srt.Tensor(np.zeros((4, 6), np.float32))[:, 1:4].is_contiguous
+    assert srt.Tensor(np.zeros(2, np.uint16)).element_storage(1.0)[0] == 0x3F80
+    assert srt.Tensor(np.zeros(2, np.uint16)).element_storage(float("nan"))[0] == 0x7FFF
+
+
 def test_kernel_selection_is_queryable_without_gpu():
     L = native.lib()
 

@@ -1,0 +1,219 @@
+"""GPU parity tests of the element-wise neighbours of the path (srtAdd ... srtFillFlat) and of
+the recurrent cells built from them, through the C ABI, against the CPU oracle.
+
+Bars: +, -, *, /, max, min, neg, copy / conversion and fill are bit-exact (one correctly rounded
+fp32 operation and one rounding to the element type on both sides); exp, sigmoid and tanh go
+through different libm implementations, so they are held to 2 units in the last place of the
+stored type (fp32: 4e-7 relative + 1e-7 absolute).  The LSTM fixtures of the reference's tests are
+reproduced to 1e-6, as there.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import swiftrt_amd as srt
+from oracle import srt_oracle as ora
+from swiftrt_amd import native
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+DTS = [H.F32, H.F16, H.BF16]
+EXACT_BINARY = [("add", "add"), ("sub", "subtract"), ("mul", "mul"), ("div", "div"), ("max", "max"), ("min", "min")]
+
+
+def rand_storage(g, shape, dt, scale=2.0):
+    return H.encode((g.standard_normal(shape) * scale).astype(np.float32), dt)
+
+
+def close_transcendental(got_st, want_st, dt):
+    got, want = H.decode(got_st).astype(np.float64), H.decode(want_st).astype(np.float64)
+    tol = 2 * (2.0 ** -23 if dt == H.F32 else 2 * H.ULP[dt])
+    return np.all(np.abs(got - want) <= tol * np.abs(want) + 1e-7)
+
+
+# ---- tensor-tensor, dense: the vector path --------------------------------------------------------
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("op,fn", EXACT_BINARY)
+def test_binary_dense_bit_exact(op, fn, dt):
+    g = H.rng(11)
+    a_st, b_st = rand_storage(g, (257, 384), dt), rand_storage(g, (257, 384), dt)
+    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+    out = srt.Tensor(shape=a.shape, dtype=a.dtype)
+    getattr(srt.current_queue(), fn)(a, b, out)
+    assert np.array_equal(out.array(), ora.elementwise(op, a_st, b_st))
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_binary_odd_sizes_and_misaligned_views(dt):
+    """Extents that are not a multiple of the vector width and views that start off a 16-byte
+    boundary take the element-at-a-time path of the same kernel."""
+    g = H.rng(12)
+    a_st, b_st = rand_storage(g, (33, 131), dt), rand_storage(g, (33, 131), dt)
+    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+    assert np.array_equal((a + b).array(), ora.elementwise("add", a_st, b_st))
+    av, bv = a[1:30, 3:100], b[2:31, 5:102]
+    got = (av * bv).array()
+    assert np.array_equal(got, ora.elementwise("mul", a_st[1:30, 3:100], b_st[2:31, 5:102]))
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_bias_broadcast_add_and_rank3(dt):
+    """matmul(x, W) + bias as the reference spells it: the bias is a stride-0 view of the result's
+    shape (Tensor(repeating:to:)); also rank 3 and a column broadcast."""
+    g = H.rng(13)
+    x_st, bias_st = rand_storage(g, (64, 256), dt), rand_storage(g, (256,), dt)
+    x, bias = srt.Tensor(x_st), srt.Tensor(bias_st)
+    assert np.array_equal((x + bias).array(), ora.elementwise("add", x_st, bias_st))
+    col_st = rand_storage(g, (64, 1), dt)
+    assert np.array_equal((x * srt.Tensor(col_st)).array(), ora.elementwise("mul", x_st, col_st))
+    t3_st, m_st = rand_storage(g, (5, 17, 24), dt), rand_storage(g, (17, 24), dt)
+    assert np.array_equal((srt.Tensor(t3_st) - srt.Tensor(m_st)).array(), ora.elementwise("sub", t3_st, m_st))
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_transposed_and_column_major_operands(dt):
+    g = H.rng(14)
+    a_st, b_st = rand_storage(g, (40, 72), dt), rand_storage(g, (72, 40), dt)
+    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+    assert np.array_equal((a + b.t).array(), ora.elementwise("add", a_st, np.ascontiguousarray(b_st.T)))
+    ac = srt.Tensor(a_st, order=srt.Order.col)
+    bc = srt.Tensor(np.ascontiguousarray(b_st.T), order=srt.Order.col)
+    assert np.array_equal((ac * bc).array(), ora.elementwise("mul", a_st, np.ascontiguousarray(b_st.T)))
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_tensor_element_forms(dt):
+    g = H.rng(15)
+    a_st = rand_storage(g, (19, 200), dt)
+    a = srt.Tensor(a_st)
+    e = H.encode(np.array([0.75], np.float32), dt)
+    assert np.array_equal((a + 0.75).array(), ora.elementwise("add", a_st, e))
+    assert np.array_equal((a * 0.75).array(), ora.elementwise("mul", a_st, e))
+    assert np.array_equal((a - 0.75).array(), ora.elementwise("sub", a_st, e))
+    assert np.array_equal((a / 0.75).array(), ora.elementwise("div", a_st, e))
+    zero = H.encode(np.array([0.0], np.float32), dt)
+    assert np.array_equal(srt.relu(a).array(), ora.elementwise("max", a_st, zero))
+    assert np.array_equal(srt.minimum(a, 0.75).array(), ora.elementwise("min", a_st, e))
+    assert np.array_equal((-a).array(), ora.elementwise("neg", a_st))
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_max_min_nan_rule(dt):
+    """max is `a >= b ? a : b` (CpuMath.swift:1197): a NaN on the left yields the right operand,
+    a NaN on the right is returned."""
+    a_st = H.encode(np.array([[np.nan, 1.0, np.nan, -0.0]], np.float32), dt)
+    b_st = H.encode(np.array([[2.0, np.nan, np.nan, 0.0]], np.float32), dt)
+    got = H.decode(srt.maximum(srt.Tensor(a_st), srt.Tensor(b_st)).array())
+    assert got[0, 0] == 2.0 and np.isnan(got[0, 1]) and np.isnan(got[0, 2])
+    assert np.array_equal(srt.maximum(srt.Tensor(a_st), srt.Tensor(b_st)).array()[:, :1],
+                          ora.elementwise("max", a_st, b_st)[:, :1])
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("op", ["exp", "sigmoid", "tanh"])
+def test_transcendentals(op, dt):
+    g = H.rng(16)
+    a_st = rand_storage(g, (48, 160), dt, scale=3.0)
+    got = getattr(srt, op)(srt.Tensor(a_st)).array()
+    assert close_transcendental(got, ora.elementwise(op, a_st), dt)
+    # closed forms on exact inputs
+    z = H.encode(np.zeros((1, 8), np.float32), dt)
+    want = {"exp": 1.0, "sigmoid": 0.5, "tanh": 0.0}[op]
+    assert np.all(H.decode(getattr(srt, op)(srt.Tensor(z)).array()) == want)
+
+
+@pytest.mark.parametrize("src", DTS)
+@pytest.mark.parametrize("dst", DTS)
+def test_conversion(src, dst):
+    """srtCopy between any two of Float / Float16 / BFloat16: round to nearest even, exact when
+    widening; bit-exact against the oracle's codecs."""
+    g = H.rng(17)
+    vals = (g.standard_normal((31, 96)) * 100).astype(np.float32)
+    vals[0, :4] = [np.inf, -np.inf, 65519.9, 1e-8]      # fp16 overflow boundary, bf16/fp16 underflow
+    a_st = H.encode(vals, src)
+    got = srt.cast(srt.Tensor(a_st), H.NP_STORAGE[dst]).array()
+    want = ora.elementwise("copy", a_st, out_dtype=dst)
+    assert got.dtype == want.dtype and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_flat_forms_and_fill(dt):
+    g = H.rng(18)
+    n = 100003
+    a_st, b_st = rand_storage(g, (n,), dt), rand_storage(g, (n,), dt)
+    q = srt.current_queue()
+    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+    out = srt.Tensor(shape=[n], dtype=a.dtype)
+    L = native.lib()
+    native.check(L.srtAddFlat(a.type_id, a.device_read(q), b.device_read(q), out.device_read_write(q), n, q.stream))
+    assert np.array_equal(out.array(), ora.elementwise("add", a_st, b_st))
+    other = H.BF16 if dt != H.BF16 else H.F32
+    conv = srt.Tensor(shape=[n], dtype=H.NP_STORAGE[other])
+    native.check(L.srtCopyFlat(a.type_id, a.device_read(q), conv.type_id, conv.device_read_write(q), n, q.stream))
+    assert np.array_equal(conv.array(), ora.elementwise("copy", a_st, out_dtype=other))
+    f = srt.filled([7, 33], -1.5, H.NP_STORAGE[dt])
+    assert np.all(H.decode(f.array()) == -1.5)
+
+
+def test_errors_and_empty():
+    q = srt.current_queue()
+    L = native.lib()
+    a = srt.Tensor(np.zeros((4, 8), np.float32))
+    b = srt.Tensor(np.zeros((4, 9), np.float32))
+    out = srt.Tensor(shape=[4, 8], dtype=np.float32)
+    ad, k1 = a.descriptor()
+    bd, k2 = b.descriptor()
+    od, k3 = out.descriptor()
+    args = (a.device_read(q), ctypes.byref(ad), b.device_read(q), ctypes.byref(bd), out.device_read_write(q),
+            ctypes.byref(od), q.stream)
+    assert L.srtAdd(*args) == native.ERROR_INVALID_VALUE            # shapes differ
+    ad.type = native.REAL64F
+    assert L.srtAdd(a.device_read(q), ctypes.byref(ad), a.device_read(q), ctypes.byref(ad), out.device_read_write(q),
+                    ctypes.byref(od), q.stream) == native.ERROR_NOT_SUPPORTED   # caller's CPU fallback
+    assert L.srtAdd(None, None, None, None, None, None, q.stream) == native.ERROR_INVALID_VALUE
+    e = srt.Tensor(shape=[0, 8], dtype=np.float32)
+    assert (e + e).array().shape == (0, 8)
+    assert L.srtFillFlat(native.REAL32F, None, None, 0, q.stream) == native.SUCCESS
+
+
+# ---- the recurrent cells, unfused, on the device ----------------------------------------------------
+def test_lstm_fixture_unfused_on_device(kats):
+    """LSTMCell as the reference writes it (Recurrent.swift:255-266): concatenate, matmul with bias,
+    four gate slices (strided views), sigmoid / tanh, mul, add -- every step a device call --
+    reproduces lstmExpectedStates / lstmExpectedOutput to 1e-6 (test_Recurrent.swift:100-167)."""
+    k = kats["lstm"]
+    cell_layer = srt.LSTMCell(srt.Tensor(np.array(k["lstmInitialCellFusedWeights"], np.float32)),
+                              srt.Tensor(np.array(k["lstmInitialCellFusedBias"], np.float32)))
+    cell = srt.Tensor(np.array(k["lstmInitialStateCell"], np.float32))
+    hidden = srt.Tensor(np.array(k["lstmInitialStateHidden"], np.float32))
+    states = []
+    for x in k["lstmInputs"]:
+        cell, hidden = cell_layer(srt.Tensor(np.array([x], np.float32)), cell, hidden)
+        states.append(hidden.array())
+    assert np.max(np.abs(np.concatenate(states) - np.array(k["lstmExpectedStates"], np.float32))) <= 1e-6
+    assert np.max(np.abs(cell.array() - np.array(k["lstmExpectedOutput"], np.float32))) <= 1e-6
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_basic_rnn_cell_fused_and_unfused(dt):
+    """tanh(matmul([x, h], W) + b) (Recurrent.swift:157-161) as one fused Dense call (one rounding)
+    and as the reference's three device operations (a rounding after each): both within the
+    roundings they make of the fp64 value -- 1e-5 for fp32; one (fused) or three (unfused) roundings
+    of the stored type otherwise."""
+    g = H.rng(19)
+    x_st, h_st = rand_storage(g, (16, 24), dt, 0.5), rand_storage(g, (16, 40), dt, 0.5)
+    w_st, b_st = rand_storage(g, (64, 40), dt, 0.2), rand_storage(g, (40,), dt, 0.2)
+    w, b = srt.Tensor(w_st), srt.Tensor(b_st)
+    fused = srt.BasicRNNCell(w, b, fused=True)(srt.Tensor(x_st), srt.Tensor(h_st)).array()
+    unfused = srt.BasicRNNCell(w, b, fused=False)(srt.Tensor(x_st), srt.Tensor(h_st)).array()
+    xin = np.concatenate([H.to64(x_st), H.to64(h_st)], axis=1)
+    mm = xin @ H.to64(w_st)
+    pre = mm + H.to64(b_st)
+    want = np.tanh(pre)
+    # a rounding of the product or of the pre-activation moves tanh by at most that rounding (slope <= 1)
+    for got, roundings in ((fused, 1), (unfused, 3)):
+        err = np.abs(H.to64(got) - want)
+        bound = 1e-5 if dt == H.F32 else roundings * H.ULP[dt] * np.maximum(np.abs(mm), np.maximum(np.abs(pre), np.abs(want))) + 1e-6
+        assert np.all(err <= bound)

@@ -276,3 +276,92 @@ def test_dense_activations_closed_forms():
     xb, wb, bb = ora.encode(x, ora.BF16), ora.encode(w, ora.BF16), ora.encode(b, ora.BF16)
     assert np.array_equal(ora.decode(ora.dense_forward(xb, wb, bb, ora.RELU)), [[2.5, 0.0]])
     assert np.array_equal(ora.decode(ora.dense_forward(xb, wb, bb, ora.RELU, fused=False)), [[2.5, 0.0]])
+
+
+# ---- element-wise neighbours and the backward of the Dense epilogue ----------------------------------
+def test_elementwise_closed_forms_and_half_library_oracle():
+    a = np.array([[1.5, -2.0, 0.25, 3.0]], np.float32)
+    b = np.array([[0.5, 4.0, -0.25, 3.0]], np.float32)
+    for dt in (ora.F32, ora.F16, ora.BF16):
+        sa, sb = ora.encode(a, dt), ora.encode(b, dt)
+        assert np.array_equal(ora.decode(ora.elementwise("add", sa, sb)), [[2.0, 2.0, 0.0, 6.0]])
+        assert np.array_equal(ora.decode(ora.elementwise("sub", sa, sb)), [[1.0, -6.0, 0.5, 0.0]])
+        assert np.array_equal(ora.decode(ora.elementwise("mul", sa, sb)), [[0.75, -8.0, -0.0625, 9.0]])
+        assert np.array_equal(ora.decode(ora.elementwise("div", sa, sb)), [[3.0, -0.5, -1.0, 1.0]])
+        assert np.array_equal(ora.decode(ora.elementwise("max", sa, sb)), [[1.5, 4.0, 0.25, 3.0]])
+        assert np.array_equal(ora.decode(ora.elementwise("min", sa, sb)), [[0.5, -2.0, -0.25, 3.0]])
+        assert np.array_equal(ora.decode(ora.elementwise("neg", sa)), -a)
+    # numpy's own half arithmetic (an independent implementation) agrees with "fp32 op, round once"
+    g = np.random.Generator(np.random.Philox(31))
+    x = (g.standard_normal(4096) * 3).astype(np.float16)
+    y = (g.standard_normal(4096) * 3).astype(np.float16)
+    for op, fn in (("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)):
+        assert np.array_equal(ora.elementwise(op, x, y), fn(x, y)), op
+    # max is `a >= b ? a : b`: a NaN on the left gives the right operand, a NaN on the right is returned
+    n = ora.elementwise("max", np.array([np.nan, 1.0], np.float32), np.array([2.0, np.nan], np.float32))
+    assert n[0] == 2.0 and np.isnan(n[1])
+    # broadcast of a bias row, and a scalar element
+    m = ora.elementwise("add", np.ones((3, 4), np.float32), np.arange(4, dtype=np.float32))
+    assert np.array_equal(m, np.ones((3, 4)) + np.arange(4))
+    assert np.array_equal(ora.elementwise("mul", np.full((2, 2), 3.0, np.float32), np.array([0.5], np.float32)),
+                          np.full((2, 2), 1.5))
+
+
+def test_lstm_fixture_pins_the_unfused_elementwise_chain(kats):
+    """The reference's LSTM states are reproduced when every step after the matmul goes through the
+    oracle's element-wise functions (slices, sigmoid, tanh, mul, add) -- the chain the device runs."""
+    k = kats["lstm"]
+    w = np.array(k["lstmInitialCellFusedWeights"], np.float32)
+    bias = np.array(k["lstmInitialCellFusedBias"], np.float32)
+    cell = np.array(k["lstmInitialStateCell"], np.float32)
+    hidden = np.array(k["lstmInitialStateHidden"], np.float32)
+    states = []
+    for x in k["lstmInputs"]:
+        gate_in = np.concatenate([np.array([x], np.float32), hidden], axis=1)
+        z = ora.elementwise("add", ora.matmul(gate_in, w), bias)
+        i, u = ora.elementwise("sigmoid", z[:, 0:4]), ora.elementwise("tanh", z[:, 4:8])
+        f, o = ora.elementwise("sigmoid", z[:, 8:12]), ora.elementwise("sigmoid", z[:, 12:16])
+        cell = ora.elementwise("add", ora.elementwise("mul", cell, f), ora.elementwise("mul", i, u))
+        hidden = ora.elementwise("mul", ora.elementwise("tanh", cell), o)
+        states.append(hidden.copy())
+    assert np.max(np.abs(np.concatenate(states) - np.array(k["lstmExpectedStates"], np.float32))) <= 1e-6
+    assert np.max(np.abs(cell - np.array(k["lstmExpectedOutput"], np.float32))) <= 1e-6
+
+
+def test_conversion_matches_numpy_half_and_independent_bf16():
+    g = np.random.Generator(np.random.Philox(32))
+    v = (g.standard_normal(8192) * 50).astype(np.float32)
+    assert np.array_equal(ora.elementwise("copy", v, out_dtype=ora.F16), v.astype(np.float16))
+    u = v.view(np.uint32)
+    assert np.array_equal(ora.elementwise("copy", v, out_dtype=ora.BF16),
+                          ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16))
+    h = v.astype(np.float16)
+    assert np.array_equal(ora.elementwise("copy", h, out_dtype=ora.F32), h.astype(np.float32))
+
+
+def test_activation_slopes_against_numerical_derivative():
+    """Pins the closed-form derivative-through-the-output used by the backward: central differences
+    of the oracle's own forward activation."""
+    z = np.linspace(-2.0, 2.0, 41) + 0.0123
+    for kind, coef in ((ora.SIGMOID, 0.0), (ora.RELU, 0.0), (ora.TANH, 0.0), (ora.CLIPPED_RELU, 0.75),
+                       (ora.ELU, 0.5), (ora.IDENTITY, 0.0)):
+        def f(t):
+            return np.array([ora.lib().srt_oracle_activation(kind, coef, float(v)) for v in t], np.float64)
+        h = 1e-3
+        numeric = (f(z + h) - f(z - h)) / (2 * h)
+        got = ora.activation_slope(kind, f(z).astype(np.float32), coef)
+        assert np.max(np.abs(got - numeric)) < 2e-3, kind
+
+
+def test_activation_backward_bias_small_case():
+    y = np.array([[0.5, -1.0], [2.0, 0.0], [1.0, 3.0]], np.float32)
+    dy = np.array([[1.0, 2.0], [3.0, 4.0], [-5.0, 6.0]], np.float32)
+    dx, db = ora.activation_backward_bias(y, dy, ora.RELU)
+    assert np.array_equal(dx, [[1.0, 0.0], [3.0, 0.0], [-5.0, 6.0]]) and np.array_equal(db, [-1.0, 6.0])
+    dx, db = ora.activation_backward_bias(y, dy, ora.IDENTITY)
+    assert np.array_equal(dx, dy) and np.array_equal(db, dy.sum(axis=0))
+    ys = np.array([[0.5, 0.25]], np.float32)
+    dx, _ = ora.activation_backward_bias(ys, np.ones_like(ys), ora.SIGMOID)
+    assert np.array_equal(dx, [[0.25, 0.1875]])
+    dx, _ = ora.activation_backward_bias(ys, np.ones_like(ys), ora.TANH)
+    assert np.array_equal(dx, [[0.75, 0.9375]])
