@@ -216,6 +216,41 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
                                const srtTensorDescriptor* oDesc, const void* a, const void* b,
                                const void* out, char* name, size_t nameCapacity);
 
+/* ---- plan / tune cache ------------------------------------------------------------------------
+ * The role of ExecutionPlanCache / ExecutionPlanner (Sources/SwiftRTCore/platform/common/
+ * ExecutionPlanner.swift:20-29), of the `plan` key a layer keeps (Sources/SwiftRTLayers/Dense.swift:29)
+ * and of CudaMatmul2.tune (Sources/SwiftRTCore/platform/cuda/functions/CudaMatmul.swift:112-120, an
+ * empty body in the reference).
+ *
+ * srtMatmulTune takes the arguments of srtMatmulBiasActivation, runs the problem with every kernel
+ * plan it qualifies for (a few timed launches each, on `stream`; the call synchronises with the
+ * stream), records the fastest in a process-wide cache and leaves `out` computed by it.  The key is
+ * the element type, M, N, K, batch, the layout class of the operands (which dimension is contiguous,
+ * whether rows keep 16-byte alignment) and the epilogue (bias present, activation).  Every later
+ * srtMatmul / srtMatmulBiasActivation call with the same key runs the recorded plan -- provided this
+ * call's pointers still meet the plan's alignment rules; otherwise, and for keys never tuned, the
+ * built-in heuristic decides.  All plans compute the same function to the documented tolerance
+ * (sums are fp32; their order differs between plans).
+ * chosen (optional): receives the plan's name ("mfma_256x256", "mfma_128x128", "mfma_64x64", "skinny",
+ * "f32_mfma_64x64", "f32_mfma_splitk", "generic").
+ * The cache is thread-safe.  Save / Load use a small text file, one plan per line:
+ *   dtype M N K batch layout epilogue plan-name
+ * (layout: bit 0 A contiguous along k, 1 A along m, 2 B along k, 3 B along n, 4 result rows
+ * contiguous, 5 bias per row of the computed tile, 6 rows 16-byte aligned; epilogue: bit 0 bias
+ * present, bits 1.. the srtActivation code), so a tuned set of shapes can be shipped with an
+ * application; Load merges into the cache and is
+ * all-or-nothing: a malformed file returns srtErrorInvalidValue and changes nothing. */
+srtStatus srtMatmulTune(const void* a, const srtTensorDescriptor* aDesc, int32_t transposeA,
+                        const void* b, const srtTensorDescriptor* bDesc, int32_t transposeB,
+                        const void* bias, const srtTensorDescriptor* biasDesc,
+                        srtActivation activation, double coef,
+                        void* out, const srtTensorDescriptor* oDesc, srtStream stream,
+                        char* chosen, size_t chosenCapacity);
+srtStatus srtPlanCacheClear(void);
+srtStatus srtPlanCacheCount(size_t* count);
+srtStatus srtPlanCacheSave(const char* path);
+srtStatus srtPlanCacheLoad(const char* path);
+
 /* ---- backward of the Dense epilogue ------------------------------------------------------------
  * dx = dy * activation'(y) and, when dbias != NULL, dbias[n] = sum over rows of dx[:, n], in one
  * pass over y and dy.  y is the OUTPUT of the forward activation: the derivative is written in

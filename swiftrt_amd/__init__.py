@@ -8,7 +8,8 @@ the first native call does, and raises if it has not been built.
 """
 from . import native
 from .native import NotSupportedError, SrtError
-from .platform import HipDevice, HipDeviceMemory, HipEvent, HipPlatform, HipQueue, current_queue, using
+from .platform import (HipDevice, HipDeviceMemory, HipEvent, HipPlatform, HipQueue, PlanCache, current_queue,
+                       using)
 from .tensor import (ActivationType, BasicRNNCell, Dense, LSTMCell, Order, Tensor, cast, concatenate, dense_backward,
                      exp, filled, matmul, matmul_gradients, maximum, minimum, relu, sigmoid, tanh)
 

@@ -174,16 +174,26 @@ bool f32_mfma_supported(const GemmProblem& p) {
   return true;
 }
 
-hipError_t launch_f32_mfma(const GemmProblem& p, hipStream_t stream) {
+// The split-K variant pays when 64 x 64 tiles alone would leave most CUs idle.
+bool f32_mfma_prefers_splitk(const GemmProblem& p) {
   const long long tiles64 = (long long)((p.M + FT - 1) / FT) * ((p.N + FT - 1) / FT) * p.batch;
-  if (tiles64 < 192 && p.K >= 64) {
+  return tiles64 < 192 && p.K >= 64;
+}
+
+hipError_t launch_f32_mfma_variant(const GemmProblem& p, bool splitk, hipStream_t stream) {
+  if (splitk) {
     dim3 grid((p.N + 31) / 32, (p.M + 31) / 32, p.batch);
     hipLaunchKernelGGL(gemm_f32_mfma_splitk_kernel, grid, dim3(256), 0, stream, p);
   } else {
+    if ((p.M + FT - 1) / FT > 65535) return hipErrorInvalidValue;
     dim3 grid((p.N + FT - 1) / FT, (p.M + FT - 1) / FT, p.batch);
     hipLaunchKernelGGL(gemm_f32_mfma_kernel, grid, dim3(256), 0, stream, p);
   }
   return hipGetLastError();
+}
+
+hipError_t launch_f32_mfma(const GemmProblem& p, hipStream_t stream) {
+  return launch_f32_mfma_variant(p, f32_mfma_prefers_splitk(p), stream);
 }
 
 }  // namespace srt

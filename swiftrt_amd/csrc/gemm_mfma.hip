@@ -329,32 +329,47 @@ inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 // The MFMA family needs: a 16-bit element type, C rows contiguous, each operand contiguous
 // along k or along its other dimension with 16-byte aligned rows, and extents along the
 // contiguous dimensions that are multiples of 8 (so every 16-byte load is whole).
-int mfma_select(const GemmProblem& p) {
-  if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
-  if (p.scn != 1 || p.K < 1) return 0;
-  if (p.batch > 65535) return 0;
+// Layout bits of a qualifying problem (bit 1: A k-contiguous, bit 0: B k-contiguous), or -1.
+static int mfma_layout(const GemmProblem& p) {
+  if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return -1;
+  if (p.scn != 1 || p.K < 1) return -1;
+  if (p.batch > 65535) return -1;
   bool a_kc, b_kc;
   if (p.sak == 1 && (p.K % 8) == 0) a_kc = true;
   else if (p.sam == 1 && (p.M % 8) == 0) a_kc = false;
-  else return 0;
+  else return -1;
   if (p.sbk == 1 && (p.K % 8) == 0) b_kc = true;
   else if (p.sbn == 1 && (p.N % 8) == 0) b_kc = false;
-  else return 0;
+  else return -1;
   const long long lda = a_kc ? p.sam : p.sak, ldb = b_kc ? p.sbn : p.sbk;
   // a single row/column operand may carry any leading stride; otherwise rows must stay aligned
-  if ((lda % 8) != 0 || (ldb % 8) != 0) return 0;
-  if ((p.sab % 8) != 0 || (p.sbb % 8) != 0) return 0;
-  if (!aligned16(p.A) || !aligned16(p.B)) return 0;
-  if (p.sam < 0 || p.sak < 0 || p.sbk < 0 || p.sbn < 0 || p.scm < 0) return 0;
+  if ((lda % 8) != 0 || (ldb % 8) != 0) return -1;
+  if ((p.sab % 8) != 0 || (p.sbb % 8) != 0) return -1;
+  if (!aligned16(p.A) || !aligned16(p.B)) return -1;
+  if (p.sam < 0 || p.sak < 0 || p.sbk < 0 || p.sbn < 0 || p.scm < 0) return -1;
+  return (a_kc ? 2 : 0) | (b_kc ? 1 : 0);
+}
 
+// Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64), or 0 when the
+// problem does not qualify for it.
+int mfma_config(const GemmProblem& p, int tile) {
+  const int layout = mfma_layout(p);
+  if (layout < 0 || tile < 1 || tile > 3) return 0;
+  if (tile == 1 && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
+  return (tile << 2) | layout;
+}
+
+int mfma_select(const GemmProblem& p) {
+  const int layout = mfma_layout(p);
+  if (layout < 0) return 0;
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
   // Largest tile that still gives every CU work: 256 x 256 (ring kernel) from 192 tiles up, 128 x 128
   // from one tile per CU up, otherwise 64 x 64 (measured on batch 32 x 256^3: 7.7 us against 15.0 us).
   int tile;
-  if (tiles(256) >= 192 && ring_fits_problem(p, a_kc, b_kc)) tile = 1;
+  if (tiles(256) >= 192 && ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) tile = 1;
   else if (tiles(128) >= 256) tile = 2;
   else tile = 3;
-  return (tile << 2) | (a_kc ? 2 : 0) | (b_kc ? 1 : 0);
+  return (tile << 2) | layout;
 }
 
 const char* mfma_name(int config) {

@@ -2,6 +2,9 @@
 // and views into one strided problem, and kernel-family selection.
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <tuple>
 
 #include "gemm_common.h"
 #include "status.h"
@@ -78,29 +81,155 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
   return srtSuccess;
 }
 
-enum Family { kGeneric, kMfma, kSkinny, kF32Mfma };
+// ---- plans ------------------------------------------------------------------------------------
+// A plan names the kernel that runs a problem.  The heuristic picks one per call; srtMatmulTune
+// measures every plan the problem qualifies for and records the fastest in a process-wide cache
+// keyed by the problem's shape, layout class and epilogue, which later calls consult first
+// (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
+// and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
+enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK, kPlanCount };
 
-Family select(const GemmProblem& p, int* config) {
-  *config = 0;
-  if (srt::skinny_supported(p)) return kSkinny;
-  int c = srt::mfma_select(p);
-  if (c) { *config = c; return kMfma; }
-  if (srt::f32_mfma_supported(p)) return kF32Mfma;
-  return kGeneric;
+const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
+                                            "f32_mfma_64x64", "f32_mfma_splitk"};
+
+bool plan_supported(const GemmProblem& p, Plan plan) {
+  switch (plan) {
+    case kPlanSkinny: return srt::skinny_supported(p);
+    case kPlanRing256: return srt::mfma_config(p, 1) != 0;
+    case kPlanMfma128: return srt::mfma_config(p, 2) != 0;
+    case kPlanMfma64: return srt::mfma_config(p, 3) != 0;
+    case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
+    case kPlanF32SplitK: return srt::f32_mfma_supported(p);
+    default: return srt::generic_supported(p);
+  }
+}
+
+Plan heuristic_plan(const GemmProblem& p) {
+  if (srt::skinny_supported(p)) return kPlanSkinny;
+  const int c = srt::mfma_select(p);
+  if (c) return (c >> 2) == 1 ? kPlanRing256 : (c >> 2) == 2 ? kPlanMfma128 : kPlanMfma64;
+  if (srt::f32_mfma_supported(p)) return srt::f32_mfma_prefers_splitk(p) ? kPlanF32SplitK : kPlanF32Tile64;
+  return kPlanGeneric;
+}
+
+hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
+  switch (plan) {
+    case kPlanSkinny: return srt::launch_skinny(p, stream);
+    case kPlanRing256: return srt::launch_mfma(p, srt::mfma_config(p, 1), stream);
+    case kPlanMfma128: return srt::launch_mfma(p, srt::mfma_config(p, 2), stream);
+    case kPlanMfma64: return srt::launch_mfma(p, srt::mfma_config(p, 3), stream);
+    case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
+    case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
+    default: return srt::launch_generic(p, stream);
+  }
+}
+
+struct PlanKey {
+  int dtype, M, N, K, batch, layout, epilogue;
+  bool operator<(const PlanKey& o) const {
+    return std::tie(dtype, M, N, K, batch, layout, epilogue) <
+           std::tie(o.dtype, o.M, o.N, o.K, o.batch, o.layout, o.epilogue);
+  }
+};
+
+// Layout class: which dimension of each operand is contiguous (bits 0-1: A along k / m, bits 2-3:
+// B along k / n), whether the batch strides are dense, and whether rows keep 16-byte alignment.
+PlanKey key_of(const GemmProblem& p) {
+  int layout = 0;
+  if (p.sak == 1) layout |= 1;
+  if (p.sam == 1) layout |= 2;
+  if (p.sbk == 1) layout |= 4;
+  if (p.sbn == 1) layout |= 8;
+  if (p.scn == 1) layout |= 16;
+  if (p.bias_per_row) layout |= 32;
+  const long long lda = p.sak == 1 ? p.sam : p.sak, ldb = p.sbk == 1 ? p.sbn : p.sbk;
+  if (lda % 8 == 0 && ldb % 8 == 0 && p.scm % 8 == 0) layout |= 64;
+  const int epilogue = (p.bias ? 1 : 0) | (p.activation << 1);
+  return PlanKey{p.dtype, p.M, p.N, p.K, p.batch, layout, epilogue};
+}
+
+class PlanCache {
+ public:
+  bool find(const PlanKey& k, Plan* plan) {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = plans_.find(k);
+    if (it == plans_.end()) return false;
+    *plan = it->second;
+    return true;
+  }
+  void put(const PlanKey& k, Plan plan) {
+    std::lock_guard<std::mutex> lock(mu_);
+    plans_[k] = plan;
+  }
+  void clear() {
+    std::lock_guard<std::mutex> lock(mu_);
+    plans_.clear();
+  }
+  size_t size() {
+    std::lock_guard<std::mutex> lock(mu_);
+    return plans_.size();
+  }
+  // One plan per line: dtype M N K batch layout epilogue plan-name
+  srtStatus save(const char* path) {
+    std::lock_guard<std::mutex> lock(mu_);
+    FILE* f = std::fopen(path, "w");
+    if (!f) return srtErrorInvalidValue;
+    std::fprintf(f, "# SwiftRTHip matmul plans v1: dtype M N K batch layout epilogue plan\n");
+    for (const auto& kv : plans_) {
+      const PlanKey& k = kv.first;
+      std::fprintf(f, "%d %d %d %d %d %d %d %s\n", k.dtype, k.M, k.N, k.K, k.batch, k.layout, k.epilogue,
+                   kPlanNames[kv.second]);
+    }
+    return std::fclose(f) == 0 ? srtSuccess : srtErrorUnknown;
+  }
+  // All or nothing: a malformed line or an unknown plan name leaves the cache as it was.
+  srtStatus load(const char* path) {
+    FILE* f = std::fopen(path, "r");
+    if (!f) return srtErrorInvalidValue;
+    std::map<PlanKey, Plan> read;
+    char line[256];
+    bool ok = true;
+    while (ok && std::fgets(line, sizeof(line), f)) {
+      if (line[0] == '#' || line[0] == '\n') continue;
+      PlanKey k;
+      char name[64];
+      if (std::sscanf(line, "%d %d %d %d %d %d %d %63s", &k.dtype, &k.M, &k.N, &k.K, &k.batch, &k.layout,
+                      &k.epilogue, name) != 8) { ok = false; break; }
+      int plan = -1;
+      for (int i = 0; i < kPlanCount; ++i)
+        if (std::strcmp(name, kPlanNames[i]) == 0) plan = i;
+      if (plan < 0 || k.M < 0 || k.N < 0 || k.K < 0 || k.batch < 0) { ok = false; break; }
+      read[k] = (Plan)plan;
+    }
+    std::fclose(f);
+    if (!ok) return srtErrorInvalidValue;
+    std::lock_guard<std::mutex> lock(mu_);
+    for (const auto& kv : read) plans_[kv.first] = kv.second;
+    return srtSuccess;
+  }
+
+ private:
+  std::mutex mu_;
+  std::map<PlanKey, Plan> plans_;
+};
+
+PlanCache& plan_cache() {
+  static PlanCache* cache = new PlanCache();   // never destroyed: calls may race with process exit
+  return *cache;
+}
+
+// The plan a call runs: the cached one when it still qualifies (alignment of this call's pointers
+// is not part of the key), else the heuristic's.
+Plan select(const GemmProblem& p) {
+  Plan plan;
+  if (plan_cache().size() != 0 && plan_cache().find(key_of(p), &plan) && plan_supported(p, plan)) return plan;
+  return heuristic_plan(p);
 }
 
 srtStatus run(const GemmProblem& p, hipStream_t stream) {
-  int config = 0;
-  hipError_t e;
-  switch (select(p, &config)) {
-    case kSkinny: e = srt::launch_skinny(p, stream); break;
-    case kMfma: e = srt::launch_mfma(p, config, stream); break;
-    case kF32Mfma: e = srt::launch_f32_mfma(p, stream); break;
-    default:
-      if (!srt::generic_supported(p)) return srtErrorNotSupported;
-      e = srt::launch_generic(p, stream);
-  }
-  return srt::from_hip(e);
+  const Plan plan = select(p);
+  if (plan == kPlanGeneric && !srt::generic_supported(p)) return srtErrorNotSupported;
+  return srt::from_hip(launch_plan(p, plan, stream));
 }
 
 }  // namespace
@@ -138,19 +267,72 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
   srtStatus s = build_problem(a, aDesc, transposeA, b, bDesc, transposeB, nullptr, nullptr,
                               srtActivationIdentity, 0.0, const_cast<void*>(out), oDesc, &p, &empty);
   if (s != srtSuccess) return s;
-  const char* n = "generic";
-  if (empty) n = "empty";
-  else {
-    int config = 0;
-    switch (select(p, &config)) {
-      case kSkinny: n = "skinny"; break;
-      case kMfma: n = srt::mfma_name(config); break;
-      case kF32Mfma: n = "f32_mfma"; break;
-      default: n = "generic";
-    }
+  const char* n = "empty";
+  if (!empty) {
+    const Plan plan = select(p);
+    n = kPlanNames[plan];
+    if (plan == kPlanF32Tile64 || plan == kPlanF32SplitK) n = "f32_mfma";   // one family name for both fp32 tiles
   }
   std::snprintf(name, nameCapacity, "%s", n);
   return srtSuccess;
 }
+
+srtStatus srtMatmulTune(const void* a, const srtTensorDescriptor* aDesc, int32_t transposeA,
+                        const void* b, const srtTensorDescriptor* bDesc, int32_t transposeB,
+                        const void* bias, const srtTensorDescriptor* biasDesc,
+                        srtActivation activation, double coef,
+                        void* out, const srtTensorDescriptor* oDesc, srtStream stream,
+                        char* chosen, size_t chosenCapacity) {
+  if (chosen && chosenCapacity) chosen[0] = 0;
+  GemmProblem p;
+  bool empty = false;
+  srtStatus s = build_problem(a, aDesc, transposeA, b, bDesc, transposeB, bias, biasDesc, (int)activation, coef,
+                              out, oDesc, &p, &empty);
+  if (s != srtSuccess || empty) return s;
+  hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return srtErrorUnknown;
+  if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return srtErrorUnknown; }
+  const Plan fallback = heuristic_plan(p);
+  Plan best = fallback;
+  float best_ms = -1.0f;
+  hipError_t err = hipSuccess;
+  for (int c = 0; c < kPlanCount && err == hipSuccess; ++c) {
+    const Plan plan = (Plan)c;
+    if (!plan_supported(p, plan)) continue;
+    // the FMA kernel is orders of magnitude slower on large problems: skip it when a matrix-core plan exists
+    if (plan == kPlanGeneric && fallback != kPlanGeneric && 2.0 * p.M * p.N * p.K * p.batch > 1e9) continue;
+    const int warm = 2, reps = 8;
+    for (int i = 0; i < warm && err == hipSuccess; ++i) err = launch_plan(p, plan, hs);
+    if (err == hipSuccess) err = hipEventRecord(e0, hs);
+    for (int i = 0; i < reps && err == hipSuccess; ++i) err = launch_plan(p, plan, hs);
+    if (err == hipSuccess) err = hipEventRecord(e1, hs);
+    if (err == hipSuccess) err = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+    if (err == hipSuccess && (best_ms < 0.0f || ms < best_ms)) { best_ms = ms; best = plan; }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (err != hipSuccess) return srt::from_hip(err);
+  if (best_ms < 0.0f) return srtErrorNotSupported;   // no kernel qualifies: the caller's CPU path
+  plan_cache().put(key_of(p), best);
+  // leave `out` written by the chosen plan
+  err = launch_plan(p, best, hs);
+  if (chosen && chosenCapacity) std::snprintf(chosen, chosenCapacity, "%s", kPlanNames[best]);
+  return srt::from_hip(err);
+}
+
+srtStatus srtPlanCacheClear(void) { plan_cache().clear(); return srtSuccess; }
+
+srtStatus srtPlanCacheCount(size_t* count) {
+  if (!count) return srtErrorInvalidValue;
+  *count = plan_cache().size();
+  return srtSuccess;
+}
+
+srtStatus srtPlanCacheSave(const char* path) { return path ? plan_cache().save(path) : srtErrorInvalidValue; }
+
+srtStatus srtPlanCacheLoad(const char* path) { return path ? plan_cache().load(path) : srtErrorInvalidValue; }
 
 }  // extern "C"

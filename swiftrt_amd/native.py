@@ -91,6 +91,12 @@ SIGNATURES = {
     "srtDelayStream": (_i32, [ctypes.c_double, _vp]),
     "srtActivationBackwardBias": (_i32, [_vp, _descp, _vp, _descp, _i32, ctypes.c_double, _vp, _descp,
                                           _vp, _descp, _vp]),
+    "srtMatmulTune": (_i32, [_vp, _descp, _i32, _vp, _descp, _i32, _vp, _descp, _i32, ctypes.c_double, _vp, _descp,
+                              _vp, ctypes.c_char_p, ctypes.c_size_t]),
+    "srtPlanCacheClear": (_i32, []),
+    "srtPlanCacheCount": (_i32, [ctypes.POINTER(ctypes.c_size_t)]),
+    "srtPlanCacheSave": (_i32, [ctypes.c_char_p]),
+    "srtPlanCacheLoad": (_i32, [ctypes.c_char_p]),
     "srtAddFlat": (_i32, [_i32, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "srtCopyFlat": (_i32, [_i32, _vp, _i32, _vp, ctypes.c_size_t, _vp]),
     "srtFillFlat": (_i32, [_i32, _vp, _vp, ctypes.c_size_t, _vp]),

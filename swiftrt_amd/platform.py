@@ -165,6 +165,29 @@ class HipQueue:
         del ka, kb, ko
         check(st, "srtMatmul")
 
+    def tune_matmul(self, lhs, transpose_lhs, rhs, transpose_rhs, result, bias=None, activation=None, coef=0.0):
+        """Role of CudaMatmul2.tune (CudaMatmul.swift:112-120): measures every kernel plan the problem
+        qualifies for, records the fastest in the native plan cache (used by every later matmul with
+        the same shape, layout class and epilogue) and returns its name.  `result` holds the product."""
+        from .tensor import ActivationType
+        self.select()
+        a_ptr, b_ptr = lhs.device_read(self), rhs.device_read(self)
+        bias_ptr = bias.device_read(self) if bias is not None else None
+        o_ptr = result.device_read_write(self)
+        ad, ka = lhs.descriptor()
+        bd, kb = rhs.descriptor()
+        od, ko = result.descriptor()
+        biasd, kbias = bias.descriptor() if bias is not None else (None, None)
+        act = ActivationType.identity if activation is None else activation
+        name = ctypes.create_string_buffer(64)
+        st = native.lib().srtMatmulTune(a_ptr, ctypes.byref(ad), int(transpose_lhs), b_ptr, ctypes.byref(bd),
+                                        int(transpose_rhs), bias_ptr,
+                                        ctypes.byref(biasd) if bias is not None else None, int(act), float(coef),
+                                        o_ptr, ctypes.byref(od), self.stream, name, 64)
+        del ka, kb, ko, kbias
+        check(st, "srtMatmulTune")
+        return name.value.decode()
+
     # -- element-wise neighbours of the path ----------------------------------------------------
     def _elementwise(self, name, lhs, rhs, out):
         """Role of CudaQueue.add / mul / max ... (platform/cuda/functions/CudaMath.swift:93-150):
@@ -317,3 +340,27 @@ class using:
     def __exit__(self, *exc):
         HipPlatform.local().queue_stack.pop()
         return False
+
+
+class PlanCache:
+    """The native module's process-wide matmul plan cache (role of ExecutionPlanCache,
+    platform/common/ExecutionPlanner.swift:20-23): filled by HipQueue.tune_matmul, consulted by every
+    matmul, persisted as a small text file."""
+
+    @staticmethod
+    def clear():
+        check(native.lib().srtPlanCacheClear(), "srtPlanCacheClear")
+
+    @staticmethod
+    def count():
+        n = ctypes.c_size_t(0)
+        check(native.lib().srtPlanCacheCount(ctypes.byref(n)), "srtPlanCacheCount")
+        return n.value
+
+    @staticmethod
+    def save(path):
+        check(native.lib().srtPlanCacheSave(str(path).encode()), "srtPlanCacheSave")
+
+    @staticmethod
+    def load(path):
+        check(native.lib().srtPlanCacheLoad(str(path).encode()), "srtPlanCacheLoad")

@@ -126,3 +126,47 @@ extension HipQueue {
     hipCheck(status)
   }
 }
+
+//==============================================================================
+/// HipMatmul2: the retained-operation form (role of CudaMatmul2, CudaMatmul.swift:63-120, whose
+/// `tune` is empty).  The first forward for a shape asks the native module to measure every kernel
+/// plan the problem qualifies for; the winner is recorded in the module's plan cache under the
+/// shape / layout / epilogue key, so this and every later matmul with that key run it.
+public final class HipMatmul2<E>: DeviceMatmul2<E>
+where E: StorageElement, E.Value: StorageElement & Numeric {
+  public let queue: HipQueue
+  public var tunedShapes = Set<[Int]>()
+
+  @inlinable public init(queue: HipQueue) { self.queue = queue }
+
+  @inlinable public override func forward(
+    _ lhs: TensorR2<E>, _ transposeLhs: Bool,
+    _ rhs: TensorR2<E>, _ transposeRhs: Bool,
+    _ result: inout TensorR2<E>
+  ) {
+    let key = [lhs.shape[0], lhs.shape[1], rhs.shape[0], rhs.shape[1], transposeLhs ? 1 : 0, transposeRhs ? 1 : 0]
+    if tunedShapes.insert(key).inserted {
+      tune(lhs, transposeLhs, rhs, transposeRhs, &result)     // leaves `result` computed
+    } else {
+      queue.matmul(lhs, transposeLhs, rhs, transposeRhs, &result)
+    }
+  }
+
+  @inlinable public func tune(
+    _ lhs: TensorR2<E>, _ transposeLhs: Bool,
+    _ rhs: TensorR2<E>, _ transposeRhs: Bool,
+    _ result: inout TensorR2<E>
+  ) {
+    var name = [CChar](repeating: 0, count: 64)
+    let status = result.withMutableTensor(using: queue) { o, oDesc in
+      lhs.withTensor(using: queue) { a, aDesc in
+        rhs.withTensor(using: queue) { b, bDesc in
+          srtMatmulTune(a, aDesc, transposeLhs ? 1 : 0, b, bDesc, transposeRhs ? 1 : 0, nil, nil,
+                        srtActivationIdentity, 0, o, oDesc, queue.stream, &name, 64)
+        }
+      }
+    }
+    HipPlatform.cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
+    queue.diagnostic(.queueGpu, "matmul plan: \(String(cString: name))", categories: .queueGpu)
+  }
+}

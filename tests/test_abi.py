@@ -139,6 +139,43 @@ def test_repeating_views_and_gradient_table_shapes():
     assert srt.Tensor(np.zeros(2, np.uint16)).element_storage(float("nan"))[0] == 0x7FFF
 
 
+def test_plan_cache_file_round_trip_and_rejects_malformed_files(tmp_path):
+    """Save / Load of the plan cache are host-only: a plan written by hand is loaded, counted, saved
+    back identically; unknown plan names, short lines and missing files change nothing."""
+    srt.PlanCache.clear()
+    assert srt.PlanCache.count() == 0
+    good = tmp_path / "plans.txt"
+    good.write_text("# comment\n14 2048 2048 2048 1 89 10 mfma_256x256\n0 512 512 512 1 89 10 f32_mfma_splitk\n")
+    srt.PlanCache.load(good)
+    assert srt.PlanCache.count() == 2
+    out = tmp_path / "saved.txt"
+    srt.PlanCache.save(out)
+    lines = [ln for ln in out.read_text().splitlines() if not ln.startswith("#")]
+    assert sorted(lines) == sorted(["14 2048 2048 2048 1 89 10 mfma_256x256", "0 512 512 512 1 89 10 f32_mfma_splitk"])
+    for text in ("14 2048 2048 2048 1 89 10 no_such_plan\n", "14 2048 2048\n", "14 64 64 64 1 89 10 generic\nx y z\n"):
+        bad = tmp_path / "bad.txt"
+        bad.write_text(text)
+        with pytest.raises(srt.SrtError):
+            srt.PlanCache.load(bad)
+        assert srt.PlanCache.count() == 2                       # all or nothing
+    with pytest.raises(srt.SrtError):
+        srt.PlanCache.load(tmp_path / "missing.txt")
+    # a loaded plan steers the (GPU-free) kernel query for that key; clearing restores the heuristic
+    ad, k1 = native.make_descriptor(native.REAL16BF, (2048, 2048), (2048, 1), native.ORDER_ROW)
+    buf = ctypes.create_string_buffer(64)
+    dummy = ctypes.c_void_p(4096)
+    L = native.lib()
+    assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
+                                  buf, 64) == 0
+    assert buf.value == b"mfma_256x256"
+    srt.PlanCache.clear()
+    assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
+                                  buf, 64) == 0
+    assert buf.value == b"mfma_128x128"
+    assert L.srtPlanCacheCount(None) == native.ERROR_INVALID_VALUE
+    assert L.srtPlanCacheLoad(None) == native.ERROR_INVALID_VALUE
+
+
 def test_kernel_selection_is_queryable_without_gpu():
     L = native.lib()
 

@@ -1,0 +1,119 @@
+"""GPU tests of the plan / tune cache: srtMatmulTune measures every kernel plan a problem qualifies
+for, records the fastest, and later matmuls with the same key run it; every plan computes the same
+product (bit-exact on integer-valued inputs)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import swiftrt_amd as srt
+from swiftrt_amd import native
+from tests import helpers as H
+from tests.test_gpu_matmul import query_kernel
+
+pytestmark = pytest.mark.gpu
+
+PLANS_16 = {"mfma_256x256", "mfma_128x128", "mfma_64x64", "skinny", "generic"}
+PLANS_32 = {"f32_mfma_64x64", "f32_mfma_splitk", "generic"}
+
+
+@pytest.fixture(autouse=True)
+def clean_cache():
+    srt.PlanCache.clear()
+    yield
+    srt.PlanCache.clear()
+
+
+def int_operands(seed, m, k, n, dt, ta=False, tb=False):
+    g = H.rng(seed)
+    a = H.encode(g.integers(-4, 5, (k, m) if ta else (m, k)).astype(np.float32), dt)
+    b = H.encode(g.integers(-4, 5, (n, k) if tb else (k, n)).astype(np.float32), dt)
+    return a, b
+
+
+@pytest.mark.parametrize("dt,m,k,n,ta,tb", [(H.BF16, 1024, 64, 1024, False, False), (H.F16, 512, 32, 768, True, False),
+                                            (H.BF16, 8, 128, 2048, False, True), (H.F32, 256, 64, 256, False, False)])
+def test_tune_records_a_plan_and_later_calls_use_it(dt, m, k, n, ta, tb):
+    a_st, b_st = int_operands(41, m, k, n, dt, ta, tb)
+    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+    q = srt.current_queue()
+    # integer sums below 2^24 are exact in fp32 in any order; the store rounds once to the element type
+    exact = H.to64(a_st.T if ta else a_st) @ H.to64(b_st.T if tb else b_st)
+    want = H.to64(H.encode(exact.astype(np.float32), dt))
+    heuristic = srt.matmul(a, b, ta, tb)
+    assert np.array_equal(H.to64(heuristic.array()), want)
+    out = srt.Tensor(shape=[m, n], dtype=a.dtype)
+    chosen = q.tune_matmul(a, ta, b, tb, out)
+    assert chosen in (PLANS_32 if dt == H.F32 else PLANS_16)
+    assert srt.PlanCache.count() == 1
+    assert np.array_equal(H.to64(out.array()), want)                            # `out` was left by the chosen plan
+    name = query_kernel(a, ta, b, tb, out)
+    assert name == chosen or (name == "f32_mfma" and chosen.startswith("f32_mfma"))
+    again = srt.matmul(a, b, ta, tb)                                            # runs the cached plan
+    assert np.array_equal(H.to64(again.array()), want)
+    # another shape is not affected
+    a2, b2 = int_operands(42, m, k + 8, n, dt, ta, tb)
+    srt.matmul(srt.Tensor(a2), srt.Tensor(b2), ta, tb)
+    assert srt.PlanCache.count() == 1
+
+
+def test_every_plan_is_the_same_function(tmp_path):
+    """Forces each 16-bit plan in turn through a hand-written cache file and compares the products:
+    bit-exact on integers, and within one bf16 rounding of each other on normal data."""
+    m = k = n = 512
+    a_st, b_st = int_operands(43, m, k, n, H.BF16)
+    g = H.rng(44)
+    ar = H.encode((g.standard_normal((m, k)) / np.sqrt(k)).astype(np.float32), H.BF16)
+    br = H.encode(g.standard_normal((k, n)).astype(np.float32), H.BF16)
+    want = H.to64(H.encode((H.to64(a_st) @ H.to64(b_st)).astype(np.float32), H.BF16))
+    results = {}
+    for plan in ("mfma_256x256", "mfma_128x128", "mfma_64x64", "generic"):
+        f = tmp_path / f"{plan}.txt"
+        f.write_text(f"14 {m} {n} {k} 1 89 10 {plan}\n")
+        srt.PlanCache.clear()
+        srt.PlanCache.load(f)
+        a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+        c = srt.matmul(a, b)
+        assert query_kernel(a, False, b, False, c) == plan
+        assert np.array_equal(H.to64(c.array()), want), plan
+        results[plan] = H.to64(srt.matmul(srt.Tensor(ar), srt.Tensor(br)).array())
+    c64 = H.to64(ar) @ H.to64(br)
+    for plan, r in results.items():
+        assert H.max_norm_rel(r, c64) <= H.TOL[H.BF16], plan
+        assert np.max(np.abs(r - results["generic"]) / (np.abs(c64) + 1e-3)) <= 2 ** -6, plan
+
+
+def test_cached_plan_is_skipped_when_this_call_does_not_qualify(tmp_path):
+    """Alignment is not part of the key: a view that starts off a 16-byte boundary with the same
+    shape and layout class falls back to the heuristic (the generic kernel) instead of the cached
+    matrix-core plan."""
+    m = k = n = 256
+    f = tmp_path / "p.txt"
+    f.write_text(f"14 {m} {n} {k} 1 89 10 mfma_64x64\n")
+    srt.PlanCache.load(f)
+    g = H.rng(45)
+    big = H.encode(g.integers(-3, 4, (m, k + 8)).astype(np.float32), H.BF16)
+    b_st = H.encode(g.integers(-3, 4, (k, n)).astype(np.float32), H.BF16)
+    a_view = srt.Tensor(big)[:, 1:k + 1]                 # row pitch 264 (16-byte multiple), start misaligned by 2 bytes
+    c = srt.matmul(a_view, srt.Tensor(b_st))
+    exact = H.to64(big[:, 1:k + 1]) @ H.to64(b_st)
+    assert np.array_equal(H.to64(c.array()), H.to64(H.encode(exact.astype(np.float32), H.BF16)))
+
+
+def test_tune_errors():
+    q = srt.current_queue()
+    L = native.lib()
+    a = srt.Tensor(np.zeros((4, 8), np.float32))
+    b = srt.Tensor(np.zeros((9, 4), np.float32))
+    o = srt.Tensor(shape=[4, 4], dtype=np.float32)
+    ad, k1 = a.descriptor()
+    bd, k2 = b.descriptor()
+    od, k3 = o.descriptor()
+    name = ctypes.create_string_buffer(16)
+    assert L.srtMatmulTune(a.device_read(q), ctypes.byref(ad), 0, b.device_read(q), ctypes.byref(bd), 0, None, None, 5,
+                           0.0, o.device_read_write(q), ctypes.byref(od), q.stream, name, 16) == native.ERROR_INVALID_VALUE
+    ad.type = bd.type = od.type = native.REAL64F
+    bd2, k4 = native.make_descriptor(native.REAL64F, (8, 4), (4, 1), native.ORDER_ROW)
+    assert L.srtMatmulTune(a.device_read(q), ctypes.byref(ad), 0, b.device_read(q), ctypes.byref(bd2), 0, None, None, 5,
+                           0.0, o.device_read_write(q), ctypes.byref(od), q.stream, name, 16) == native.ERROR_NOT_SUPPORTED
+    assert srt.PlanCache.count() == 0
