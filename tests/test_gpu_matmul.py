@@ -148,6 +148,9 @@ def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, ke
     a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
     b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
     a_st, b_st = H.encode(a, dt), H.encode(b, dt)
+    # two k-contiguous operands take the 64-deep variant of the 256 x 256 kernel
+    if kernel == "mfma_256x256" and not ta and tb:
+        kernel = "mfma_256x256_k64"
     got = gpu_matmul(a_st, b_st, ta, tb, want_kernel=kernel)
     exact = (np.swapaxes(a, 0, 1) if ta else a).astype(np.int64) @ (np.swapaxes(b, 0, 1) if tb else b).astype(np.int64)
     assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
@@ -335,6 +338,51 @@ def test_ring_kernel_epilogues_vs_oracle(act, dt):
     want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, acc=ora.ACC_F32, fused=True))
     tol = {H.F16: 2.0 ** -10, H.BF16: 2.0 ** -7}[dt]
     assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("act", list(srt.ActivationType))
+def test_k64_kernel_epilogues_vs_oracle(act, dt):
+    """y = act(x . W^T + b) with W stored [N, K] (both operands k-contiguous): every activation through
+    the 64-deep 256 x 256 kernel; ragged M / N edges and a K that ends inside a stage."""
+    r = H.rng(17)
+    M, N, K = 3600, 3592, 200
+    x = H.encode(r.standard_normal((M, K)).astype(np.float32), dt)
+    w = H.encode((r.standard_normal((N, K)) / 8).astype(np.float32), dt)
+    b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
+    coef = 0.75
+    xt, wt, bt = srt.Tensor(x), srt.Tensor(w), srt.Tensor(b)
+    out = srt.Tensor(shape=[M, N], dtype=x.dtype)
+    assert query_kernel(xt, False, wt, True, out) == "mfma_256x256_k64"
+    srt.current_queue().matmul(xt, False, wt, True, out, bias=bt, activation=act, coef=coef)
+    got = H.decode(out.array())
+    rows = np.concatenate([np.arange(0, M, 211), [M - 1]])
+    want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, transpose_w=True,
+                                      acc=ora.ACC_F32, fused=True))
+    tol = {H.F16: 2.0 ** -10, H.BF16: 2.0 ** -7}[dt]
+    assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
+
+
+def test_k64_kernel_batched_short_k_and_nan():
+    """Strided batch, K shorter than one stage (8) and of one, two and three stages, a NaN row."""
+    r = H.rng(18)
+    for K in (8, 64, 72, 136, 192):
+        B_, M, N = 3, 2048, 2056
+        a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+        w = r.integers(-3, 4, (B_, N, K)).astype(np.float32)
+        at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+        out = srt.matmul(at, wt, transposed_rhs=True)
+        assert query_kernel(at, False, wt, True, out) == "mfma_256x256_k64"
+        exact = a.astype(np.int64) @ np.swapaxes(w, 1, 2).astype(np.int64)
+        assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), H.BF16)), K
+    a = np.zeros((3584, 64), np.float32)
+    w = np.zeros((3584, 64), np.float32)
+    a[:, 0] = 1.0
+    w[:, 0] = 2.0
+    a[5, 1] = np.nan
+    w[:, 1] = 1.0
+    got = gpu_matmul(H.encode(a, H.BF16), H.encode(w, H.BF16), tb=True, want_kernel="mfma_256x256_k64")
+    assert np.all(got[5] == 0x7FFF) and np.all(got[6] == H.encode(np.array([2.0], np.float32), H.BF16)[0])
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
