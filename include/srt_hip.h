@@ -149,8 +149,11 @@ srtStatus srtEventElapsedTime(float* milliseconds, srtEvent start, srtEvent stop
 /* Replace srtDeviceAllocate / srtDeviceFree, Modules/SwiftRTCuda/memory_api.h:26-27 (called
  * from CudaDeviceMemory, CudaDevice.swift:147,159).  Stream-ordered caching allocator: a
  * freed block is reused at once on the stream it was last used on, and on other streams once
- * the work queued on that stream at the time of the free has finished.  Thread safe.  The
- * caller owns the pointer; the library keeps no reference to tensor memory. */
+ * the work queued on that stream at the time of the free has finished.  "The stream it was used
+ * on" is the stream given to srtDeviceAllocate: a caller that also used the block on another
+ * stream orders that work before the free itself (event + srtStreamWaitEvent, as the storage layer
+ * does for cross-queue reads, DiscreteStorage.swift:271-296).  Thread safe.  The caller owns the
+ * pointer; the library keeps no reference to tensor memory. */
 srtStatus srtDeviceAllocate(void** devPtr, size_t size, srtStream stream);
 srtStatus srtDeviceFree(void* devPtr);
 /* Returns every cached (free) block of every device to the driver. */
@@ -265,8 +268,8 @@ srtStatus srtPlanCacheLoad(const char* path);
  * MathDerivatives.swift:460-482).
  * y, dy, dx: rank 2, [M, N], one element type (32F, 16F, 16BF), any strides; dbias: rank 1, N
  * elements.  Sums are fp32 in a fixed order (results do not vary from run to run).
- * May allocate a stream-ordered workspace of at most about 4096 x 64 x 16 bytes from the library's
- * allocator.  srtErrorNotSupported for other ranks or element types. */
+ * With dbias, takes a stream-ordered workspace of at most max(8 MiB, 4 N bytes) from the library's
+ * allocator for the duration of the call's kernels.  srtErrorNotSupported for other ranks or element types. */
 srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yDesc,
                                     const void* dy, const srtTensorDescriptor* dyDesc,
                                     srtActivation activation, double coef,

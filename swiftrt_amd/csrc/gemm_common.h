@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/srt_hip.h"
 
 namespace srt {
@@ -134,6 +136,19 @@ struct Epilogue {
     return T::from_float(v);
   }
 };
+
+// Raises a kernel's dynamic-LDS limit above the 64 KiB default, once per device (the attribute
+// belongs to the kernel's image on the current device).  `done` holds one bit per device.
+inline hipError_t ensure_lds_limit(const void* kernel, int bytes, std::atomic<uint32_t>& done) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  const uint32_t bit = 1u << (device & 31);
+  if (done.load(std::memory_order_relaxed) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_relaxed);
+  return e;
+}
 
 // ---- launchers (one per kernel family), defined in the .hip files ------------------------
 // Each returns hipSuccess/hip error from the launch; `name` receives the kernel family.

@@ -276,13 +276,9 @@ hipError_t launch_one(const GemmProblem& p, hipStream_t stream) {
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROW_BYTES;
   auto kernel = gemm_mfma_kernel<T, BM, BN, A_KC, B_KC>;
   if (lds_bytes > 64 * 1024) {
-    static bool configured = false;  // benign race: the attribute is idempotent
-    if (!configured) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-      if (e != hipSuccess) return e;
-      configured = true;
-    }
+    static std::atomic<uint32_t> configured{0};
+    if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), (int)lds_bytes, configured); e != hipSuccess)
+      return e;
   }
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);

@@ -632,13 +632,8 @@ template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   auto kernel = gemm_ring_kernel<T, A_KC, B_KC, EPI, NS>;
   constexpr int lds_bytes = NS * STAGE;
-  static bool configured = false;   // benign race: setting the attribute twice is harmless
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);
   return hipGetLastError();

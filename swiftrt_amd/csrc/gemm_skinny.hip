@@ -215,13 +215,8 @@ template <typename T, int XR>
 hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
   auto kernel = gemm_skinny_kernel<T, XR>;
   constexpr int lds_bytes = SkinnyShape<XR>::LDS;
-  static bool configured = false;   // benign race: setting the attribute twice is harmless
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
   hipLaunchKernelGGL(kernel, dim3((p.N + 31) / 32, p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
   return hipGetLastError();
 }

@@ -29,6 +29,8 @@ struct Block {
   hipEvent_t ready;  // recorded at free time; null while live
 };
 
+const hipStream_t kNoStream = reinterpret_cast<hipStream_t>(~uintptr_t(0));   // matches no real stream
+
 size_t round_size(size_t n) {
   if (n < 512) return 512;
   if (n <= (size_t(1) << 20)) {  // up to 1 MiB: next power of two
@@ -101,15 +103,24 @@ class CachingAllocator {
       if (hipEventRecord(ev, blk.stream) != hipSuccess) { (void)hipEventDestroy(ev); ev = nullptr; }
     }
     if (!ev) {
-      // could not order the free: make it safe the slow way
+      // could not order the free (e.g. the stream no longer exists): make it safe the slow way
       (void)hipGetLastError();
-      (void)hipStreamSynchronize(blk.stream);
+      (void)hipDeviceSynchronize();
+      blk.stream = kNoStream;
     }
     if (prev != blk.device) (void)hipSetDevice(prev);
     blk.ready = ev;
     std::lock_guard<std::mutex> lock(mu_);
     free_.emplace(Key{blk.device, blk.size}, blk);
     return srtSuccess;
+  }
+
+  // A destroyed stream's handle value may be given to a new stream: cached blocks must not treat
+  // that new stream as "the stream I was last used on".
+  void forget_stream(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto& kv : free_)
+      if (kv.second.stream == stream) kv.second.stream = kNoStream;
   }
 
   srtStatus empty_cache() {
@@ -254,6 +265,7 @@ srtStatus srtStreamCreate(srtStream* stream) {
 
 srtStatus srtStreamDestroy(srtStream stream) {
   if (!stream) return srtSuccess;
+  allocator().forget_stream(hs(stream));
   return from_hip(hipStreamDestroy(hs(stream)));
 }
 
