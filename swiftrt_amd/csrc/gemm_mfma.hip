@@ -364,13 +364,23 @@ int mfma_select(const GemmProblem& p) {
   const int layout = mfma_layout(p);
   if (layout < 0) return 0;
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
-  // Largest tile that still gives every CU work: 256 x 256 (ring kernel) from 192 tiles up, 128 x 128
-  // from one tile per CU up, otherwise 64 x 64 (measured on batch 32 x 256^3: 7.7 us against 15.0 us).
-  // With both operands k-contiguous the 64-deep variant of the 256 x 256 kernel moves whole cache
-  // lines where the ring kernel moves half lines (measured 8192^3: 1313 against 1277 TFLOP/s).
+  // Tile choice, from measurements over mid-size problems (1024^3 .. 4096 x 14336 x 4096):
+  //  * the 256 x 256 kernels are so much more efficient per tile (deep prefetch, 4x the arithmetic
+  //    intensity) that they win long before they can fill the device: from 48 tiles up for the
+  //    ring kernel (3072^3, 144 tiles: 64 us against 143 us with 128 x 128 tiles);
+  //  * with both operands k-contiguous the 64 x 64 kernel reads whole lines too and stays ahead up
+  //    to about 96 tiles of 256 x 256 (2048^3 NT: 36 us against 44 us); above that the 64-deep
+  //    256 x 256 kernel takes over (whole-line loads where the ring kernel moves half lines:
+  //    8192^3 NT 1313 against 1277 TFLOP/s);
+  //  * below those thresholds every CU should get a workgroup: 64 x 64 tiles (batch 32 x 256^3:
+  //    7.7 us against 15.0 us with 128 x 128).  128 x 128 is kept for problems that do not meet
+  //    the 256 x 256 kernels' preconditions but have at least one such tile per CU.
+  const bool big_ok = ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0);
+  const long long t256 = tiles(256);
   int tile;
-  if (tiles(256) >= 192 && ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) tile = layout == 3 ? 4 : 1;
-  else if (tiles(128) >= 256) tile = 2;
+  if (big_ok && layout == 3 && t256 >= 96) tile = 4;
+  else if (big_ok && layout != 3 && t256 >= 48) tile = 1;
+  else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
 }

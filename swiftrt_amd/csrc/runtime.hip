@@ -99,7 +99,8 @@ class CachingAllocator {
     (void)hipGetDevice(&prev);
     if (prev != blk.device) (void)hipSetDevice(blk.device);
     hipEvent_t ev = nullptr;
-    if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess) {
+    // a block whose stream has been destroyed cannot be ordered by an event on it
+    if (blk.stream != kNoStream && hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess) {
       if (hipEventRecord(ev, blk.stream) != hipSuccess) { (void)hipEventDestroy(ev); ev = nullptr; }
     }
     if (!ev) {
@@ -115,11 +116,15 @@ class CachingAllocator {
     return srtSuccess;
   }
 
-  // A destroyed stream's handle value may be given to a new stream: cached blocks must not treat
-  // that new stream as "the stream I was last used on".
+  // Called before a stream is destroyed.  Its handle value may be given to a new stream later, so
+  // cached blocks must not treat that stream as "the stream I was last used on"; and blocks still
+  // live on it can no longer record an event there when they are freed (they fall back to a
+  // device-wide synchronisation).
   void forget_stream(hipStream_t stream) {
     std::lock_guard<std::mutex> lock(mu_);
     for (auto& kv : free_)
+      if (kv.second.stream == stream) kv.second.stream = kNoStream;
+    for (auto& kv : live_)
       if (kv.second.stream == stream) kv.second.stream = kNoStream;
   }
 

@@ -145,13 +145,13 @@ def test_plan_cache_file_round_trip_and_rejects_malformed_files(tmp_path):
     srt.PlanCache.clear()
     assert srt.PlanCache.count() == 0
     good = tmp_path / "plans.txt"
-    good.write_text("# comment\n14 2048 2048 2048 1 89 10 mfma_256x256\n0 512 512 512 1 89 10 f32_mfma_splitk\n")
+    good.write_text("# comment\n14 2048 2048 2048 1 89 10 mfma_128x128\n0 512 512 512 1 89 10 f32_mfma_splitk\n")
     srt.PlanCache.load(good)
     assert srt.PlanCache.count() == 2
     out = tmp_path / "saved.txt"
     srt.PlanCache.save(out)
     lines = [ln for ln in out.read_text().splitlines() if not ln.startswith("#")]
-    assert sorted(lines) == sorted(["14 2048 2048 2048 1 89 10 mfma_256x256", "0 512 512 512 1 89 10 f32_mfma_splitk"])
+    assert sorted(lines) == sorted(["14 2048 2048 2048 1 89 10 mfma_128x128", "0 512 512 512 1 89 10 f32_mfma_splitk"])
     for text in ("14 2048 2048 2048 1 89 10 no_such_plan\n", "14 2048 2048\n", "14 64 64 64 1 89 10 generic\nx y z\n"):
         bad = tmp_path / "bad.txt"
         bad.write_text(text)
@@ -167,11 +167,11 @@ def test_plan_cache_file_round_trip_and_rejects_malformed_files(tmp_path):
     L = native.lib()
     assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
                                   buf, 64) == 0
-    assert buf.value == b"mfma_256x256"
+    assert buf.value == b"mfma_128x128"
     srt.PlanCache.clear()
     assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
                                   buf, 64) == 0
-    assert buf.value == b"mfma_128x128"
+    assert buf.value == b"mfma_256x256"
     assert L.srtPlanCacheCount(None) == native.ERROR_INVALID_VALUE
     assert L.srtPlanCacheLoad(None) == native.ERROR_INVALID_VALUE
 
@@ -195,6 +195,14 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 8192, 8192, 8192) == "mfma_256x256"
     assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256"
     assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256"
+    assert query(native.REAL16BF, 8192, 8192, 8192, tb=True) == "mfma_256x256_k64"   # both operands k-contiguous
+    # mid-size problems: the 256 x 256 kernels from 48 tiles up (96 when both operands are k-contiguous),
+    # 64 x 64 tiles below, so that every CU gets a workgroup
+    assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256"                 # 144 tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_256x256"                 # 64 tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_64x64"
+    assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_64x64"                    # 32 tiles
+    assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 33, 33, 33) == "generic"

@@ -142,8 +142,16 @@ def test_integer_inputs_bit_exact_vs_oracle(dt, ta, tb):
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("M,N,K,kernel", [(200, 264, 72, "mfma_64x64"), (2040, 2056, 136, "mfma_128x128"),
                                           (4000, 3976, 200, "mfma_256x256")])
-def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, kernel):
+def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, kernel, tmp_path):
     """Aligned shapes with ragged edges in M, N and K, every tile config and staging layout."""
+    if kernel == "mfma_128x128":
+        # the heuristic reaches this tile only when the 256 x 256 kernels' preconditions fail: pin it
+        # for this shape through the plan cache instead
+        layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
+        f = tmp_path / "plan.txt"
+        f.write_text(f"{dt} {M} {N} {K} 1 {layout} 10 mfma_128x128\n")
+        srt.PlanCache.clear()
+        srt.PlanCache.load(f)
     r = H.rng(100 + M)
     a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
     b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
@@ -158,6 +166,25 @@ def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, ke
     b = r.standard_normal(b.shape).astype(np.float32)
     a_st, b_st = H.encode(a, dt), H.encode(b, dt)
     check_against_fp64(gpu_matmul(a_st, b_st, ta, tb), a_st, b_st, ta, tb, dt)
+    srt.PlanCache.clear()
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_result_view_with_odd_pitch_takes_the_128_tile(dt):
+    """A result that is a view with a row pitch that is not a multiple of 8 elements cannot take the
+    256 x 256 kernels' 16-byte stores; with one 128 x 128 tile per CU or more that tile runs."""
+    r = H.rng(19)
+    M, N, K = 2048, 2048, 72
+    a = r.integers(-3, 4, (M, K)).astype(np.float32)
+    b = r.integers(-3, 4, (K, N)).astype(np.float32)
+    at, bt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(b, dt))
+    big = srt.Tensor(shape=[M, N + 4], dtype=at.dtype)
+    out = big[:, :N]
+    assert query_kernel(at, False, bt, False, out) == "mfma_128x128"
+    srt.current_queue().matmul(at, False, bt, False, out)
+    exact = a.astype(np.int64) @ b.astype(np.int64)
+    assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt))
+    assert np.all(H.decode(big.array()[:, N:]) == 0)          # the padding columns are untouched
 
 
 @pytest.mark.parametrize("dt", DTS)
