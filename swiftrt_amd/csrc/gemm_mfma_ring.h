@@ -42,6 +42,8 @@
 #pragma once
 #include "gemm_common.h"
 
+#include <type_traits>
+
 namespace srt {
 namespace ring {
 
@@ -109,11 +111,10 @@ __device__ __forceinline__ void load_to_lds_at_m0(u32x4_t rsrc, uint32_t voff, u
 
 // ---- global -> LDS ---------------------------------------------------------------------------
 // Per-lane byte offsets (into the operand's buffer) of the 4 loads a wave issues per stage for
-// one operand; the k advance goes through the scalar offset.
+// one operand; the tile's position and the k advance go through the scalar offset.
 template <bool KC>
 struct Loader {
   uint32_t voff[4];
-  uint32_t kstep;   // bytes per k stage
 
   // tile_row0: first m (or n) of the tile.  ld: elements between rows (KC) or between k (MN).
   __device__ __forceinline__ void init(int wave, int lane, int tile_row0, long long ld) {
@@ -125,7 +126,6 @@ struct Loader {
         const int chunk = (lane & 3) ^ ((row >> 2) & 3);
         voff[i] = (uint32_t)(((long long)(tile_row0 + row) * ld + chunk * 8) * 2);
       }
-      kstep = BK * 2;
     } else {
       // load i covers k rows (wave*4 + i)*2 .. +1, 32 lanes per 512-byte k row
 #pragma unroll
@@ -134,36 +134,37 @@ struct Loader {
         const int chunk = (lane & 31) ^ ((krow & 3) << 2);
         voff[i] = (uint32_t)(((long long)krow * ld + tile_row0 + chunk * 8) * 2);
       }
-      kstep = (uint32_t)(BK * ld * 2);
     }
   }
 
-  // Load i of this wave for the k stage at scalar byte offset `soff` (stage * kstep, or OOB to
-  // make the whole load read zeros without touching memory), into the operand region at LDS
-  // address `region`.  `tail`: this is a ragged last stage; for a k-contiguous operand the
-  // logical chunks >= mask_from lie at or beyond K and must read as zero (an mn-contiguous
-  // operand gets that from the bounds check, its k rows >= K being past the end of the view).
+  // Load i of this wave for the k stage at scalar byte offset `soff` (tile offset + stage * kstep,
+  // or OOB to make the whole load read zeros without touching memory), into the operand region
+  // at LDS address `region`.  `tail`: this is a ragged last stage holding only `krem` (< BK) k
+  // values; what lies at or beyond K must read as zero: for a k-contiguous operand the logical
+  // 16-byte chunks >= ceil(krem / 8) of every row, for an mn-contiguous one the k rows >= krem.
   __device__ __forceinline__ void issue_one(u32x4_t rsrc, uint32_t region, int wave, int lane, uint32_t soff, int i,
-                                            bool tail, int mask_from) const {
+                                            bool tail, int krem) const {
     uint32_t v = voff[i];
-    if (KC) {
-      // (row >> 2) & 3 of the row this lane fetches does not depend on i or the wave
-      const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
-      v = (tail && chunk >= mask_from) ? OOB : v;
-    }
+    if (tail && beyond_k(wave, lane, i, krem)) v = OOB;
     load_to_lds(rsrc, region + (uint32_t)(wave * 4 + i) * 1024u, v, soff);
   }
 
-  // Permanently aim the chunks at or beyond K out of range (called once, just before the loads
-  // of a ragged last stage are issued; every later load is out of range as a whole anyway).
-  __device__ __forceinline__ void mask_tail(int lane, int mask_from) {
+  // does load i of this lane fetch k values at or beyond K in a ragged last stage of krem values?
+  __device__ __forceinline__ bool beyond_k(int wave, int lane, int i, int krem) const {
     if (KC) {
+      // (row >> 2) & 3 of the row this lane fetches does not depend on i or the wave
       const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
-      if (chunk >= mask_from) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) voff[i] = OOB;
-      }
+      return chunk >= (krem + 7) / 8;
     }
+    return (wave * 4 + i) * 2 + (lane >> 5) >= krem;
+  }
+
+  // Aim what lies at or beyond K out of range for good (called just before the loads of a ragged
+  // last stage are issued; the per-lane state is derived afresh for the next tile).
+  __device__ __forceinline__ void mask_tail(int wave, int lane, int krem) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (beyond_k(wave, lane, i, krem)) voff[i] = OOB;
   }
 };
 
@@ -234,7 +235,20 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
   *tn = in_group / gsize;
 }
 
+
 #define SRT_FENCE() __builtin_amdgcn_sched_barrier(0)
+// An empty statement that "rewrites" an accumulator tile in the accumulator registers.  After an
+// MFMA it ties the MFMA to its place in the instruction stream (MFMAs have no side effects;
+// without this the compiler is free to gather them elsewhere).  In the epilogue it ends the life
+// of the copies the compiler makes in ordinary registers to test or convert accumulators, which
+// it would otherwise keep -- and spill -- until their next use.
+__device__ __forceinline__ void pin(f32x16_t& acc) { asm volatile("" : "+a"(acc)); }
+__device__ __forceinline__ void pin_all(f32x16_t (&acc)[4][4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pin(acc[i][j]);
+}
 
 // Epilogue of one wave.
 // acc[i][j] is a transposed 32 x 32 tile: lane l owns row m = wave_m0 + 32 i + l % 32 and, in
@@ -260,7 +274,7 @@ __device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = wave_m0 + 32 * i + r;
-      brow[i] = (per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+      brow[i] = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
     }
   }
   bool nan = false;
@@ -273,7 +287,7 @@ __device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
-          bcol[e] = (!per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+          bcol[e] = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
         }
       }
 #pragma unroll
@@ -419,9 +433,41 @@ constexpr int EPI_BIAS_RELU = 3;   // bias, relu (the Dense configuration)
 constexpr int EPI_CLIPPED = 4;     // clippedRelu, bias optional (a null bias adds nothing)
 constexpr int EPI_TRANS = 5;       // sigmoid / tanh / elu (+ bias)
 
+// One tile as the loads see it: the byte offsets of its first row (column) inside the operand
+// tensors, batch offset included.  All scalar.
+struct TileRef {
+  uint32_t offa, offb;
+  int m0, n0, bz;
+};
+
+template <bool A_KC, bool B_KC>
+__device__ __forceinline__ TileRef locate_tile(const GemmProblem& p, int v, int tiles_m, int tiles_n) {
+  const int per_batch = tiles_m * tiles_n;
+  const int bz = v / per_batch;
+  int tm, tn;
+  tile_coords(v - bz * per_batch, tiles_m, tiles_n, &tm, &tn);
+  TileRef t;
+  t.m0 = tm * BM;
+  t.n0 = tn * BN;
+  t.bz = bz;
+  const long long lda = A_KC ? p.sam : p.sak;
+  const long long ldb = B_KC ? p.sbn : p.sbk;
+  t.offa = (uint32_t)(((long long)bz * p.sab + (A_KC ? (long long)t.m0 * lda : (long long)t.m0)) * 2);
+  t.offb = (uint32_t)(((long long)bz * p.sbb + (B_KC ? (long long)t.n0 * ldb : (long long)t.n0)) * 2);
+  return t;
+}
+
+// The kernel is persistent: the grid has one workgroup per compute unit (or per tile when there
+// are fewer tiles), and workgroup w computes tiles w, w + G, w + 2 G, ... of the XCD-aware order.
+// The k loop runs across tile boundaries: while the last stages of a tile are multiplied, the
+// ring slots they vacate receive the first NS - 2 stages of the workgroup's next tile, so that
+// tile starts with its operands already in LDS; the two slots vacated last are the epilogue's
+// staging area, and the remaining stages of the next tile's ring are requested right after the
+// epilogue.  With a ragged last k stage or fewer than NS stages the overlap is off and the next
+// tile starts from a full prologue.
 template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
-  static_assert(NS >= 3 && NS <= 5, "ring depth");
+  static_assert(NS == 5, "ring depth");   // slot arithmetic below assumes the staging slots are NS-2, NS-1 ahead
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
 
@@ -431,42 +477,26 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
   const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
 
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  int tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, &tm, &tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int bz = blockIdx.y;
+  const int total = tiles_m * tiles_n * p.batch;
+  const int grid = (int)gridDim.x;
+  int v = (int)blockIdx.x;
 
-  const uint16_t* A = (const uint16_t*)p.A + (long long)bz * p.sab;
-  const uint16_t* B = (const uint16_t*)p.B + (long long)bz * p.sbb;
   const long long lda = A_KC ? p.sam : p.sak;
   const long long ldb = B_KC ? p.sbn : p.sbk;
-  // bytes spanned by each operand view: anything beyond reads as zero
-  const uint32_t a_bytes = (uint32_t)((A_KC ? (long long)(p.M - 1) * lda + p.K : (long long)(p.K - 1) * lda + p.M) * 2);
-  const uint32_t b_bytes = (uint32_t)((B_KC ? (long long)(p.N - 1) * ldb + p.K : (long long)(p.K - 1) * ldb + p.N) * 2);
-  const u32x4_t ra = make_rsrc(A, a_bytes);
-  const u32x4_t rb = make_rsrc(B, b_bytes);
-
-  Loader<A_KC> la;
-  Loader<B_KC> lb;
-  la.init(wave, lane, m0, lda);
-  lb.init(wave, lane, n0, ldb);
-  FragReader<A_KC> fa;
-  FragReader<B_KC> fb;
-  fa.init(lane, wm0);
-  fb.init(lane, wn0);
-
-  // acc[i][j] is the transposed 32 x 32 tile: m = 32 i + lane % 32, n = 32 j + 8 (v/4) + 4 (lane/32) + v % 4
-  f32x16_t acc[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
+  // One descriptor per operand, spanning the views of all batches: anything beyond the last
+  // batch's view reads as zero.  Inside the tensor nothing is masked by the descriptor: rows of a
+  // partial tile beyond M (columns beyond N) read whatever follows and only reach accumulators
+  // that are never stored; k beyond K is masked by the loaders (ragged last stage).
+  const long long a_view = A_KC ? (long long)(p.M - 1) * lda + p.K : (long long)(p.K - 1) * lda + p.M;
+  const long long b_view = B_KC ? (long long)(p.N - 1) * ldb + p.K : (long long)(p.K - 1) * ldb + p.N;
+  const u32x4_t ra = make_rsrc(p.A, (uint32_t)(((long long)(p.batch - 1) * p.sab + a_view) * 2));
+  const u32x4_t rb = make_rsrc(p.B, (uint32_t)(((long long)(p.batch - 1) * p.sbb + b_view) * 2));
+  const uint32_t kstep_a = A_KC ? (uint32_t)(BK * 2) : (uint32_t)(BK * lda * 2);   // bytes per k stage
+  const uint32_t kstep_b = B_KC ? (uint32_t)(BK * 2) : (uint32_t)(BK * ldb * 2);
   const int KT = (p.K + BK - 1) / BK;
-  // first logical 16-byte chunk of the last k stage that lies at or beyond K (4 = stage is whole)
-  const int tail_mask = (p.K % BK) ? ((p.K % BK) + 7) / 8 : 4;
+  const int krem = p.K % BK;   // k values in a ragged last stage (0: the stage is whole)
+  const bool ragged = krem != 0;
+  const bool overlap = !ragged && KT >= NS;
 
   // With A stored k x m (transposed lhs) the k stages are walked in rotated order, starting at a
   // stage that depends on the XCD the workgroup runs on (its id mod 8): k rows of A are a power
@@ -477,155 +507,273 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
   // last-level cache reuse between XCDs outweighs the channel spread (measured -3 % rotated).
   // (Summation order changes with the start; the result is still one fp32 accumulation per
   // element.)  Not applied when the last stage is ragged.
-  const int rot = (A_KC || tail_mask < 4) ? 0 : (int)(((unsigned)(blockIdx.x & 7) * (unsigned)KT) / 8u);
+  const int rot = (A_KC || ragged) ? 0 : (int)(((unsigned)(blockIdx.x & 7) * (unsigned)KT) / 8u);
   auto stage_at = [&](int t) {   // t-th stage of the walk (t < KT)
     int e = t + rot;
     if (e >= KT) e -= KT;
     return e;
   };
 
-  // ---- prologue: fill the ring (stages 0 .. NS-2 and the A part of stage NS-1; its B part is
-  //      the first thing the loop requests), wait for stage 0 only ----
-#pragma unroll
-  for (int t = 0; t < NS; ++t) {
-    const uint32_t slot = lds + (uint32_t)t * STAGE;
-    const bool tail = (t == KT - 1) && tail_mask < 4;
-    const uint32_t soa = t < KT ? (uint32_t)stage_at(t) * la.kstep : OOB;
-    const uint32_t sob = t < KT ? (uint32_t)stage_at(t) * lb.kstep : OOB;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) la.issue_one(ra, slot, wave, lane, soa, i, tail, tail_mask);
-    if (t < NS - 1) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) lb.issue_one(rb, slot + REGION, wave, lane, sob, i, tail, tail_mask);
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(8 * (NS - 2) + 4) : "memory");
-  SRT_FENCE();
+  TileRef cur_tile = locate_tile<A_KC, B_KC>(p, v, tiles_m, tiles_n);
 
-  u32x4_t af[2][4], bf[2][4];   // [k slice][32-wide tile]
+  // Requests stages first .. NS-2 of `tile` and the A part of stage NS-1 (its B part is the first
+  // thing the loop requests); stage t goes to the slot t places after `slot0`.
+  auto fill_ring = [&](const Loader<A_KC>& la, const Loader<B_KC>& lb, const TileRef& tile, uint32_t slot0, int first) {
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    af[0][t] = fa.read(lds, t, 0);
-    bf[0][t] = fb.read(lds + REGION, t, 0);
-  }
-
-  // The loop body is branch-free: loads past the last stage are aimed out of range (they return
-  // zeros without touching memory and land in a slot nobody reads again), and the reads of
-  // "stage KT" in the last trip fetch LDS contents that are never used.
-  // Loop-carried scalars: LDS slots of stage kt-1 (prv) and kt (cur), and the byte offsets of
-  // the stages being requested.  Loads of one stage are split over two phases: its A part in
-  // phase 1 of iteration kt (stage kt+NS into slot cur), its B part in phase 0 of iteration
-  // kt+1 (same stage, same slot, by then called prv).
-  uint32_t cur = lds, prv = lds + (NS - 1) * STAGE;
-  const bool ragged = tail_mask < 4;
-  const uint32_t wave_lds = (uint32_t)wave * 4096u;   // this wave's 4 KiB share of an operand region
-  for (int kt = 0; kt < KT; ++kt) {
-    uint32_t nxt = cur + STAGE;
-    if (nxt == lds + NS * STAGE) nxt = lds;
-
-    // ---- phase 0: MFMAs of slice 0.  The eight fragment reads of slice 1 ride on the first
-    //      eight MFMAs so that they have returned by the time the barrier is reached; the B part
-    //      of stage kt-1+NS rides on the second eight. ----
-    const int kb = kt - 1 + NS;
-    const uint32_t sob = kb < KT ? (uint32_t)stage_at(kb) * lb.kstep : OOB;
-    if (ragged && kb == KT - 1) lb.mask_tail(lane, tail_mask);
-    const uint32_t b_target = prv + REGION + wave_lds;
+    for (int t = 0; t < NS; ++t) {
+      if (t < first) continue;
+      uint32_t slot = slot0 + (uint32_t)t * STAGE;
+      if (slot >= lds + NS * STAGE) slot -= NS * STAGE;
+      const bool tail = (t == KT - 1) && ragged;
+      const uint32_t soa = t < KT ? tile.offa + (uint32_t)stage_at(t) * kstep_a : OOB;
+      const uint32_t sob = t < KT ? tile.offb + (uint32_t)stage_at(t) * kstep_b : OOB;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 4; ++i) la.issue_one(ra, slot, wave, lane, soa, i, tail, krem);
+      if (t < NS - 1) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int u = i * 4 + j;   // 0..15
-        if (u == 8) set_lds_target<0>(b_target);
-        if (u == 10) set_lds_target<1024>(b_target);
-        if (u == 12) set_lds_target<2048>(b_target);
-        if (u == 14) set_lds_target<3072>(b_target);
-        if (u >= 8 && (u & 1) == 0) SRT_FENCE();
-        acc[i][j] = mfma<T>(bf[0][j], af[0][i], acc[i][j]);
-        if (u >= 8 && (u & 1) == 0) {
-          SRT_FENCE();
-          load_to_lds_at_m0(rb, lb.voff[(u - 8) >> 1], sob);
-        }
-        // order of first use in phase 1: a0 b0 b1 b2 b3 a1 a2 a3
-        if (u == 0) af[1][0] = fa.read(cur, 0, 1);
-        else if (u >= 1 && u <= 4) bf[1][u - 1] = fb.read(cur + REGION, u - 1, 1);
-        else if (u >= 5 && u <= 7) af[1][u - 4] = fa.read(cur, u - 4, 1);
-        SRT_FENCE();
+        for (int i = 0; i < 4; ++i) lb.issue_one(rb, slot + REGION, wave, lane, sob, i, tail, krem);
       }
     }
+  };
 
-    // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(8 * (NS - 2)) : "memory");
+  // Loop-carried scalars: LDS slots of stage kt-1 (prv) and kt (cur).  Loads of one stage are
+  // split over two phases: its A part in phase 1 of iteration kt (stage kt+NS into slot cur), its
+  // B part in phase 0 of iteration kt+1 (same stage, same slot, by then called prv).
+  uint32_t cur = lds, prv = lds + (NS - 1) * STAGE;
+  const uint32_t wave_lds = (uint32_t)wave * 4096u;   // this wave's 4 KiB share of an operand region
+
+  bool first_tile = true;
+  for (;;) {
+    // Per-lane addressing state, derived for every tile from a lane id the compiler cannot see
+    // through and scoped to the tile: none of it may stay live across the epilogue, which needs
+    // every register it can get for the 256 accumulators.
+    Loader<A_KC> la;
+    Loader<B_KC> lb;
+    FragReader<A_KC> fa;
+    FragReader<B_KC> fb;
+    {
+      int l = lane;
+      asm volatile("" : "+v"(l));
+      la.init(wave, l, 0, lda);
+      lb.init(wave, l, 0, ldb);
+      fa.init(l, wm0);
+      fb.init(l, wn0);
+    }
+    // ---- the tile's ring: everything for the first tile and without the overlap (wait for
+    //      stage 0 only); else stages 0 .. NS-3 landed before the previous epilogue ----
+    if (first_tile || !overlap) {
+      fill_ring(la, lb, cur_tile, cur, 0);
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(8 * (NS - 2) + 4) : "memory");
+    } else {
+      fill_ring(la, lb, cur_tile, cur, NS - 2);
+    }
+    first_tile = false;
     SRT_FENCE();
 
-    // ---- phase 1: MFMAs of slice 1; the A part of stage kt+NS goes into the slot just vacated
-    //      (even MFMAs 0..6), the reads of slice 0 of stage kt+1 ride on the odd MFMAs ----
-    const int ka = kt + NS;
-    const uint32_t soa = ka < KT ? (uint32_t)stage_at(ka) * la.kstep : OOB;
-    if (ragged && ka == KT - 1) la.mask_tail(lane, tail_mask);
-    const uint32_t a_target = cur + wave_lds;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int u = i * 4 + j;   // 0..15
-        if (u == 0) set_lds_target<0>(a_target);
-        if (u == 2) set_lds_target<1024>(a_target);
-        if (u == 4) set_lds_target<2048>(a_target);
-        if (u == 6) set_lds_target<3072>(a_target);
-        if (u < 8 && (u & 1) == 0) SRT_FENCE();
-        acc[i][j] = mfma<T>(bf[1][j], af[1][i], acc[i][j]);
-        if (u < 8 && (u & 1) == 0) {
-          SRT_FENCE();
-          load_to_lds_at_m0(ra, la.voff[u >> 1], soa);
-        }
-        if (u & 1) {
-          const int r = u >> 1;   // 0..7, same first-use order as above
-          if (r == 0) af[0][0] = fa.read(nxt, 0, 0);
-          else if (r <= 4) bf[0][r - 1] = fb.read(nxt + REGION, r - 1, 0);
-          else af[0][r - 4] = fa.read(nxt, r - 4, 0);
-        }
-        SRT_FENCE();
-      }
-    }
-    prv = cur;
-    cur = nxt;
-  }
-  // every load still in flight (all out of range by now, but still writing zeros into LDS) must
-  // retire, in every wave, before the LDS is reused as the epilogue's staging area
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  const uint32_t stage = lds + (uint32_t)wave * 16384u;
+    const int vn = v + grid;
+    const bool has_next = vn < total;
+    const TileRef next_tile = locate_tile<A_KC, B_KC>(p, has_next ? vn : v, tiles_m, tiles_n);
+    const bool prefetch = overlap && has_next;
 
-  // ---- epilogue ----
-  if (EPI == EPI_TRANS) {
-    store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
-  } else {
-    bool any_nan;
-    if (EPI == EPI_PLAIN) any_nan = any_nan_in_tile(acc);   // the accumulators are final as they are
-    else if (EPI == EPI_BIAS) any_nan = apply_linear_epilogue<T, true, 0>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_RELU) any_nan = apply_linear_epilogue<T, false, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_BIAS_RELU) any_nan = apply_linear_epilogue<T, true, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else any_nan = p.bias ? apply_linear_epilogue<T, true, 2>(p, acc, m0 + wm0, n0 + wn0, lane)
-                          : apply_linear_epilogue<T, false, 2>(p, acc, m0 + wm0, n0 + wn0, lane);
-    if (any_nan) store_tile<T, true>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
-    else store_tile<T, false>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+    // acc[i][j] is the transposed 32 x 32 tile: m = 32 i + lane % 32, n = 32 j + 8 (v/4) + 4 (lane/32) + v % 4
+    f32x16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    u32x4_t af[2][4], bf[2][4];   // [k slice][32-wide tile]
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      af[0][t] = fa.read(cur, t, 0);
+      bf[0][t] = fb.read(cur + REGION, t, 0);
+    }
+
+    // The loop body is branch-free.  A request past the tile's last stage is either a stage of
+    // the next tile (the first NS - 2 of them, when the overlap is on) or aimed out of range: it
+    // returns zeros without touching memory and lands in a slot nobody reads before it is
+    // refilled -- those requests are still issued so that the count of loads in flight, which
+    // the waits below rely on, is the same in every iteration.
+    // Request r (r-th stage counted from this tile's first) reads stage (r + rot) mod KT of its
+    // tile -- the same expression for this tile's stages and the next one's -- at the tile's
+    // base offset, through the tile's descriptor.  Iteration kt requests the A part of r = kt + NS
+    // in its phase 1 and iteration kt + 1 the B part of the same r in its phase 0, so the scalars
+    // of both are worked out together, in the shadow of phase 0's MFMAs, from a stage counter
+    // that is advanced by one per iteration (no multiplications, no branches).
+    const int limit = prefetch ? KT + NS - 2 : KT;   // requests below this index are real
+    auto stage_of = [&](int r) {
+      int e = r + rot;
+      e = e >= KT ? e - KT : e;
+      e = e >= KT ? e - KT : e;
+      return e;
+    };
+    uint32_t sob, soa = 0;
+    sob = NS - 1 < KT ? cur_tile.offb + (uint32_t)stage_of(NS - 1) * kstep_b : OOB;   // B part of r = NS - 1
+    int e_req = stage_of(NS);                                                         // stage of r = NS
+    uint32_t ea_off = (uint32_t)e_req * kstep_a, eb_off = (uint32_t)e_req * kstep_b;
+    // The loop exists twice: the copy for a ragged last k stage also aims the chunks at or beyond
+    // K out of range when that stage is requested (a dozen instructions per trip that the
+    // common case does without).
+    auto k_loop = [&](auto ragged_tag) {
+    constexpr bool RAGGED = decltype(ragged_tag)::value;
+    for (int kt = 0; kt < KT; ++kt) {
+      uint32_t nxt = cur + STAGE;
+      if (nxt == lds + NS * STAGE) nxt = lds;
+
+      // ---- phase 0: MFMAs of slice 0.  The eight fragment reads of slice 1 ride on the first
+      //      eight MFMAs so that they have returned by the time the barrier is reached; the B part
+      //      of stage kt-1+NS rides on the second eight. ----
+      const int kb = kt - 1 + NS;
+      const int ka = kt + NS;
+      uint32_t sob_next = OOB;
+      if (RAGGED) {   // the requests of this iteration that fetch the ragged last stage
+        if (kb == KT - 1) lb.mask_tail(wave, lane, krem);
+        if (ka == KT - 1) la.mask_tail(wave, lane, krem);
+      }
+      const uint32_t b_target = prv + REGION + wave_lds;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int u = i * 4 + j;   // 0..15
+          if (u == 8) set_lds_target<0>(b_target);
+          if (u == 10) set_lds_target<1024>(b_target);
+          if (u == 12) set_lds_target<2048>(b_target);
+          if (u == 14) set_lds_target<3072>(b_target);
+          if (u >= 8 && (u & 1) == 0) SRT_FENCE();
+          acc[i][j] = mfma<T>(bf[0][j], af[0][i], acc[i][j]);
+          pin(acc[i][j]);
+          if (u >= 8 && (u & 1) == 0) {
+            SRT_FENCE();
+            load_to_lds_at_m0(rb, lb.voff[(u - 8) >> 1], sob);
+          }
+          // order of first use in phase 1: a0 b0 b1 b2 b3 a1 a2 a3
+          if (u == 0) af[1][0] = fa.read(cur, 0, 1);
+          else if (u >= 1 && u <= 4) bf[1][u - 1] = fb.read(cur + REGION, u - 1, 1);
+          else if (u >= 5 && u <= 7) af[1][u - 4] = fa.read(cur, u - 4, 1);
+          // scalars of request r = ka (A part now, B part in the next iteration), a few per MFMA
+          if (u == 2) soa = ka < limit ? (ka < KT ? cur_tile.offa : next_tile.offa) + ea_off : OOB;
+          if (u == 3) sob_next = ka < limit ? (ka < KT ? cur_tile.offb : next_tile.offb) + eb_off : OOB;
+          if (u == 6) {
+            const bool wrap = e_req + 1 == KT;
+            e_req = wrap ? 0 : e_req + 1;
+            ea_off = wrap ? 0u : ea_off + kstep_a;
+            eb_off = wrap ? 0u : eb_off + kstep_b;
+          }
+          SRT_FENCE();
+        }
+      }
+
+      // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(8 * (NS - 2)) : "memory");
+      SRT_FENCE();
+
+      // ---- phase 1: MFMAs of slice 1; the A part of stage kt+NS goes into the slot just vacated
+      //      (even MFMAs 0..6), the reads of slice 0 of stage kt+1 ride on the odd MFMAs ----
+      const uint32_t a_target = cur + wave_lds;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int u = i * 4 + j;   // 0..15
+          if (u == 0) set_lds_target<0>(a_target);
+          if (u == 2) set_lds_target<1024>(a_target);
+          if (u == 4) set_lds_target<2048>(a_target);
+          if (u == 6) set_lds_target<3072>(a_target);
+          if (u < 8 && (u & 1) == 0) SRT_FENCE();
+          acc[i][j] = mfma<T>(bf[1][j], af[1][i], acc[i][j]);
+          pin(acc[i][j]);
+          if (u < 8 && (u & 1) == 0) {
+            SRT_FENCE();
+            load_to_lds_at_m0(ra, la.voff[u >> 1], soa);
+          }
+          if (u & 1) {
+            const int r = u >> 1;   // 0..7, same first-use order as above
+            if (r == 0) af[0][0] = fa.read(nxt, 0, 0);
+            else if (r <= 4) bf[0][r - 1] = fb.read(nxt + REGION, r - 1, 0);
+            else af[0][r - 4] = fa.read(nxt, r - 4, 0);
+          }
+          SRT_FENCE();
+        }
+      }
+      prv = cur;
+      cur = nxt;
+      sob = sob_next;
+    }
+    };
+    if (ragged) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
+    // Every load in flight must have landed, in every wave, before the slots vacated last become
+    // the staging area (the out-of-range fillers write zeros there); with the overlap on this
+    // also covers the next tile's first stages.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1
+    uint32_t pprv = prv - STAGE;
+    if (prv == lds) pprv = lds + (NS - 1) * STAGE;
+    const uint32_t stage = ((wave & 2) ? prv : pprv) + (uint32_t)(wave & 1) * 16384u;
+    const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
+    // the epilogue's per-lane address arithmetic starts from a lane id the compiler cannot see
+    // through: otherwise it is hoisted out of the tile loop and held (spilled) across the k loop
+    int le = lane;
+    asm volatile("" : "+v"(le));
+
+    // ---- epilogue ----
+    if (EPI == EPI_TRANS) {
+      store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
+    } else {
+      bool any_nan;
+      if (EPI == EPI_PLAIN) any_nan = any_nan_in_tile(acc);   // the accumulators are final as they are
+      else if (EPI == EPI_BIAS) any_nan = apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
+      else if (EPI == EPI_RELU) any_nan = apply_linear_epilogue<T, false, 1>(p, acc, em0, en0, le);
+      else if (EPI == EPI_BIAS_RELU) any_nan = apply_linear_epilogue<T, true, 1>(p, acc, em0, en0, le);
+      else any_nan = apply_linear_epilogue<T, true, 2>(p, acc, em0, en0, le);   // a null bias adds nothing
+      pin_all(acc);
+      if (any_nan) store_tile<T, true>(p, acc, em0, en0, bz, le, stage);
+      else store_tile<T, false>(p, acc, em0, en0, bz, le, stage);
+    }
+    if (!has_next) break;
+
+    // ---- next tile: the rest of its ring.  Every wave has finished reading its staging area
+    //      before any wave's loads overwrite it. ----
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    v = vn;
+    cur_tile = next_tile;
   }
 }
 
 #undef SRT_FENCE
 
-// Host-side preconditions beyond those of the MFMA family: every view must span less than 1 Gi
-// elements so 32-bit byte offsets reach it (including the rows of a partial last tile), and C
+// Host-side preconditions beyond those of the MFMA family: every operand tensor (all
+// batches) must span less than 1 Gi elements so 32-bit byte offsets reach it (including the rows
+// of a partial last tile), and C
 // must take aligned 16-byte stores of eight whole columns.
 inline bool ring_fits(const GemmProblem& p, bool a_kc, bool b_kc) {
   const long long lda = a_kc ? p.sam : p.sak, ldb = b_kc ? p.sbn : p.sbk;
-  const long long a_reach = a_kc ? ((long long)p.M + BM) * lda + p.K : ((long long)p.K + BK) * lda + p.M + BM;
-  const long long b_reach = b_kc ? ((long long)p.N + BN) * ldb + p.K : ((long long)p.K + BK) * ldb + p.N + BN;
+  const long long nb = p.batch - 1;
+  const long long a_reach = nb * p.sab + (a_kc ? ((long long)p.M + BM) * lda + p.K : ((long long)p.K + BK) * lda + p.M + BM);
+  const long long b_reach = nb * p.sbb + (b_kc ? ((long long)p.N + BN) * ldb + p.K : ((long long)p.K + BK) * ldb + p.N + BN);
   const long long c_reach = ((long long)p.M + BM) * p.scm + p.N + BN;
   const long long lim = 0x7fffffffLL / 2 - 4096;   // in elements: byte offsets stay below 2^31
   if (!(a_reach < lim && b_reach < lim && c_reach < lim)) return false;
+  if (p.sab < 0 || p.sbb < 0) return false;
   if ((p.N % 8) != 0 || (p.scm % 8) != 0 || (p.scb % 8) != 0) return false;
   if ((reinterpret_cast<uintptr_t>(p.C) & 15u) != 0) return false;
   return true;
+}
+
+// Compute units of the current device (cached per device).
+inline int compute_units() {
+  static std::atomic<int> cached[32];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 256;
+  int n = cached[device & 31].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+    cached[device & 31].store(n, std::memory_order_relaxed);
+  }
+  return n;
 }
 
 template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
@@ -634,8 +782,13 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   constexpr int lds_bytes = NS * STAGE;
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
-  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);
+  const long long tiles = (long long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN) * p.batch;
+  // one workgroup per compute unit (a workgroup takes a whole unit's LDS); the XCD-aware tile
+  // order wants the stride between a workgroup's tiles to be a multiple of 8
+  int grid = compute_units() & ~7;
+  if (grid <= 0) grid = 8;
+  if (tiles < grid) grid = (int)tiles;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return hipGetLastError();
 }
 
