@@ -197,15 +197,11 @@ __global__ __launch_bounds__(NT) void gemm_kc64_kernel(GemmProblem p) {
   if (EPI == EPI_TRANS) {
     store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   } else {
-    bool any_nan;
-    if (EPI == EPI_PLAIN) any_nan = any_nan_in_tile(acc);
-    else if (EPI == EPI_BIAS) any_nan = apply_linear_epilogue<T, true, 0>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_RELU) any_nan = apply_linear_epilogue<T, false, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_BIAS_RELU) any_nan = apply_linear_epilogue<T, true, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else any_nan = p.bias ? apply_linear_epilogue<T, true, 2>(p, acc, m0 + wm0, n0 + wn0, lane)
-                          : apply_linear_epilogue<T, false, 2>(p, acc, m0 + wm0, n0 + wn0, lane);
-    if (any_nan) store_tile<T, true>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
-    else store_tile<T, false>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+    if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, m0 + wm0, n0 + wn0, lane);
+    else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
+    else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
+    else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2>(p, acc, m0 + wm0, n0 + wn0, lane);
+    store_tile<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   }
 }
 

@@ -257,12 +257,11 @@ __device__ __forceinline__ void pin_all(f32x16_t (&acc)[4][4]) {
 // Step 1 for identity / relu / clippedRelu (apply_linear_epilogue): bias, then the activation as
 // one or two min/max instructions, in place and in straight-line code (the accumulators never
 // cross a branch); HAS_BIAS and CLAMP are compile-time so each variant carries only the
-// instructions it needs.  CLAMP: 0 none, 1 relu = max(x, 0), 2 clippedRelu = min(max(x, 0), coef).
-// max(NaN, 0) is 0 on this hardware, which is also what x > 0 ? x : 0 gives.
-// Returns whether any lane of the wave holds a NaN, so the rounding step can use the
-// one-instruction hardware converter when there is none.
+// instructions it needs (with HAS_BIAS a null bias pointer adds nothing).  CLAMP: 0 none,
+// 1 relu = max(x, 0), 2 clippedRelu = min(max(x, 0), coef).  max(NaN, 0) is 0 on this hardware,
+// which is also what x > 0 ? x : 0 gives.
 template <typename T, bool HAS_BIAS, int CLAMP>
-__device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x16_t (&acc)[4][4], int wave_m0,
+__device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x16_t (&acc)[4][4], int wave_m0,
                                                       int wave_n0, int lane) {
   using S = typename T::storage;
   const S* bias = (const S*)p.bias;
@@ -277,7 +276,6 @@ __device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x
       brow[i] = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
     }
   }
-  bool nan = false;
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -300,23 +298,8 @@ __device__ __forceinline__ bool apply_linear_epilogue(const GemmProblem& p, f32x
           if (CLAMP == 2) x = __builtin_fminf(x, ceiling);
           acc[i][j][4 * g + e] = x;
         }
-        nan |= __builtin_isunordered(acc[i][j][4 * g], acc[i][j][4 * g + 1]);
-        nan |= __builtin_isunordered(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
       }
     }
-  return __builtin_amdgcn_ballot_w64(nan) != 0;
-}
-
-// NaN test alone, for the plain matmul case.
-__device__ __forceinline__ bool any_nan_in_tile(const f32x16_t (&acc)[4][4]) {
-  bool nan = false;
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; v += 2) nan |= __builtin_isunordered(acc[i][j][v], acc[i][j][v + 1]);
-  return __builtin_amdgcn_ballot_w64(nan) != 0;
 }
 
 // Step 2 (store_tile): one rounding to the element type, then a trip through LDS so that global
@@ -326,10 +309,21 @@ __device__ __forceinline__ bool any_nan_in_tile(const f32x16_t (&acc)[4][4]) {
 // 16 B], chunk c of row r at position c ^ (r & 15) (reads of a row are conflict-free, writes of
 // a column 2-way).  Global stores go through a bounds-checked buffer; chunks outside M x N aim
 // out of range.
-template <typename T, bool EXACT>
+// Rounding uses the one-instruction hardware converter, which rounds to nearest even like the
+// reference's encoder but leaves a NaN some quiet-NaN pattern where the reference stores 0x7FFF:
+// the values are tested as they are converted, and for a half in which any lane of the wave saw
+// a NaN every NaN pattern is rewritten to 0x7FFF on its way from the staging area to memory.
+__device__ __forceinline__ uint32_t canonical_nans_bf16x2(uint32_t w) {
+  const uint32_t lo = w & 0xffffu, hi = w >> 16;
+  const uint32_t l = (lo & 0x7fffu) > 0x7f80u ? 0x7fffu : lo;
+  const uint32_t u = (hi & 0x7fffu) > 0x7f80u ? 0x7fffu : hi;
+  return l | (u << 16);
+}
+template <typename T>
 __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t (&acc)[4][4], int wave_m0, int wave_n0,
                                            int bz, int lane, uint32_t stage) {
   using S = typename T::storage;
+  constexpr bool FIXUP = T::dtype == srtReal16BF;   // the fp16 converter already encodes NaNs as required
   S* C = (S*)p.C + (long long)bz * p.scb;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;   // elements spanned by C (< 2^30, checked on the host)
   const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
@@ -342,7 +336,9 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t 
 
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
-    // ---- registers -> staging ----
+    // ---- registers -> staging (fenced per accumulator tile so that the compiler does not pull
+    //      all the accumulator reads of a half, or of the next half, to the front) ----
+    bool nan = false;
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
       const int i = 2 * half + ii;
@@ -350,24 +346,44 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t 
       const uint32_t row_addr = stage + (uint32_t)row * 256u + (uint32_t)h * 8u;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        SRT_FENCE();
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const u32x2_t w = {T::template pack2<EXACT>(acc[i][j][4 * g], acc[i][j][4 * g + 1]),
-                             T::template pack2<EXACT>(acc[i][j][4 * g + 2], acc[i][j][4 * g + 3])};
+          float a0 = acc[i][j][4 * g], a1 = acc[i][j][4 * g + 1], a2 = acc[i][j][4 * g + 2], a3 = acc[i][j][4 * g + 3];
+          // one copy out of the accumulator registers, here, for both the test and the conversion
+          asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+          if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
+          const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};
           const int c = 4 * j + g;
           *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
         }
       }
     }
-    // ---- staging -> global: 16 instructions of 4 rows x 256 bytes ----
+    SRT_FENCE();
+    const bool fix = FIXUP && __builtin_amdgcn_ballot_w64(nan) != 0;
+    // ---- staging -> global: 16 instructions of 4 rows x 256 bytes, read four at a time ----
 #pragma unroll
-    for (int it = 0; it < 16; ++it) {
-      const int row = rd_row + 4 * it;
-      const u32x4_t v =
-          *reinterpret_cast<const SRT_LDS u32x4_t*>(stage + (uint32_t)row * 256u + (uint32_t)((rd_chunk ^ (row & 15)) << 4));
-      const int m = wave_m0 + 64 * half + row;
-      const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc2 + n_rd * 2) : OOB;
-      __builtin_amdgcn_raw_buffer_store_b128(v, rc, (int)off, 0, SRT_STORE_AUX);
+    for (int it4 = 0; it4 < 4; ++it4) {
+      u32x4_t v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 4 * (4 * it4 + q);
+        v[q] = *reinterpret_cast<const SRT_LDS u32x4_t*>(stage + (uint32_t)row * 256u + (uint32_t)((rd_chunk ^ (row & 15)) << 4));
+      }
+      if (fix) {   // rare: some accumulator of this half was a NaN
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[q][e] = canonical_nans_bf16x2(v[q][e]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 4 * (4 * it4 + q);
+        const int m = wave_m0 + 64 * half + row;
+        const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc2 + n_rd * 2) : OOB;
+        __builtin_amdgcn_raw_buffer_store_b128(v[q], rc, (int)off, 0, SRT_STORE_AUX);
+      }
+      SRT_FENCE();
     }
   }
 }
@@ -471,9 +487,14 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  // The lane id is worked out afresh (two instructions) wherever per-lane state is derived from
+  // it, instead of being held in a register for the life of the kernel.
+  auto lane_id = []() {
+    uint32_t zero = 0;
+    asm volatile("" : "+s"(zero));   // opaque: keeps the two instructions where they are written
+    return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
+  };
   const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
 
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
@@ -518,7 +539,7 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
 
   // Requests stages first .. NS-2 of `tile` and the A part of stage NS-1 (its B part is the first
   // thing the loop requests); stage t goes to the slot t places after `slot0`.
-  auto fill_ring = [&](const Loader<A_KC>& la, const Loader<B_KC>& lb, const TileRef& tile, uint32_t slot0, int first) {
+  auto fill_ring = [&](const Loader<A_KC>& la, const Loader<B_KC>& lb, int lane, const TileRef& tile, uint32_t slot0, int first) {
 #pragma unroll
     for (int t = 0; t < NS; ++t) {
       if (t < first) continue;
@@ -551,21 +572,18 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
     Loader<B_KC> lb;
     FragReader<A_KC> fa;
     FragReader<B_KC> fb;
-    {
-      int l = lane;
-      asm volatile("" : "+v"(l));
-      la.init(wave, l, 0, lda);
-      lb.init(wave, l, 0, ldb);
-      fa.init(l, wm0);
-      fb.init(l, wn0);
-    }
+    const int lane = lane_id();
+    la.init(wave, lane, 0, lda);
+    lb.init(wave, lane, 0, ldb);
+    fa.init(lane, wm0);
+    fb.init(lane, wn0);
     // ---- the tile's ring: everything for the first tile and without the overlap (wait for
     //      stage 0 only); else stages 0 .. NS-3 landed before the previous epilogue ----
     if (first_tile || !overlap) {
-      fill_ring(la, lb, cur_tile, cur, 0);
+      fill_ring(la, lb, lane, cur_tile, cur, 0);
       asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(8 * (NS - 2) + 4) : "memory");
     } else {
-      fill_ring(la, lb, cur_tile, cur, NS - 2);
+      fill_ring(la, lb, lane, cur_tile, cur, NS - 2);
     }
     first_tile = false;
     SRT_FENCE();
@@ -716,22 +734,18 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
     const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
     // the epilogue's per-lane address arithmetic starts from a lane id the compiler cannot see
     // through: otherwise it is hoisted out of the tile loop and held (spilled) across the k loop
-    int le = lane;
-    asm volatile("" : "+v"(le));
+    const int le = lane_id();
 
     // ---- epilogue ----
     if (EPI == EPI_TRANS) {
       store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
     } else {
-      bool any_nan;
-      if (EPI == EPI_PLAIN) any_nan = any_nan_in_tile(acc);   // the accumulators are final as they are
-      else if (EPI == EPI_BIAS) any_nan = apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
-      else if (EPI == EPI_RELU) any_nan = apply_linear_epilogue<T, false, 1>(p, acc, em0, en0, le);
-      else if (EPI == EPI_BIAS_RELU) any_nan = apply_linear_epilogue<T, true, 1>(p, acc, em0, en0, le);
-      else any_nan = apply_linear_epilogue<T, true, 2>(p, acc, em0, en0, le);   // a null bias adds nothing
-      pin_all(acc);
-      if (any_nan) store_tile<T, true>(p, acc, em0, en0, bz, le, stage);
-      else store_tile<T, false>(p, acc, em0, en0, bz, le, stage);
+      if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
+      else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1>(p, acc, em0, en0, le);
+      else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1>(p, acc, em0, en0, le);
+      else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2>(p, acc, em0, en0, le);   // a null bias adds nothing
+      if (EPI != EPI_PLAIN) pin_all(acc);   // ends the life of the copies made above
+      store_tile<T>(p, acc, em0, en0, bz, le, stage);
     }
     if (!has_next) break;
 
