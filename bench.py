@@ -31,7 +31,7 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFM
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # and scaled by a 256 MiB device copy (profiles/gemm_ring_bf16_8192_counters.txt).
-TRAFFIC_BYTES_8192 = 1.759e9   # 2.000 x FETCH_SIZE (790 216 KiB) + 1.000 x WRITE_SIZE (137 216 KiB)
+TRAFFIC_BYTES_8192 = 1.747e9   # 2.000 x FETCH_SIZE (787 645 KiB) + 1.000 x WRITE_SIZE (131 115 KiB)
 
 
 def rng(seed):
@@ -140,7 +140,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=8192, row-major, no transposes, fp32 accumulate, bf16 out; "
                                "A,B ~ N(0,1)/sqrt(K) seed 2; inputs resident in HBM",
-                   "entry_point": "srtMatmul", "kernel": "gemm_ring_kernel<BF16> 256x256x32, 5-stage LDS ring"},
+                   "entry_point": "srtMatmul", "kernel": "gemm_ring_kernel<BF16> 256x256x32, 5-stage LDS ring, persistent (one workgroup per CU)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": TRAFFIC_BYTES_8192},
         "max_rel_err_vs_fp64": max_rel,
