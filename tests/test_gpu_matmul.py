@@ -217,6 +217,28 @@ def test_cfg1_f32_512_vs_oracle_and_fp64():
     assert err <= 2 * max(H.max_norm_rel(want, c64), 1e-7)
 
 
+def test_f32_split_k_row_major_ragged_and_batched():
+    """Row-major fp32 problems small enough for the split-K tile: ragged M, N a multiple of 4 but not
+    of the tile, K a multiple of 4 but not of the 16-deep slab (and longer than one wave's prefetch),
+    a batch, bias + activation.  Integer-valued inputs are bit-exact; random ones within 1e-5 of fp64."""
+    r = H.rng(31)
+    for (M, N, K, batch) in [(70, 132, 200, None), (33, 36, 2052, None), (96, 64, 520, 3)]:
+        lead = () if batch is None else (batch,)
+        a = r.integers(-3, 4, lead + (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, lead + (K, N)).astype(np.float32)
+        got = gpu_matmul(a, b, want_kernel="f32_mfma")
+        assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)), (M, N, K)
+        a = r.uniform(-1, 1, a.shape).astype(np.float32)
+        b = r.uniform(-1, 1, b.shape).astype(np.float32)
+        check_against_fp64(gpu_matmul(a, b), a, b, False, False, H.F32)
+    x = r.uniform(-1, 1, (70, 200)).astype(np.float32)
+    w = r.uniform(-1, 1, (200, 132)).astype(np.float32)
+    bias = r.uniform(-0.5, 0.5, 132).astype(np.float32)
+    y = srt.Dense(srt.Tensor(w), srt.Tensor(bias), srt.ActivationType.relu)(srt.Tensor(x)).array()
+    want = np.maximum(x.astype(np.float64) @ w.astype(np.float64) + bias, 0.0)
+    assert H.max_norm_rel(y, want) <= H.TOL[H.F32]
+
+
 def test_cfg2_f16_batched_transpose_rhs():
     r = H.rng(1)
     a = (r.standard_normal((32, 256, 256)) * 0.1).astype(np.float16)
