@@ -369,17 +369,19 @@ int mfma_select(const GemmProblem& p) {
   //    intensity) that they win long before they can fill the device: from 48 tiles up for the
   //    ring kernel (3072^3, 144 tiles: 64 us against 143 us with 128 x 128 tiles);
   //  * with both operands k-contiguous the 64 x 64 kernel reads whole lines too and stays ahead up
-  //    to about 96 tiles of 256 x 256 (2048^3 NT: 36 us against 44 us); above that the 64-deep
-  //    256 x 256 kernel takes over (whole-line loads where the ring kernel moves half lines:
-  //    8192^3 NT 1313 against 1277 TFLOP/s);
+  //    to about 96 tiles of 256 x 256 (2048^3 NT: 36 us against 44 us); from there the ring kernel
+  //    runs until the device is three quarters full (2048 x 4096 x 4096 NT, 128 tiles: 84 us
+  //    against 88 us) and then the 64-deep 256 x 256 kernel takes over (whole-line loads where
+  //    the ring kernel moves half lines: 4096^3 NT 114 us against 126 us, 8192^3 NT 1351 against
+  //    1336 TFLOP/s);
   //  * below those thresholds every CU should get a workgroup: 64 x 64 tiles (batch 32 x 256^3:
   //    7.7 us against 15.0 us with 128 x 128).  128 x 128 is kept for problems that do not meet
   //    the 256 x 256 kernels' preconditions but have at least one such tile per CU.
   const bool big_ok = ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0);
   const long long t256 = tiles(256);
   int tile;
-  if (big_ok && layout == 3 && t256 >= 96) tile = 4;
-  else if (big_ok && layout != 3 && t256 >= 48) tile = 1;
+  if (big_ok && layout == 3 && t256 >= 192) tile = 4;
+  else if (big_ok && t256 >= (layout == 3 ? 96 : 48)) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
