@@ -78,8 +78,10 @@ def time_steps(queue, fn, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed launches before the timed ones; the memory and fabric clocks of an idle device take "
+                         "a few hundred milliseconds of load to settle (10 warm-up launches read 3 %% low)")
     ap.add_argument("--all", action="store_true", help="also report the other configurations on stderr")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ceiling", action="store_true",
