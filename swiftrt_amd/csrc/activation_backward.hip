@@ -50,6 +50,18 @@ struct alignas(V * sizeof(typename T::storage)) Pack {
   typename T::storage v[V];
 };
 
+// One vector of y or dy, with the non-temporal hint: both are read exactly once.
+template <typename T, int V>
+__device__ __forceinline__ Pack<T, V> load_once(const typename T::storage* p) {
+  constexpr int BYTES = V * (int)sizeof(typename T::storage);
+  if constexpr (BYTES >= 8) {
+    typedef uint32_t words_t __attribute__((ext_vector_type(BYTES / 4)));
+    return __builtin_bit_cast(Pack<T, V>, __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p)));
+  } else {
+    return *reinterpret_cast<const Pack<T, V>*>(p);
+  }
+}
+
 template <typename T, int V>
 __global__ __launch_bounds__(256) void activation_backward_kernel(BackwardProblem p) {
   using S = typename T::storage;
@@ -71,12 +83,12 @@ __global__ __launch_bounds__(256) void activation_backward_kernel(BackwardProble
       const bool second = m2 < m_end;
       float fy[2][V], fd[2][V];
       if (V > 1) {
-        const Pack<T, V> py0 = *reinterpret_cast<const Pack<T, V>*>(y + (long long)m * p.sym + n0);
-        const Pack<T, V> pd0 = *reinterpret_cast<const Pack<T, V>*>(dy + (long long)m * p.sdm + n0);
+        const Pack<T, V> py0 = load_once<T, V>(y + (long long)m * p.sym + n0);
+        const Pack<T, V> pd0 = load_once<T, V>(dy + (long long)m * p.sdm + n0);
         Pack<T, V> py1 = py0, pd1 = pd0;
         if (second) {
-          py1 = *reinterpret_cast<const Pack<T, V>*>(y + (long long)m2 * p.sym + n0);
-          pd1 = *reinterpret_cast<const Pack<T, V>*>(dy + (long long)m2 * p.sdm + n0);
+          py1 = load_once<T, V>(y + (long long)m2 * p.sym + n0);
+          pd1 = load_once<T, V>(dy + (long long)m2 * p.sdm + n0);
         }
 #pragma unroll
         for (int i = 0; i < V; ++i) {
