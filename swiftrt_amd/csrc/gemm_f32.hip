@@ -1,14 +1,16 @@
 // fp32 matmul on the matrix cores: v_mfma_f32_32x32x2_f32 (true fp32 products and sums, no
-// reduced-precision path), any strides.
+// reduced-precision path), any strides.  Operands are staged through LDS k-major ([k][m],
+// [k][n]) so the MFMA operand of lane l (row / column l % 32, k = 2 kk + l / 32) is a
+// conflict-free LDS read; the next k tile is prefetched into registers while the current one
+// multiplies.  Four kernels:
 //
-//   tile    64 x 64 x 16 per workgroup of 4 waves (2 x 2, each one 32 x 32 MFMA tile = 16 fp32
-//           accumulators per lane); operands are staged through LDS k-major ([k][m], [k][n]) so
-//           the MFMA operand of lane l (row / column l % 32, k = 2 kk + l / 32) is one
-//           conflict-free ds_read_b32.
-//   loads   element-wise with the caller's strides (views, transposes, column-major all land
-//           here), next k tile prefetched into registers while the current one multiplies.
-//   split   when the 64 x 64 tiles alone would leave most CUs idle (e.g. 512^3 = 64 tiles), the
-//           tile shrinks to 32 x 32 and the 4 waves split K between them, summing through LDS.
+//   128 x 128, vector   every operand has a unit stride along k or m / n with 16-byte aligned rows:
+//                       16-byte global loads, 8-byte operand reads (4096^3: ~120 TFLOP/s)
+//   128 x 128 / 64 x 64 element-wise loads with the caller's strides (views, column-major, odd
+//                       pitches all land here); the small tile when the large one would leave CUs idle
+//   32 x 32 split-K     launch-latency-sized problems (512^3 = 64 tiles of 64 x 64): the 4 waves split
+//                       K between them and sum through LDS; row-major operands take a variant that
+//                       keeps a wave's whole k range in flight
 #include "gemm_common.h"
 
 namespace srt {
@@ -16,53 +18,66 @@ namespace srt {
 namespace {
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4v_t __attribute__((ext_vector_type(4)));
 
 constexpr int FT = 64;   // tile edge
 constexpr int FK = 16;   // k per stage
 
-// ---- 64 x 64 tiles, waves 2 x 2 ----------------------------------------------------------------
+// ---- 64 x 64 or 128 x 128 tiles, waves 2 x 2 -----------------------------------------------------
+// TW = 32 x 32 MFMA tiles per wave and dimension: 1 -> 64 x 64 per workgroup, 2 -> 128 x 128.
+// The fixed cost of a k stage (global loads, LDS writes, two barriers) is the same for both,
+// so the large tile, with four times the MFMAs per stage, is the one that approaches the matrix
+// more efficient one (4096^3: 87 -> 96 TFLOP/s); the small one is for problems that would
+// otherwise leave CUs idle.
+template <int TW>
 __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(GemmProblem p) {
-  __shared__ float As[2][FK][FT + 4];
-  __shared__ float Bs[2][FK][FT + 4];
+  constexpr int TILE = FT * TW;          // 64 or 128
+  constexpr int PER = 4 * TW;            // elements of each operand a thread stages per k tile
+  __shared__ float As[2][FK][TILE + 4];
+  __shared__ float Bs[2][FK][TILE + 4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int wm = (wave >> 1) * 32 * TW, wn = (wave & 1) * 32 * TW;
   const int r = lane & 31, kh = lane >> 5;
-  const int m0 = blockIdx.y * FT, n0 = blockIdx.x * FT, bz = blockIdx.z;
+  const int m0 = blockIdx.y * TILE, n0 = blockIdx.x * TILE, bz = blockIdx.z;
   const float* A = (const float*)p.A + (long long)bz * p.sab;
   const float* B = (const float*)p.B + (long long)bz * p.sbb;
   float* C = (float*)p.C + (long long)bz * p.scb;
 
   // thread -> element mapping that walks the unit stride first
   const bool a_k_fast = (p.sak == 1), b_n_fast = (p.sbn == 1);
-  int am[4], ak[4], bn[4], bk[4];
+  int am[PER], ak[PER], bn[PER], bk[PER];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < PER; ++i) {
     const int idx = tid + i * 256;
-    if (a_k_fast) { ak[i] = idx & (FK - 1); am[i] = idx >> 4; } else { am[i] = idx & (FT - 1); ak[i] = idx >> 6; }
-    if (b_n_fast) { bn[i] = idx & (FT - 1); bk[i] = idx >> 6; } else { bk[i] = idx & (FK - 1); bn[i] = idx >> 4; }
+    if (a_k_fast) { ak[i] = idx & (FK - 1); am[i] = idx >> 4; } else { am[i] = idx & (TILE - 1); ak[i] = idx / TILE; }
+    if (b_n_fast) { bn[i] = idx & (TILE - 1); bk[i] = idx / TILE; } else { bk[i] = idx & (FK - 1); bn[i] = idx >> 4; }
   }
-  auto fetch = [&](int k0, float (&ra)[4], float (&rb)[4]) {
+  auto fetch = [&](int k0, float (&ra)[PER], float (&rb)[PER]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < PER; ++i) {
       const int m = m0 + am[i], ka = k0 + ak[i], n = n0 + bn[i], kb = k0 + bk[i];
       ra[i] = (m < p.M && ka < p.K) ? A[(long long)m * p.sam + (long long)ka * p.sak] : 0.0f;
       rb[i] = (n < p.N && kb < p.K) ? B[(long long)kb * p.sbk + (long long)n * p.sbn] : 0.0f;
     }
   };
-  auto stash = [&](int buf, const float (&ra)[4], const float (&rb)[4]) {
+  auto stash = [&](int buf, const float (&ra)[PER], const float (&rb)[PER]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < PER; ++i) {
       As[buf][ak[i]][am[i]] = ra[i];
       Bs[buf][bk[i]][bn[i]] = rb[i];
     }
   };
 
-  f32x16_t acc;
+  f32x16_t acc[TW][TW];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  for (int i = 0; i < TW; ++i)
+#pragma unroll
+    for (int j = 0; j < TW; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  float ra[4], rb[4];
+  float ra[PER], rb[PER];
   fetch(0, ra, rb);
   stash(0, ra, rb);
   __syncthreads();
@@ -71,21 +86,192 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(GemmProblem p) {
     const int buf = kt & 1;
     if (kt + 1 < KT) fetch((kt + 1) * FK, ra, rb);
 #pragma unroll
-    for (int kk = 0; kk < FK / 2; ++kk)
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(As[buf][2 * kk + kh][wm + r], Bs[buf][2 * kk + kh][wn + r], acc, 0, 0, 0);
+    for (int kk = 0; kk < FK / 2; ++kk) {
+      float af[TW], bf[TW];
+#pragma unroll
+      for (int i = 0; i < TW; ++i) af[i] = As[buf][2 * kk + kh][wm + 32 * i + r];
+#pragma unroll
+      for (int j = 0; j < TW; ++j) bf[j] = Bs[buf][2 * kk + kh][wn + 32 * j + r];
+#pragma unroll
+      for (int i = 0; i < TW; ++i)
+#pragma unroll
+        for (int j = 0; j < TW; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
     if (kt + 1 < KT) stash(buf ^ 1, ra, rb);
     __syncthreads();
   }
 
-  // lane holds column r and rows 8 (v / 4) + 4 kh + v % 4 of the wave's 32 x 32 tile
+  // lane holds column r and rows 8 (v / 4) + 4 kh + v % 4 of each 32 x 32 tile
   Epilogue<F32> ep(p);
-  const int n = n0 + wn + r;
-  if (n >= p.N) return;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    const int m = m0 + wm + 8 * (v >> 2) + 4 * kh + (v & 3);
-    if (m < p.M) C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(acc[v], ep.bias_at(m, n));
+  for (int j = 0; j < TW; ++j) {
+    const int n = n0 + wn + 32 * j + r;
+    if (n >= p.N) continue;
+#pragma unroll
+    for (int i = 0; i < TW; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm + 32 * i + 8 * (v >> 2) + 4 * kh + (v & 3);
+        if (m < p.M) C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(acc[i][j][v], ep.bias_at(m, n));
+      }
+    }
   }
+}
+
+// ---- 128 x 128 tiles, unit-stride operands: 16-byte loads, 8-byte LDS operand reads ------------
+// The kernel above spends about as many issue cycles on scalar loads, address arithmetic and
+// 4-byte LDS traffic as on MFMAs.  When every operand has a unit stride along k (K_FAST) or along
+// m / n, 16-byte aligned rows and an extent along that stride that is a multiple of 4, a thread
+// stages two 16-byte vectors per operand and k tile, and the wave's 64 x 64 tile is laid out so
+// that the operands of both of its MFMA tiles along a dimension are neighbours in LDS:
+//   LDS     k-major [16 k][128 mn], pitch 132.  A vector along mn is one ds_write_b128; a vector
+//           along k is four ds_write_b32 (conflict-free: the lanes of a wave cover 16 rows x 4 k
+//           groups, and 16 kq + row spans the 64 banks).
+//   MFMA    tile (i, j) of a wave takes rows wm + 2 r + i and columns wn + 2 r + j (lane r):
+//           one ds_read_b64 per operand and k pair feeds both tiles, and the two results a lane
+//           holds for a row are neighbouring columns of C (one 8-byte store).
+// 4096^3: 117-121 TFLOP/s for the four transpose combinations (96 with the kernel above).
+template <bool K_FAST>
+struct VecStage {
+  f32x4v_t v[2];
+  const float* ptr[2];
+  int mn[2], k[2];
+  bool ok[2];
+
+  // mn0: first row / column of the tile; extent: M or N; ld: stride of the other dimension
+  __device__ __forceinline__ void init(const float* base, int tid, int mn0, int extent, long long ld) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int f = tid + 256 * i;
+      if (K_FAST) { mn[i] = f >> 2; k[i] = (f & 3) * 4; } else { k[i] = f >> 5; mn[i] = (f & 31) * 4; }
+      ok[i] = mn0 + mn[i] < extent;   // the extent along a unit stride is a multiple of 4: whole vectors
+      ptr[i] = K_FAST ? base + (long long)(mn0 + mn[i]) * ld + k[i] : base + (long long)k[i] * ld + mn0 + mn[i];
+    }
+  }
+  __device__ __forceinline__ void load(int k0, int K, long long ld) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const f32x4v_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+      const float* q = K_FAST ? ptr[i] + k0 : ptr[i] + (long long)k0 * ld;
+      v[i] = (ok[i] && k0 + k[i] < K) ? *reinterpret_cast<const f32x4v_t*>(q) : zero;
+    }
+  }
+  __device__ __forceinline__ void store(float (*dst)[132]) const {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      if (K_FAST) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[k[i] + e][mn[i]] = v[i][e];
+      } else {
+        *reinterpret_cast<f32x4v_t*>(&dst[k[i]][mn[i]]) = v[i];
+      }
+    }
+  }
+};
+
+typedef float f32x2v_t __attribute__((ext_vector_type(2)));
+
+template <bool A_KF, bool B_KF>
+__global__ __launch_bounds__(256) void gemm_f32_mfma128_vec_kernel(GemmProblem p) {
+  __shared__ __attribute__((aligned(16))) float As[2][FK][132];
+  __shared__ __attribute__((aligned(16))) float Bs[2][FK][132];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int r = lane & 31, kh = lane >> 5;
+  const int m0 = blockIdx.y * 128, n0 = blockIdx.x * 128, bz = blockIdx.z;
+  const float* A = (const float*)p.A + (long long)bz * p.sab;
+  const float* B = (const float*)p.B + (long long)bz * p.sbb;
+  float* C = (float*)p.C + (long long)bz * p.scb;
+  const long long lda = A_KF ? p.sam : p.sak, ldb = B_KF ? p.sbn : p.sbk;
+
+  VecStage<A_KF> sa;
+  VecStage<B_KF> sb;
+  sa.init(A, tid, m0, p.M, lda);
+  sb.init(B, tid, n0, p.N, ldb);
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  sa.load(0, p.K, lda);
+  sb.load(0, p.K, ldb);
+  sa.store(As[0]);
+  sb.store(Bs[0]);
+  __syncthreads();
+  const int KT = (p.K + FK - 1) / FK;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) {
+      sa.load((kt + 1) * FK, p.K, lda);
+      sb.load((kt + 1) * FK, p.K, ldb);
+    }
+#pragma unroll
+    for (int kk = 0; kk < FK / 2; ++kk) {
+      const f32x2v_t af = *reinterpret_cast<const f32x2v_t*>(&As[buf][2 * kk + kh][wm + 2 * r]);
+      const f32x2v_t bf = *reinterpret_cast<const f32x2v_t*>(&Bs[buf][2 * kk + kh][wn + 2 * r]);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) {
+      sa.store(As[buf ^ 1]);
+      sb.store(Bs[buf ^ 1]);
+    }
+    __syncthreads();
+  }
+
+  // tile (i, j): lane r holds column wn + 2 r + j and rows wm + 2 (8 (v / 4) + 4 kh + v % 4) + i
+  Epilogue<F32> ep(p);
+  const int n = n0 + wn + 2 * r;
+  const bool pair_store = p.scn == 1 && (p.scm % 2) == 0 && (p.scb % 2) == 0 &&
+                          (reinterpret_cast<uintptr_t>(p.C) & 7u) == 0 && n + 1 < p.N;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int m = m0 + wm + 2 * (8 * (v >> 2) + 4 * kh + (v & 3)) + i;
+      if (m >= p.M) continue;
+      const float c0 = n < p.N ? ep.finish(acc[i][0][v], ep.bias_at(m, n)) : 0.0f;
+      const float c1 = n + 1 < p.N ? ep.finish(acc[i][1][v], ep.bias_at(m, n + 1)) : 0.0f;
+      if (pair_store) {
+        const f32x2v_t c = {c0, c1};
+        *reinterpret_cast<f32x2v_t*>(C + (long long)m * p.scm + n) = c;
+      } else {
+        if (n < p.N) C[(long long)m * p.scm + (long long)n * p.scn] = c0;
+        if (n + 1 < p.N) C[(long long)m * p.scm + (long long)(n + 1) * p.scn] = c1;
+      }
+    }
+  }
+}
+
+// Preconditions of the 128 x 128 vector kernel: unit stride along k or along m / n for both
+// operands, 16-byte aligned rows, whole 16-byte vectors along the unit stride.
+bool mfma128_vec_fits(const GemmProblem& p) {
+  const bool a_kf = p.sak == 1, a_mf = p.sam == 1;
+  const bool b_kf = p.sbk == 1, b_nf = p.sbn == 1;
+  if (!(a_kf || a_mf) || !(b_kf || b_nf)) return false;
+  const long long lda = a_kf ? p.sam : p.sak, ldb = b_kf ? p.sbn : p.sbk;
+  if ((lda % 4) != 0 || (ldb % 4) != 0 || (p.sab % 4) != 0 || (p.sbb % 4) != 0) return false;
+  if ((a_kf ? p.K : p.M) % 4 != 0 || (b_kf ? p.K : p.N) % 4 != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(p.A) & 15u) != 0 || (reinterpret_cast<uintptr_t>(p.B) & 15u) != 0) return false;
+  return true;
+}
+
+hipError_t launch_mfma128_vec(const GemmProblem& p, hipStream_t stream) {
+  dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, p.batch);
+  const bool a_kf = p.sak == 1, b_kf = p.sbk == 1 && p.sbn != 1;
+  // an operand with both strides 1 (a single row or column) counts as k-contiguous for A, n-contiguous for B
+  if (a_kf && b_kf) hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<true, true>), grid, dim3(256), 0, stream, p);
+  else if (a_kf) hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<true, false>), grid, dim3(256), 0, stream, p);
+  else if (b_kf) hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<false, true>), grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<false, false>), grid, dim3(256), 0, stream, p);
+  return hipGetLastError();
 }
 
 // ---- 32 x 32 tiles, the 4 waves split K ---------------------------------------------------------
@@ -177,7 +363,6 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_splitk_kernel(GemmProblem p
 //           in banks 0-31 and odd ones in 32-63, which is exactly the split of the MFMA operand
 //           read (lanes 0-31 take k = 2 kk, lanes 32-63 k = 2 kk + 1).
 constexpr int SV_SLABS = 8;
-typedef float f32x4v_t __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void gemm_f32_mfma_splitk_vec_kernel(GemmProblem p) {
   __shared__ float As[4][2][FK][36];
@@ -303,9 +488,18 @@ hipError_t launch_f32_mfma_variant(const GemmProblem& p, bool splitk, hipStream_
     if (splitk_vec_fits(p)) hipLaunchKernelGGL(gemm_f32_mfma_splitk_vec_kernel, grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL(gemm_f32_mfma_splitk_kernel, grid, dim3(256), 0, stream, p);
   } else {
-    if ((p.M + FT - 1) / FT > 65535) return hipErrorInvalidValue;
-    dim3 grid((p.N + FT - 1) / FT, (p.M + FT - 1) / FT, p.batch);
-    hipLaunchKernelGGL(gemm_f32_mfma_kernel, grid, dim3(256), 0, stream, p);
+    // the 128 x 128 tile once it gives every CU a workgroup, the 64 x 64 tile below that
+    const long long tiles128 = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+    if (tiles128 >= 256) {
+      if ((p.M + 127) / 128 > 65535) return hipErrorInvalidValue;
+      if (mfma128_vec_fits(p)) return launch_mfma128_vec(p, stream);
+      dim3 grid((p.N + 127) / 128, (p.M + 127) / 128, p.batch);
+      hipLaunchKernelGGL(gemm_f32_mfma_kernel<2>, grid, dim3(256), 0, stream, p);
+    } else {
+      if ((p.M + FT - 1) / FT > 65535) return hipErrorInvalidValue;
+      dim3 grid((p.N + FT - 1) / FT, (p.M + FT - 1) / FT, p.batch);
+      hipLaunchKernelGGL(gemm_f32_mfma_kernel<1>, grid, dim3(256), 0, stream, p);
+    }
   }
   return hipGetLastError();
 }

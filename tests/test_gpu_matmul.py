@@ -239,6 +239,39 @@ def test_f32_split_k_row_major_ragged_and_batched():
     assert H.max_norm_rel(y, want) <= H.TOL[H.F32]
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_f32_128_tile_all_layouts_ragged(ta, tb):
+    """fp32 problems large enough for the 128 x 128 tile, every transpose combination (16-byte loads
+    along k or along m / n), ragged M and N edges, K that ends inside a 16-deep stage; a view with an
+    unaligned pitch takes the element-wise variant of the same tile.  Bit-exact on integers, 1e-5 on
+    random data, bias + relu on top."""
+    r = H.rng(41)
+    M, N, K = 2040, 2056, 136
+    a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
+    b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+    got = gpu_matmul(a, b, ta, tb, want_kernel="f32_mfma")
+    exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+    assert np.array_equal(got, exact.astype(np.float32))
+    a = r.uniform(-1, 1, a.shape).astype(np.float32)
+    b = r.uniform(-1, 1, b.shape).astype(np.float32)
+    check_against_fp64(gpu_matmul(a, b, ta, tb), a, b, ta, tb, H.F32)
+    bias = r.uniform(-0.5, 0.5, N).astype(np.float32)
+    at, bt = srt.Tensor(a), srt.Tensor(b)
+    out = srt.Tensor(shape=[M, N], dtype=np.float32)
+    srt.current_queue().matmul(at, ta, bt, tb, out, bias=srt.Tensor(bias), activation=srt.ActivationType.relu)
+    want = np.maximum((a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64) + bias, 0.0)
+    assert H.max_norm_rel(out.array(), want) <= H.TOL[H.F32]
+    if not ta and not tb:
+        # operand views with a pitch that is not a multiple of 4 elements: no 16-byte loads
+        av_host = r.integers(-3, 4, (M, K)).astype(np.float32)
+        padded = np.zeros((M, K + 3), np.float32)
+        padded[:, :K] = av_host
+        av = srt.Tensor(padded)[:, :K]
+        bi = r.integers(-3, 4, (K, N)).astype(np.float32)
+        out2 = srt.matmul(av, srt.Tensor(bi))
+        assert np.array_equal(out2.array(), (av_host.astype(np.int64) @ bi.astype(np.int64)).astype(np.float32))
+
+
 def test_cfg2_f16_batched_transpose_rhs():
     r = H.rng(1)
     a = (r.standard_normal((32, 256, 256)) * 0.1).astype(np.float16)
