@@ -157,7 +157,8 @@ hipError_t launch_generic(const GemmProblem& p, hipStream_t stream);
 
 // Tile configuration chosen for the MFMA family, or 0 if the problem does not qualify.
 int mfma_select(const GemmProblem& p);
-// Same for a caller-chosen tile (1: 256 x 256, 2: 128 x 128, 3: 64 x 64); 0 if it does not qualify.
+// Same for a caller-chosen tile (1: 256 x 256, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with 64-deep
+// stages, 5: 256 x 256 on 16x16x32 MFMAs); 0 if it does not qualify.
 int mfma_config(const GemmProblem& p, int tile);
 const char* mfma_name(int config);
 hipError_t launch_mfma(const GemmProblem& p, int config, hipStream_t stream);

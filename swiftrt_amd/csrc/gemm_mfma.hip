@@ -37,6 +37,14 @@ hipError_t launch_kc64_F16(const GemmProblem& p, hipStream_t stream);
 SRT_RING_DECL(BF16)
 SRT_RING_DECL(F16)
 #undef SRT_RING_DECL
+#define SRT_M16_DECL(T)                                                  \
+  hipError_t launch_m16_##T##_00(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16_##T##_01(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16_##T##_10(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16_##T##_11(const GemmProblem&, hipStream_t);
+SRT_M16_DECL(BF16)
+SRT_M16_DECL(F16)
+#undef SRT_M16_DECL
 
 namespace {
 
@@ -310,12 +318,31 @@ hipError_t launch_ring<F16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStrea
   return launch_ring_F16_00(p, stream);
 }
 
-// tile 1 (256 x 256) is the ring kernel; tiles 2 and 3 are the register-staged kernels above
+template <typename T>
+hipError_t launch_m16(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream);
+template <>
+hipError_t launch_m16<BF16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_m16_BF16_11(p, stream);
+  if (a_kc) return launch_m16_BF16_10(p, stream);
+  if (b_kc) return launch_m16_BF16_01(p, stream);
+  return launch_m16_BF16_00(p, stream);
+}
+template <>
+hipError_t launch_m16<F16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_m16_F16_11(p, stream);
+  if (a_kc) return launch_m16_F16_10(p, stream);
+  if (b_kc) return launch_m16_F16_01(p, stream);
+  return launch_m16_F16_00(p, stream);
+}
+
+// tile 1 (256 x 256) is the ring kernel, tile 5 the same ring on 16x16x32 MFMAs; tiles 2 and 3 are the
+// register-staged kernels above
 template <typename T>
 hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hipStream_t stream) {
   switch (tile) {
     case 1: return launch_ring<T>(p, a_kc, b_kc, stream);
     case 4: return T::dtype == srtReal16BF ? launch_kc64_BF16(p, stream) : launch_kc64_F16(p, stream);
+    case 5: return launch_m16<T>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     default: return launch_layout<T, 64, 64>(p, a_kc, b_kc, stream);
   }
@@ -350,12 +377,12 @@ static int mfma_layout(const GemmProblem& p) {
 }
 
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
-// 64-deep stages for two k-contiguous operands), or 0 when the
-// problem does not qualify for it.
+// 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs), or 0
+// when the problem does not qualify for it.
 int mfma_config(const GemmProblem& p, int tile) {
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || tile > 4) return 0;
-  if ((tile == 1 || tile == 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
+  if (layout < 0 || tile < 1 || tile > 5) return 0;
+  if ((tile == 1 || tile == 4 || tile == 5) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
 }
@@ -374,13 +401,20 @@ int mfma_select(const GemmProblem& p) {
   //    against 88 us) and then the 64-deep 256 x 256 kernel takes over (whole-line loads where
   //    the ring kernel moves half lines: 4096^3 NT 114 us against 126 us, 8192^3 NT 1351 against
   //    1336 TFLOP/s);
+  //  * once the device is three quarters full and the k loop is long, sustained speed is set by
+  //    the power limit, and the 16x16x32 form of the ring kernel, cheaper per flop, wins in every
+  //    layout (8192^3: 1390-1440 against 1300-1350 TFLOP/s; 4096 x 11008 x 4096: 292 us against
+  //    306-320 us).  Its loop has less slack per MFMA, so where clocks are not the limit -- a
+  //    partly filled device -- the 32x32x16 kernels stay ahead (2048^3: 42 us against 45 us),
+  //    and with short k loops (K = 1024) nothing separates them;
   //  * below those thresholds every CU should get a workgroup: 64 x 64 tiles (batch 32 x 256^3:
   //    7.7 us against 15.0 us with 128 x 128).  128 x 128 is kept for problems that do not meet
   //    the 256 x 256 kernels' preconditions but have at least one such tile per CU.
   const bool big_ok = ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0);
   const long long t256 = tiles(256);
   int tile;
-  if (big_ok && layout == 3 && t256 >= 192) tile = 4;
+  if (big_ok && t256 >= 192 && p.K >= 2048) tile = 5;
+  else if (big_ok && layout == 3 && t256 >= 192) tile = 4;
   else if (big_ok && t256 >= (layout == 3 ? 96 : 48)) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
@@ -391,6 +425,7 @@ const char* mfma_name(int config) {
   switch (config >> 2) {
     case 1: return "mfma_256x256";
     case 4: return "mfma_256x256_k64";
+    case 5: return "mfma_256x256_m16";
     case 2: return "mfma_128x128";
     default: return "mfma_64x64";
   }

@@ -1,0 +1,574 @@
+// 256 x 256 bf16 / fp16 matmul tile kernel for gfx950 on v_mfma_f32_16x16x32: the persistent,
+// direct-to-LDS ring of gemm_mfma_ring.h (same LDS layouts, loaders, tile walk and cross-tile
+// prefetch -- see there) with the 128 x 128 wave tile cut into 8 x 8 MFMA tiles of 16 x 16
+// instead of 4 x 4 tiles of 32 x 32.
+//
+// Why a second instruction shape.  On N(0,1) data this part runs against its power limit, and
+// what a GEMM sustains is set by the energy it spends per flop.  A loop of nothing but MFMAs on
+// such data, all CUs, four waves each with 256 accumulator registers per lane:
+//     32x32x16                         1780-1800 TFLOP/s
+//     16x16x32                         2050      TFLOP/s
+// and with the LDS fragment reads a 128 x 128 wave tile needs (16 KiB per wave and k = 32):
+//     32x32x16, 16 reads / 32 MFMAs    1575-1585 TFLOP/s
+//     16x16x32, 16 reads / 64 MFMAs    1720      TFLOP/s
+// Both shapes read the same fragment bytes per flop; the 16x16x32 instruction itself is the
+// cheaper one.
+//
+// The MFMAs are written as inline assembly with the accumulator tile as a tied in/out operand.
+// Given the builtin, the register allocator does not keep source and destination accumulator in
+// the same registers once all 256 accumulator registers are live: it rotates tiles through
+// spare registers with v_accvgpr moves between the MFMAs (measured on an MFMA-only loop: 1760
+// instead of 2435 TFLOP/s on zeros).  The compiler does not know the statement is an MFMA, so the
+// wait states the hardware needs between an MFMA and a dependent non-MFMA access of its
+// accumulator are written out where they could matter (after the k loop, after the zero fill).
+//
+// An MFMA operand is 16 rows x 32 k: lane l holds row l % 16, k = 8 (l / 16) .. + 7 -- one
+// ds_read_b128 from a k-contiguous region, two ds_read_b64_tr_b16 from an mn-contiguous one.
+// The MFMA takes the B fragment first, so a 16 x 16 accumulator tile is C^T: lane l owns row
+// m = l % 16 and the four consecutive columns n = 4 (l / 16) .. + 3.
+//
+// Pipeline per stage and wave (two phases of 32 MFMAs, 16 cycles each):
+//   phase 0   MFMAs of A tiles 0-3 x B tiles 0-7; the reads of B tiles 4-7 and A tiles 4-7 ride on
+//             the first half, the four B loads of stage s-1+NS on the second
+//   sync      s_waitcnt vmcnt(8 (NS-2)) lgkmcnt(0); s_barrier -- stage s+1 has landed for every
+//             wave, every wave holds all of stage s in registers: its slot is free
+//   phase 1   MFMAs of A tiles 4-7, with the four A loads of stage s+NS and the reads of stage
+//             s+1 (A and B tiles 0-3, B tile j as soon as its last MFMA of the stage has issued)
+#pragma once
+#include "gemm_mfma_ring.h"
+
+namespace srt {
+namespace m16 {
+
+using ring::bf16x8_t;
+using ring::f16x8_t;
+using ring::f32x4_t;
+using ring::u32x2_t;
+using ring::u32x4_t;
+using ring::s16x4_t;
+using ring::BK;
+using ring::BM;
+using ring::BN;
+using ring::NT;
+using ring::OOB;
+using ring::REGION;
+using ring::STAGE;
+using ring::TileRef;
+using ring::EPI_PLAIN;
+using ring::EPI_BIAS;
+using ring::EPI_RELU;
+using ring::EPI_BIAS_RELU;
+using ring::EPI_CLIPPED;
+using ring::EPI_TRANS;
+
+#define SRT_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// acc += b x a (operands are 16 x 32 fragments, the accumulator a 16 x 16 fp32 tile in AGPRs)
+template <typename T>
+__device__ __forceinline__ void mfma16(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a);
+template <>
+__device__ __forceinline__ void mfma16<BF16>(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+template <>
+__device__ __forceinline__ void mfma16<F16>(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a) {
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+
+// Ends the life of the register copies the compiler makes of accumulators (see ring::pin).
+__device__ __forceinline__ void pin_all(f32x4_t (&acc)[8][8]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+}
+
+// ---- global -> LDS --------------------------------------------------------------------------------
+// The ring kernel's loader; an mn-contiguous region gets one more swizzle term.  A 16 x 32
+// fragment read takes its four 16-lane groups from k rows 8 g .. 8 g + 3 (+ 4), which the ring
+// kernel's swizzle (k & 3) puts on the same banks for every g; with bit 3 of k moving the row by
+// two chunks, the two groups served together fall on different banks.
+template <bool KC>
+struct Loader : ring::Loader<KC> {
+  __device__ __forceinline__ void init(int wave, int lane, long long ld) {
+    if constexpr (KC) {
+      ring::Loader<KC>::init(wave, lane, 0, ld);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int krow = (wave * 4 + i) * 2 + (lane >> 5);
+        const int chunk = (lane & 31) ^ ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1);
+        this->voff[i] = (uint32_t)(((long long)krow * ld + chunk * 8) * 2);
+      }
+    }
+  }
+};
+
+// ---- LDS -> MFMA operands: 16 rows x 32 k -------------------------------------------------------
+template <bool KC>
+struct FragReader {
+  uint32_t off[KC ? 1 : 8];   // KC: tile t adds t * 1024; MN: one offset per tile (the swizzle is an XOR)
+
+  // wave_row0: first m (n) of the wave's slice inside the tile (a multiple of 128)
+  __device__ __forceinline__ void init(int lane, int wave_row0) {
+    const int g = lane >> 4, jn = lane & 15;
+    if constexpr (KC) {
+      const int f = (jn >> 2) & 3;   // (row >> 2) & 3 for rows wave_row0 + 16 t + jn
+      off[0] = (uint32_t)((wave_row0 + jn) * 64 + ((g ^ f) << 4));
+    } else {
+      // lane supplies the address of T[k = 8 g + e (+ 4 for the second read)][mn = wave_row0 + 16 t + 4 q]
+      const int e = jn >> 2, q = jn & 3;
+      const int krow = 8 * g + e;
+      const int mn = wave_row0 + 4 * q;   // tile t adds 16: two 16-byte chunks
+      const uint32_t base = (uint32_t)(krow * 512 + ((mn >> 2) & 1) * 8);
+      const int chunk0 = mn >> 3, swz = (e << 2) ^ ((g & 1) << 1);   // k & 3 = e, bit 3 of k = g & 1
+#pragma unroll
+      for (int t = 0; t < 8; ++t) off[t] = base + (uint32_t)(((chunk0 + 2 * t) ^ swz) << 4);
+    }
+  }
+  __device__ __forceinline__ u32x4_t read(uint32_t region, int t) const {
+    if constexpr (KC) {
+      return *reinterpret_cast<const SRT_LDS u32x4_t*>(region + off[0] + t * 1024);
+    } else {
+      const uint32_t a = region + off[t];
+      const u32x2_t lo =
+          __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a)));
+      const u32x2_t hi = __builtin_bit_cast(
+          u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a + 2048)));
+      u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+      return v;
+    }
+  }
+};
+
+// ---- epilogue ------------------------------------------------------------------------------------
+// acc[i][j] is a transposed 16 x 16 tile: lane l owns row m = wave_m0 + 16 i + l % 16 and the
+// columns n = wave_n0 + 16 j + 4 (l / 16) + 0..3.
+template <typename T, bool HAS_BIAS, int CLAMP>
+__device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x4_t (&acc)[8][8], int wave_m0,
+                                                      int wave_n0, int lane) {
+  using S = typename T::storage;
+  const S* bias = (const S*)p.bias;
+  const bool per_row = p.bias_per_row != 0;
+  const float ceiling = p.coef;
+  const int jn = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float bcol[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (HAS_BIAS) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int n = wave_n0 + 16 * j + 4 * g + e;
+        bcol[e] = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float brow = 0.0f;
+      if (HAS_BIAS) {
+        const int m = wave_m0 + 16 * i + jn;
+        brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float x = acc[i][j][e];
+        if (HAS_BIAS) x += per_row ? brow : bcol[e];
+        if (CLAMP >= 1) x = __builtin_fmaxf(x, 0.0f);
+        if (CLAMP == 2) x = __builtin_fminf(x, ceiling);
+        acc[i][j][e] = x;
+      }
+    }
+  }
+}
+
+// One rounding to the element type, then a trip through the wave's 16 KiB staging area at LDS
+// address `stage` so that global stores are whole 16-byte chunks of 256-byte row segments.  Two
+// halves of 64 rows: [64 rows][16 chunks of 16 B], chunk c of row r at position c ^ (r & 15)
+// (conflict-free on both sides: a write instruction covers 16 rows x 32 B, a read 4 whole rows).
+// NaN handling as in ring::store_tile: the hardware converter rounds everything, and when any
+// lane of the wave saw a NaN the staged patterns are rewritten to 0x7FFF on the way out.
+template <typename T>
+__device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0, int wave_n0,
+                                           int bz, int lane, uint32_t stage) {
+  using S = typename T::storage;
+  constexpr bool FIXUP = T::dtype == srtReal16BF;
+  S* C = (S*)p.C + (long long)bz * p.scb;
+  const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
+  const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
+  const int ldc2 = (int)(p.scm * 2);
+  const int jn = lane & 15, g = lane >> 4;
+  const int rd_chunk = lane & 15, rd_row = lane >> 4;   // read side: chunk of rows rd_row + 4 it
+  const int n_rd = wave_n0 + 8 * rd_chunk;
+  const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8 (checked on the host): the chunk is whole
+
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    bool nan = false;
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int i = 4 * half + ii;
+      const int row = 16 * ii + jn;
+      const uint32_t row_addr = stage + (uint32_t)row * 256u + (uint32_t)(g & 1) * 8u;
+      SRT_FENCE();
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float a0 = acc[i][j][0], a1 = acc[i][j][1], a2 = acc[i][j][2], a3 = acc[i][j][3];
+        // one copy out of the accumulator registers, here, for both the test and the conversion
+        asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+        if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
+        const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};
+        const int c = 2 * j + (g >> 1);
+        *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
+      }
+    }
+    SRT_FENCE();
+    const bool fix = FIXUP && __builtin_amdgcn_ballot_w64(nan) != 0;
+    // ---- staging -> global: 16 instructions of 4 rows x 256 bytes, read four at a time ----
+#pragma unroll
+    for (int it4 = 0; it4 < 4; ++it4) {
+      u32x4_t v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 4 * (4 * it4 + q);
+        v[q] = *reinterpret_cast<const SRT_LDS u32x4_t*>(stage + (uint32_t)row * 256u +
+                                                         (uint32_t)((rd_chunk ^ (row & 15)) << 4));
+      }
+      if (fix) {   // rare: some accumulator of this half was a NaN
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[q][e] = ring::canonical_nans_bf16x2(v[q][e]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 4 * (4 * it4 + q);
+        const int m = wave_m0 + 64 * half + row;
+        const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc2 + n_rd * 2) : OOB;
+        __builtin_amdgcn_raw_buffer_store_b128(v[q], rc, (int)off, 0, SRT_STORE_AUX);
+      }
+      SRT_FENCE();
+    }
+  }
+}
+
+// sigmoid / tanh / elu: acc + bias goes to the staging area as fp32 ([32 rows][32 chunks of 16 B],
+// chunk c of row r at c ^ (r & 31)); activation, rounding and store run in a rolled loop.
+template <typename T>
+__device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, const f32x4_t (&acc)[8][8],
+                                                          int wave_m0, int wave_n0, int bz, int lane, uint32_t stage) {
+  using S = typename T::storage;
+  S* C = (S*)p.C + (long long)bz * p.scb;
+  const S* bias = (const S*)p.bias;
+  const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
+  const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
+  const int ldc2 = (int)(p.scm * 2);
+  const bool per_row = p.bias_per_row != 0;
+  const int jn = lane & 15, g = lane >> 4;
+  const int rd_chunk = lane & 31, rd_row = lane >> 5;   // read side: 4 columns of rows rd_row + 2 it
+  const int n_rd = wave_n0 + 4 * rd_chunk;
+  const bool n_rd_ok = n_rd < p.N;
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const int i = 2 * pass + ii;
+      const int row = 16 * ii + jn;
+      const int m = wave_m0 + 16 * i + jn;
+      const float brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        f32x4_t x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int n = wave_n0 + 16 * j + 4 * g + e;
+          const float bcol = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+          x[e] = acc[i][j][e] + (per_row ? brow : bcol);
+        }
+        const int c = 4 * j + g;
+        *reinterpret_cast<SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u + (uint32_t)((c ^ (row & 31)) << 4)) = x;
+      }
+    }
+#pragma unroll 1
+    for (int it = 0; it < 16; ++it) {
+      const int row = rd_row + 2 * it;
+      const f32x4_t x = *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u +
+                                                                  (uint32_t)((rd_chunk ^ (row & 31)) << 4));
+      uint32_t lo = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[0])) |
+                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[1])) << 16);
+      uint32_t hi = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[2])) |
+                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[3])) << 16);
+      const u32x2_t w = {lo, hi};
+      const int mm = wave_m0 + 32 * pass + row;
+      const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
+      __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, SRT_STORE_AUX);
+    }
+    // the rolled loop's reads must have returned before the next pass overwrites the area
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+}
+
+template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
+__global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
+  static_assert(NS == 5, "ring depth");   // slot arithmetic below assumes the staging slots are NS-2, NS-1 ahead
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
+  const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  auto lane_id = []() {
+    uint32_t zero = 0;
+    asm volatile("" : "+s"(zero));   // opaque: keeps the two instructions where they are written
+    return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
+  };
+  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int total = tiles_m * tiles_n * p.batch;
+  const int grid = (int)gridDim.x;
+  int v = (int)blockIdx.x;
+
+  const long long lda = A_KC ? p.sam : p.sak;
+  const long long ldb = B_KC ? p.sbn : p.sbk;
+  const long long a_view = A_KC ? (long long)(p.M - 1) * lda + p.K : (long long)(p.K - 1) * lda + p.M;
+  const long long b_view = B_KC ? (long long)(p.N - 1) * ldb + p.K : (long long)(p.K - 1) * ldb + p.N;
+  const u32x4_t ra = ring::make_rsrc(p.A, (uint32_t)(((long long)(p.batch - 1) * p.sab + a_view) * 2));
+  const u32x4_t rb = ring::make_rsrc(p.B, (uint32_t)(((long long)(p.batch - 1) * p.sbb + b_view) * 2));
+  const uint32_t kstep_a = A_KC ? (uint32_t)(BK * 2) : (uint32_t)(BK * lda * 2);   // bytes per k stage
+  const uint32_t kstep_b = B_KC ? (uint32_t)(BK * 2) : (uint32_t)(BK * ldb * 2);
+  const int KT = (p.K + BK - 1) / BK;
+  const int krem = p.K % BK;   // k values in a ragged last stage (0: the stage is whole)
+  const bool ragged = krem != 0;
+  const bool overlap = !ragged && KT >= NS;
+
+  const int rot = (A_KC || ragged) ? 0 : (int)(((unsigned)(blockIdx.x & 7) * (unsigned)KT) / 8u);
+  auto stage_at = [&](int t) {   // t-th stage of the walk (t < KT)
+    int e = t + rot;
+    if (e >= KT) e -= KT;
+    return e;
+  };
+
+  TileRef cur_tile = ring::locate_tile<A_KC, B_KC>(p, v, tiles_m, tiles_n);
+
+  // Requests stages first .. NS-2 of `tile` and the A part of stage NS-1 (its B part is the first
+  // thing the loop requests); stage t goes to the slot t places after `slot0`.
+  auto fill_ring = [&](const Loader<A_KC>& la, const Loader<B_KC>& lb, int lane, const TileRef& tile, uint32_t slot0,
+                       int first) {
+#pragma unroll
+    for (int t = 0; t < NS; ++t) {
+      if (t < first) continue;
+      uint32_t slot = slot0 + (uint32_t)t * STAGE;
+      if (slot >= lds + NS * STAGE) slot -= NS * STAGE;
+      const bool tail = (t == KT - 1) && ragged;
+      const uint32_t soa = t < KT ? tile.offa + (uint32_t)stage_at(t) * kstep_a : OOB;
+      const uint32_t sob = t < KT ? tile.offb + (uint32_t)stage_at(t) * kstep_b : OOB;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) la.issue_one(ra, slot, wave, lane, soa, i, tail, krem);
+      if (t < NS - 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lb.issue_one(rb, slot + REGION, wave, lane, sob, i, tail, krem);
+      }
+    }
+  };
+
+  uint32_t cur = lds, prv = lds + (NS - 1) * STAGE;
+  const uint32_t wave_lds = (uint32_t)wave * 4096u;   // this wave's 4 KiB share of an operand region
+
+  bool first_tile = true;
+  for (;;) {
+    // per-lane addressing state, derived per tile and scoped to it (see gemm_ring_kernel)
+    Loader<A_KC> la;
+    Loader<B_KC> lb;
+    FragReader<A_KC> fa;
+    FragReader<B_KC> fb;
+    const int lane = lane_id();
+    la.init(wave, lane, lda);
+    lb.init(wave, lane, ldb);
+    fa.init(lane, wm0);
+    fb.init(lane, wn0);
+    if (first_tile || !overlap) {
+      fill_ring(la, lb, lane, cur_tile, cur, 0);
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(8 * (NS - 2) + 4) : "memory");
+    } else {
+      fill_ring(la, lb, lane, cur_tile, cur, NS - 2);
+    }
+    first_tile = false;
+    SRT_FENCE();
+
+    const int vn = v + grid;
+    const bool has_next = vn < total;
+    const TileRef next_tile = ring::locate_tile<A_KC, B_KC>(p, has_next ? vn : v, tiles_m, tiles_n);
+    const bool prefetch = overlap && has_next;
+
+    f32x4_t acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4_t af[8], bf[8];   // the stage's A and B tiles
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      bf[t] = fb.read(cur + REGION, t);
+      af[t] = fa.read(cur, t);
+    }
+    // wait states between the zero fill above (v_accvgpr_write) and the first MFMA reading it
+    asm volatile("s_nop 3" ::: "memory");
+
+    const int limit = prefetch ? KT + NS - 2 : KT;   // requests below this index are real
+    auto stage_of = [&](int r) {
+      int e = r + rot;
+      e = e >= KT ? e - KT : e;
+      e = e >= KT ? e - KT : e;
+      return e;
+    };
+    uint32_t sob, soa = 0;
+    sob = NS - 1 < KT ? cur_tile.offb + (uint32_t)stage_of(NS - 1) * kstep_b : OOB;   // B part of r = NS - 1
+    int e_req = stage_of(NS);                                                         // stage of r = NS
+    uint32_t ea_off = (uint32_t)e_req * kstep_a, eb_off = (uint32_t)e_req * kstep_b;
+
+    // Both phases walk their 4 x 8 MFMA tiles B tile by B tile (u = 4 j + i), so that in phase 1
+    // B tile j is finished with after MFMA 4 j + 3 and its registers can take tile j of the next
+    // stage -- one register set per operand is enough.  Tiles 0-3 of both operands are read in
+    // phase 1 of the stage before, tiles 4-7 in phase 0 of their own stage: eight fragment reads
+    // per phase, at most one every other MFMA (an MFMA is 16 cycles, an instruction issues in 4).  The loop exists twice (ragged /
+    // whole last stage) like the ring kernel's.
+    auto k_loop = [&](auto ragged_tag) __attribute__((always_inline)) {
+    constexpr bool RAGGED = decltype(ragged_tag)::value;
+    for (int kt = 0; kt < KT; ++kt) {
+      uint32_t nxt = cur + STAGE;
+      if (nxt == lds + NS * STAGE) nxt = lds;
+      const int kb = kt - 1 + NS;
+      const int ka = kt + NS;
+      uint32_t sob_next = OOB;
+      if (RAGGED) {
+        if (kb == KT - 1) lb.mask_tail(wave, lane, krem);
+        if (ka == KT - 1) la.mask_tail(wave, lane, krem);
+      }
+      // ---- phase 0: A tiles 0-3 ----
+      const uint32_t b_target = prv + REGION + wave_lds;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int u = j * 4 + i;   // 0..31
+          const bool load_here = u >= 16 && (u & 3) == 0;   // 16, 20, 24, 28
+          if (u == 16) ring::set_lds_target<0>(b_target);
+          if (u == 20) ring::set_lds_target<1024>(b_target);
+          if (u == 24) ring::set_lds_target<2048>(b_target);
+          if (u == 28) ring::set_lds_target<3072>(b_target);
+          if (load_here) SRT_FENCE();
+          mfma16<T>(acc[i][j], bf[j], af[i]);
+          if (load_here) {
+            SRT_FENCE();
+            ring::load_to_lds_at_m0(rb, lb.voff[(u - 16) >> 2], sob);
+          }
+          // the rest of stage kt: B tiles 4-7 (first used by MFMA 16), A tiles 4-7 (phase 1)
+          if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.read(cur + REGION, 4 + (u >> 1));
+          if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.read(cur, 4 + ((u - 8) >> 1));
+          if (u == 17) soa = ka < limit ? (ka < KT ? cur_tile.offa : next_tile.offa) + ea_off : OOB;
+          if (u == 19) sob_next = ka < limit ? (ka < KT ? cur_tile.offb : next_tile.offb) + eb_off : OOB;
+          if (u == 21) {
+            const bool wrap = e_req + 1 == KT;
+            e_req = wrap ? 0 : e_req + 1;
+            ea_off = wrap ? 0u : ea_off + kstep_a;
+            eb_off = wrap ? 0u : eb_off + kstep_b;
+          }
+          SRT_FENCE();
+        }
+      }
+      // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(8 * (NS - 2)) : "memory");
+      SRT_FENCE();
+      // ---- phase 1: A tiles 4-7; A loads of stage kt+NS; reads of stage kt+1 ----
+      const uint32_t a_target = cur + wave_lds;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int u = j * 4 + i;   // 0..31
+          const bool load_here = u < 16 && (u & 3) == 0;   // 0, 4, 8, 12
+          if (u == 0) ring::set_lds_target<0>(a_target);
+          if (u == 4) ring::set_lds_target<1024>(a_target);
+          if (u == 8) ring::set_lds_target<2048>(a_target);
+          if (u == 12) ring::set_lds_target<3072>(a_target);
+          if (load_here) SRT_FENCE();
+          mfma16<T>(acc[4 + i][j], bf[j], af[4 + i]);
+          if (load_here) {
+            SRT_FENCE();
+            ring::load_to_lds_at_m0(ra, la.voff[u >> 2], soa);
+          }
+          // stage kt+1: A tiles 0-3 (idle since phase 0) and B tiles 0-3, each as it falls free
+          if (u < 16 && i == 1) af[j] = fa.read(nxt, j);
+          if (u < 16 && i == 3) bf[j] = fb.read(nxt + REGION, j);
+          SRT_FENCE();
+        }
+      }
+      prv = cur;
+      cur = nxt;
+      sob = sob_next;
+    }
+    };
+    if (ragged) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
+
+    // Every load in flight must have landed, in every wave, before the slots vacated last become
+    // the staging area.  The s_nops are the wait states between the last MFMAs and the first
+    // reads of their accumulators by other instructions.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+    // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1 (16 KiB each)
+    uint32_t pprv = prv - STAGE;
+    if (prv == lds) pprv = lds + (NS - 1) * STAGE;
+    const uint32_t stage = ((wave & 2) ? prv : pprv) + (uint32_t)(wave & 1) * 16384u;
+    const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
+    const int le = lane_id();
+
+    if (EPI == EPI_TRANS) {
+      store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
+    } else {
+      if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
+      else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1>(p, acc, em0, en0, le);
+      else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1>(p, acc, em0, en0, le);
+      else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2>(p, acc, em0, en0, le);
+      if (EPI != EPI_PLAIN) pin_all(acc);
+      store_tile<T>(p, acc, em0, en0, bz, le, stage);
+    }
+    if (!has_next) break;
+
+    // every wave has finished reading its staging area before any wave's loads overwrite it
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    v = vn;
+    cur_tile = next_tile;
+  }
+}
+
+#undef SRT_FENCE
+
+template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
+hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_m16_kernel<T, A_KC, B_KC, EPI, NS>;
+  constexpr int lds_bytes = NS * STAGE;
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
+  const long long tiles = (long long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN) * p.batch;
+  int grid = ring::compute_units() & ~7;
+  if (grid <= 0) grid = 8;
+  if (tiles < grid) grid = (int)tiles;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
+  return hipGetLastError();
+}
+
+template <typename T, bool A_KC, bool B_KC, int NS = 5>
+hipError_t launch(const GemmProblem& p, hipStream_t stream) {
+  const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
+                     p.activation == srtActivationElu;
+  if (trans) return launch_kernel<T, A_KC, B_KC, EPI_TRANS, NS>(p, stream);
+  if (p.activation == srtActivationClippedRelu) return launch_kernel<T, A_KC, B_KC, EPI_CLIPPED, NS>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS_RELU, NS>(p, stream);
+    return launch_kernel<T, A_KC, B_KC, EPI_RELU, NS>(p, stream);
+  }
+  if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS, NS>(p, stream);
+  return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS>(p, stream);
+}
+
+}  // namespace m16
+}  // namespace srt

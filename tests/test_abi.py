@@ -192,10 +192,14 @@ def test_kernel_selection_is_queryable_without_gpu():
         assert st == 0
         return buf.value.decode()
 
-    assert query(native.REAL16BF, 8192, 8192, 8192) == "mfma_256x256"
-    assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256"
-    assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256"
-    assert query(native.REAL16BF, 8192, 8192, 8192, tb=True) == "mfma_256x256_k64"   # both operands k-contiguous
+    # a full device and a long k loop: the 256 x 256 ring on 16x16x32 MFMAs, in every layout
+    assert query(native.REAL16BF, 8192, 8192, 8192) == "mfma_256x256_m16"
+    assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256_m16"
+    assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256_m16"
+    assert query(native.REAL16BF, 8192, 8192, 8192, tb=True) == "mfma_256x256_m16"
+    # short k loops: the 32x32x16 kernels (64-deep stages when both operands are k-contiguous)
+    assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256"
+    assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_k64"
     # mid-size problems: the 256 x 256 kernels from 48 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256"                 # 144 tiles

@@ -294,7 +294,7 @@ def test_cfg3_bf16_8192_sampled_rows_and_invariants(ta):
     a = H.encode((r.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n))), H.BF16)
     b = H.encode((r.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n))), H.BF16)
     a_stored = np.ascontiguousarray(a.T) if ta else a
-    got = gpu_matmul(a_stored, b, ta=ta, want_kernel="mfma_256x256")
+    got = gpu_matmul(a_stored, b, ta=ta, want_kernel="mfma_256x256_m16")
     rows = np.unique(np.concatenate([np.arange(0, n, 131), [n - 1, 255, 256, 4095, 4096]]))
     c64 = H.to64(a[rows]) @ H.to64(b)
     absprod = np.abs(H.to64(a[rows])) @ np.abs(H.to64(b))
@@ -420,6 +420,99 @@ def test_ring_kernel_epilogues_vs_oracle(act, dt):
     want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, acc=ora.ACC_F32, fused=True))
     tol = {H.F16: 2.0 ** -10, H.BF16: 2.0 ** -7}[dt]
     assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
+
+
+# ---- the 256 x 256 ring kernel on 16x16x32 MFMAs ----------------------------------------------------
+def pin_m16(tmp_path, dt, M, N, K, ta, tb, batch=1, bias=False, act=srt.ActivationType.identity):
+    """The heuristic takes this kernel for a full device and a long k loop only: pin it for a small shape."""
+    layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
+    epilogue = (1 if bias else 0) | (int(act) << 1)
+    f = tmp_path / "plan.txt"
+    f.write_text(f"{dt} {M} {N} {K} {batch} {layout} {epilogue} mfma_256x256_m16\n")
+    srt.PlanCache.clear()
+    srt.PlanCache.load(f)
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_m16_kernel_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
+    """Every staging layout; ragged edges in M and N, K of one stage, ending inside a stage, with an
+    even and an odd number of stages, fewer stages than the ring holds; several tiles per workgroup."""
+    r = H.rng(300)
+    for (M, N, K) in [(512, 512, 32), (512, 768, 160), (1000, 520, 72), (2048, 2056, 200), (4400, 4360, 328)]:
+        pin_m16(tmp_path, dt, M, N, K, ta, tb)
+        a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+        got = gpu_matmul(H.encode(a, dt), H.encode(b, dt), ta, tb, want_kernel="mfma_256x256_m16")
+        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    M, N, K = 2040, 2056, 264
+    pin_m16(tmp_path, dt, M, N, K, ta, tb)
+    a = (r.standard_normal((K, M) if ta else (M, K)) / np.sqrt(K)).astype(np.float32)
+    b = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    a_st, b_st = H.encode(a, dt), H.encode(b, dt)
+    check_against_fp64(gpu_matmul(a_st, b_st, ta, tb, want_kernel="mfma_256x256_m16"), a_st, b_st, ta, tb, dt)
+    srt.PlanCache.clear()
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("act", list(srt.ActivationType))
+@pytest.mark.parametrize("tw", [False, True])
+def test_m16_kernel_epilogues_vs_oracle(act, dt, tw, tmp_path):
+    """y = act(x . W + b) and act(x . W^T + b): every activation through the fused epilogue, ragged M / N
+    edges and a K that ends inside a stage."""
+    r = H.rng(19)
+    M, N, K = 2100, 2056, 200
+    x = H.encode(r.standard_normal((M, K)).astype(np.float32), dt)
+    w = H.encode((r.standard_normal((N, K) if tw else (K, N)) / 8).astype(np.float32), dt)
+    b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
+    coef = 0.75
+    pin_m16(tmp_path, dt, M, N, K, False, tw, bias=True, act=act)
+    xt, wt, bt = srt.Tensor(x), srt.Tensor(w), srt.Tensor(b)
+    out = srt.Tensor(shape=[M, N], dtype=x.dtype)
+    srt.current_queue().matmul(xt, False, wt, tw, out, bias=bt, activation=act, coef=coef)
+    got = H.decode(out.array())
+    rows = np.concatenate([np.arange(0, M, 131), [M - 1]])
+    want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, transpose_w=tw,
+                                      acc=ora.ACC_F32, fused=True))
+    tol = {H.F16: 2.0 ** -10, H.BF16: 2.0 ** -7}[dt]
+    assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
+    srt.PlanCache.clear()
+
+
+def test_m16_kernel_batched_short_k_and_nan(tmp_path):
+    """Strided batch, K shorter than one stage (8) and of one, two and three stages, a NaN row."""
+    r = H.rng(20)
+    for K in (8, 32, 72, 136, 192):
+        B_, M, N = 3, 1024, 1032
+        a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+        w = r.integers(-3, 4, (B_, K, N)).astype(np.float32)
+        pin_m16(tmp_path, H.BF16, M, N, K, False, False, batch=B_)
+        at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+        out = srt.matmul(at, wt)
+        assert query_kernel(at, False, wt, False, out) == "mfma_256x256_m16"
+        exact = a.astype(np.int64) @ w.astype(np.int64)
+        assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), H.BF16)), K
+    M = N = 1536
+    a = np.zeros((M, 64), np.float32)
+    w = np.zeros((64, N), np.float32)
+    a[:, 0] = 1.0
+    w[0, :] = 2.0
+    a[5, 1] = np.nan
+    w[1, :] = 1.0
+    pin_m16(tmp_path, H.BF16, M, N, 64, False, False)
+    got = gpu_matmul(H.encode(a, H.BF16), H.encode(w, H.BF16), want_kernel="mfma_256x256_m16")
+    assert np.all(got[5] == 0x7FFF) and np.all(got[6] == H.encode(np.array([2.0], np.float32), H.BF16)[0])
+    srt.PlanCache.clear()
+
+
+def test_m16_kernel_is_the_choice_for_a_full_device_and_long_k():
+    a = srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16))
+    b = srt.Tensor(H.encode(np.zeros((2048, 4096), np.float32), H.BF16))
+    out = srt.Tensor(shape=[4096, 4096], dtype=a.dtype)
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_m16"
+    assert query_kernel(a, False, srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16)), True, out) == \
+        "mfma_256x256_m16"
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
