@@ -142,7 +142,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=8192, row-major, no transposes, fp32 accumulate, bf16 out; "
                                "A,B ~ N(0,1)/sqrt(K) seed 2; inputs resident in HBM",
-                   "entry_point": "srtMatmul", "kernel": "gemm_ring_kernel<BF16> 256x256x32, 5-stage LDS ring, persistent (one workgroup per CU)"},
+                   "entry_point": "srtMatmul", "kernel": "gemm_m16_kernel<BF16> 256x256x32, v_mfma_f32_16x16x32, 5-stage LDS ring, persistent (one workgroup per CU)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": TRAFFIC_BYTES_8192},
         "max_rel_err_vs_fp64": max_rel,
@@ -168,7 +168,7 @@ def main():
 
 def mfma_ceiling():
     """Runs the stand-alone probe built next to the library (a child process; the GPU is idle while
-    it runs): a loop of v_mfma_f32_32x32x16_bf16 on register operands, once with operands from the
+    it runs): a loop of v_mfma_f32_16x16x32_bf16 (the GEMM kernel's instruction) on register operands, once with operands from the
     GEMM's input distribution and once with zeros.  The first figure is what the matrix cores sustain
     on this device under its power limit -- the practical ceiling for a GEMM on such data; the
     published peak stays the denominator of `roofline.frac`."""

@@ -401,19 +401,21 @@ int mfma_select(const GemmProblem& p) {
   //    against 88 us) and then the 64-deep 256 x 256 kernel takes over (whole-line loads where
   //    the ring kernel moves half lines: 4096^3 NT 114 us against 126 us, 8192^3 NT 1351 against
   //    1336 TFLOP/s);
-  //  * once the device is three quarters full and the k loop is long, sustained speed is set by
-  //    the power limit, and the 16x16x32 form of the ring kernel, cheaper per flop, wins in every
-  //    layout (8192^3: 1390-1440 against 1300-1350 TFLOP/s; 4096 x 11008 x 4096: 292 us against
-  //    306-320 us).  Its loop has less slack per MFMA, so where clocks are not the limit -- a
-  //    partly filled device -- the 32x32x16 kernels stay ahead (2048^3: 42 us against 45 us),
-  //    and with short k loops (K = 1024) nothing separates them;
+  //  * once the device is half full and the k loop is long, sustained speed is set by the power
+  //    limit, and the 16x16x32 form of the ring kernel, cheaper per flop, wins in every layout
+  //    (8192^3: 1410-1490 against 1340-1390 TFLOP/s; 4096 x 11008 x 4096: 280 us against
+  //    298-308 us; 3072^3, 144 tiles: 68 us against 71 us; 2048 x 4096 x 4096, 128 tiles: 84 us
+  //    against 85 us).  Its loop has less slack per MFMA, so where clocks are not the limit -- a
+  //    partly filled device -- the 32x32x16 kernels stay ahead (2048^3: 42 us against 43.5 us;
+  //    1024 x 4096 x 4096: 73 us against 77 us), and with short k loops (K = 1024) nothing
+  //    separates them;
   //  * below those thresholds every CU should get a workgroup: 64 x 64 tiles (batch 32 x 256^3:
   //    7.7 us against 15.0 us with 128 x 128).  128 x 128 is kept for problems that do not meet
   //    the 256 x 256 kernels' preconditions but have at least one such tile per CU.
   const bool big_ok = ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0);
   const long long t256 = tiles(256);
   int tile;
-  if (big_ok && t256 >= 192 && p.K >= 2048) tile = 5;
+  if (big_ok && t256 >= 128 && p.K >= 2048) tile = 5;
   else if (big_ok && layout == 3 && t256 >= 192) tile = 4;
   else if (big_ok && t256 >= (layout == 3 ? 96 : 48)) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;

@@ -1,6 +1,6 @@
 // 256 x 256 bf16 / fp16 matmul tile kernel for gfx950 on v_mfma_f32_16x16x32: the persistent,
-// direct-to-LDS ring of gemm_mfma_ring.h (same LDS layouts, loaders, tile walk and cross-tile
-// prefetch -- see there) with the 128 x 128 wave tile cut into 8 x 8 MFMA tiles of 16 x 16
+// direct-to-LDS ring of gemm_mfma_ring.h (same stage layout, tile walk and cross-tile prefetch --
+// see there; swizzles of its own) with the 128 x 128 wave tile cut into 8 x 8 MFMA tiles of 16 x 16
 // instead of 4 x 4 tiles of 32 x 32.
 //
 // Why a second instruction shape.  On N(0,1) data this part runs against its power limit, and
@@ -84,23 +84,64 @@ __device__ __forceinline__ void pin_all(f32x4_t (&acc)[8][8]) {
 }
 
 // ---- global -> LDS --------------------------------------------------------------------------------
-// The ring kernel's loader; an mn-contiguous region gets one more swizzle term.  A 16 x 32
-// fragment read takes its four 16-lane groups from k rows 8 g .. 8 g + 3 (+ 4), which the ring
-// kernel's swizzle (k & 3) puts on the same banks for every g; with bit 3 of k moving the row by
-// two chunks, the two groups served together fall on different banks.
+// The ring kernel's loader (four loads per wave, operand and stage; lane l of a load lands at
+// LDS byte M0 + 16 l, so the swizzle is applied on the global side) with the swizzles that make
+// 16 x 32 fragment reads free of bank conflicts.  The ring kernel's own do not: its k-contiguous
+// swizzle (row >> 2) & 3 costs a 16-row ds_read_b128 4 extra cycles (8.0 against 4.75 per
+// instruction at full LDS load), and its mn-contiguous one puts the four 16-lane groups of a
+// ds_read_b64_tr_b16, which come from k rows 8 g .. 8 g + 3, on the same banks for every g.
+//   k-contiguous:  [256 rows][4 chunks of 16 B], chunk c of row r at position c ^ ((r >> 1) & 3)
+//   mn-contiguous: [32 k][32 chunks of 16 B], chunk c of k row k at c ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1)
 template <bool KC>
-struct Loader : ring::Loader<KC> {
+struct Loader {
+  uint32_t voff[4];
+
+  // ld: elements between rows (KC) or between k (MN)
   __device__ __forceinline__ void init(int wave, int lane, long long ld) {
     if constexpr (KC) {
-      ring::Loader<KC>::init(wave, lane, 0, ld);
+      // load i of this wave covers tile rows (wave*4 + i)*16 .. +15, 4 lanes per 64-byte row
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = (wave * 4 + i) * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ ((row >> 1) & 3);
+        voff[i] = (uint32_t)(((long long)row * ld + chunk * 8) * 2);
+      }
     } else {
+      // load i covers k rows (wave*4 + i)*2 .. +1, 32 lanes per 512-byte k row
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int krow = (wave * 4 + i) * 2 + (lane >> 5);
         const int chunk = (lane & 31) ^ ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1);
-        this->voff[i] = (uint32_t)(((long long)krow * ld + chunk * 8) * 2);
+        voff[i] = (uint32_t)(((long long)krow * ld + chunk * 8) * 2);
       }
     }
+  }
+
+  // does load i of this lane fetch k values at or beyond K in a ragged last stage of krem values?
+  __device__ __forceinline__ bool beyond_k(int wave, int lane, int i, int krem) const {
+    if constexpr (KC) {
+      const int chunk = (lane & 3) ^ ((lane >> 3) & 3);   // (row >> 1) & 3 depends on the lane only
+      return chunk >= (krem + 7) / 8;
+    } else {
+      return (wave * 4 + i) * 2 + (lane >> 5) >= krem;
+    }
+  }
+
+  // Load i of this wave for the k stage at scalar byte offset `soff` (or OOB: the load reads zeros
+  // without touching memory) into the operand region at LDS address `region`; `tail`: a ragged
+  // last stage holding only `krem` k values, what lies at or beyond K must read as zero.
+  __device__ __forceinline__ void issue_one(u32x4_t rsrc, uint32_t region, int wave, int lane, uint32_t soff, int i,
+                                            bool tail, int krem) const {
+    uint32_t v = voff[i];
+    if (tail && beyond_k(wave, lane, i, krem)) v = OOB;
+    ring::load_to_lds(rsrc, region + (uint32_t)(wave * 4 + i) * 1024u, v, soff);
+  }
+
+  // aims what lies at or beyond K out of range for good (the state is derived afresh per tile)
+  __device__ __forceinline__ void mask_tail(int wave, int lane, int krem) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (beyond_k(wave, lane, i, krem)) voff[i] = OOB;
   }
 };
 
@@ -113,7 +154,7 @@ struct FragReader {
   __device__ __forceinline__ void init(int lane, int wave_row0) {
     const int g = lane >> 4, jn = lane & 15;
     if constexpr (KC) {
-      const int f = (jn >> 2) & 3;   // (row >> 2) & 3 for rows wave_row0 + 16 t + jn
+      const int f = (jn >> 1) & 3;   // (row >> 1) & 3 for rows wave_row0 + 16 t + jn
       off[0] = (uint32_t)((wave_row0 + jn) * 64 + ((g ^ f) << 4));
     } else {
       // lane supplies the address of T[k = 8 g + e (+ 4 for the second read)][mn = wave_row0 + 16 t + 4 q]
@@ -428,23 +469,24 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     // Both phases walk their 4 x 8 MFMA tiles B tile by B tile (u = 4 j + i), so that in phase 1
     // B tile j is finished with after MFMA 4 j + 3 and its registers can take tile j of the next
     // stage -- one register set per operand is enough.  Tiles 0-3 of both operands are read in
-    // phase 1 of the stage before, tiles 4-7 in phase 0 of their own stage: eight fragment reads
-    // per phase, at most one every other MFMA (an MFMA is 16 cycles, an instruction issues in 4).  The loop exists twice (ragged /
-    // whole last stage) like the ring kernel's.
-    auto k_loop = [&](auto ragged_tag) __attribute__((always_inline)) {
-    constexpr bool RAGGED = decltype(ragged_tag)::value;
-    for (int kt = 0; kt < KT; ++kt) {
-      uint32_t nxt = cur + STAGE;
-      if (nxt == lds + NS * STAGE) nxt = lds;
+    // phase 1 of the stage before, tiles 4-7 in phase 0 of their own stage.
+    // An MFMA occupies the matrix pipe for 16 cycles and the wave issues one instruction every
+    // four, so no gap between two MFMAs should hold more than three other instructions.  Fragment
+    // reads take the first half of each phase (one every other MFMA), the loads the second half
+    // (one every fourth), and the scalar bookkeeping of the requests is dealt out over the odd
+    // slots of the second halves, a few instructions each.
+    uint32_t b_target = prv + REGION + wave_lds;   // landing address of the next B request
+    auto one_stage = [&](auto ragged_tag, int kt) __attribute__((always_inline)) {
+      constexpr bool RAGGED = decltype(ragged_tag)::value;
       const int kb = kt - 1 + NS;
       const int ka = kt + NS;
-      uint32_t sob_next = OOB;
       if (RAGGED) {
         if (kb == KT - 1) lb.mask_tail(wave, lane, krem);
         if (ka == KT - 1) la.mask_tail(wave, lane, krem);
       }
+      uint32_t nxt = 0, a_target = 0, sel = 0, sob_next = OOB;
+      bool wrap = false;
       // ---- phase 0: A tiles 0-3 ----
-      const uint32_t b_target = prv + REGION + wave_lds;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
 #pragma unroll
@@ -464,48 +506,67 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
           // the rest of stage kt: B tiles 4-7 (first used by MFMA 16), A tiles 4-7 (phase 1)
           if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.read(cur + REGION, 4 + (u >> 1));
           if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.read(cur, 4 + ((u - 8) >> 1));
-          if (u == 17) soa = ka < limit ? (ka < KT ? cur_tile.offa : next_tile.offa) + ea_off : OOB;
-          if (u == 19) sob_next = ka < limit ? (ka < KT ? cur_tile.offb : next_tile.offb) + eb_off : OOB;
-          if (u == 21) {
-            const bool wrap = e_req + 1 == KT;
-            e_req = wrap ? 0 : e_req + 1;
-            ea_off = wrap ? 0u : ea_off + kstep_a;
-            eb_off = wrap ? 0u : eb_off + kstep_b;
-          }
+          if (u == 17) nxt = cur + STAGE;
+          if (u == 19) nxt = nxt == lds + NS * STAGE ? lds : nxt;
+          // request r = ka: its A part goes out in phase 1, its B part in phase 0 of the next stage
+          if (u == 21) sel = ka < KT ? cur_tile.offa : next_tile.offa;
+          if (u == 23) soa = ka < limit ? sel + ea_off : OOB;
+          if (u == 25) sel = ka < KT ? cur_tile.offb : next_tile.offb;
+          if (u == 27) sob_next = ka < limit ? sel + eb_off : OOB;
+          if (u == 29) a_target = cur + wave_lds;
           SRT_FENCE();
         }
       }
       // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(8 * (NS - 2)) : "memory");
       SRT_FENCE();
-      // ---- phase 1: A tiles 4-7; A loads of stage kt+NS; reads of stage kt+1 ----
-      const uint32_t a_target = cur + wave_lds;
+      // ---- phase 1: A tiles 4-7; reads of stage kt+1; A loads of stage kt+NS ----
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int u = j * 4 + i;   // 0..31
-          const bool load_here = u < 16 && (u & 3) == 0;   // 0, 4, 8, 12
-          if (u == 0) ring::set_lds_target<0>(a_target);
-          if (u == 4) ring::set_lds_target<1024>(a_target);
-          if (u == 8) ring::set_lds_target<2048>(a_target);
-          if (u == 12) ring::set_lds_target<3072>(a_target);
+          const bool load_here = u >= 16 && (u & 3) == 0;   // 16, 20, 24, 28
+          if (u == 16) ring::set_lds_target<0>(a_target);
+          if (u == 20) ring::set_lds_target<1024>(a_target);
+          if (u == 24) ring::set_lds_target<2048>(a_target);
+          if (u == 28) ring::set_lds_target<3072>(a_target);
           if (load_here) SRT_FENCE();
           mfma16<T>(acc[4 + i][j], bf[j], af[4 + i]);
           if (load_here) {
             SRT_FENCE();
-            ring::load_to_lds_at_m0(ra, la.voff[u >> 2], soa);
+            ring::load_to_lds_at_m0(ra, la.voff[(u - 16) >> 2], soa);
           }
           // stage kt+1: A tiles 0-3 (idle since phase 0) and B tiles 0-3, each as it falls free
           if (u < 16 && i == 1) af[j] = fa.read(nxt, j);
           if (u < 16 && i == 3) bf[j] = fb.read(nxt + REGION, j);
+          // the stage of request r = ka + 1, and where its B part will land
+          if (u == 17) {
+            wrap = e_req + 1 == KT;
+            e_req = wrap ? 0 : e_req + 1;
+          }
+          if (u == 19) ea_off = wrap ? 0u : ea_off + kstep_a;
+          if (u == 21) eb_off = wrap ? 0u : eb_off + kstep_b;
+          if (u == 23) b_target = cur + REGION + wave_lds;
           SRT_FENCE();
         }
       }
       prv = cur;
       cur = nxt;
       sob = sob_next;
-    }
+    };
+    // The loop exists twice (ragged / whole last stage) like the ring kernel's; the common one is
+    // unrolled by two, which halves the loop's own bookkeeping.
+    auto k_loop = [&](auto ragged_tag) __attribute__((always_inline)) {
+      constexpr bool RAGGED = decltype(ragged_tag)::value;
+      int kt = 0;
+      if (!RAGGED) {
+        for (; kt + 1 < KT; kt += 2) {
+          one_stage(ragged_tag, kt);
+          one_stage(ragged_tag, kt + 1);
+        }
+      }
+      for (; kt < KT; ++kt) one_stage(ragged_tag, kt);
     };
     if (ragged) k_loop(std::true_type{});
     else k_loop(std::false_type{});

@@ -202,7 +202,8 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_k64"
     # mid-size problems: the 256 x 256 kernels from 48 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
-    assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256"                 # 144 tiles
+    assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16"             # 144 tiles, long k loop
+    assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256"
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_256x256"                 # 64 tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_64x64"                    # 32 tiles
