@@ -30,8 +30,8 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# and scaled by a 256 MiB device copy (profiles/gemm_ring_bf16_8192_counters.txt).
-TRAFFIC_BYTES_8192 = 1.747e9   # 2.000 x FETCH_SIZE (787 645 KiB) + 1.000 x WRITE_SIZE (131 115 KiB)
+# and scaled by a 256 MiB device copy (profiles/gemm_m16_bf16_8192_counters.txt).
+TRAFFIC_BYTES_8192 = 1.816e9   # 2.000 x FETCH_SIZE (820 971 KiB) + 1.000 x WRITE_SIZE (131 111 KiB)
 
 
 def rng(seed):
@@ -168,9 +168,10 @@ def main():
 
 def mfma_ceiling():
     """Runs the stand-alone probe built next to the library (a child process; the GPU is idle while
-    it runs): a loop of v_mfma_f32_16x16x32_bf16 (the GEMM kernel's instruction) on register operands, once with operands from the
-    GEMM's input distribution and once with zeros.  The first figure is what the matrix cores sustain
-    on this device under its power limit -- the practical ceiling for a GEMM on such data; the
+    it runs): a loop of v_mfma_f32_16x16x32_bf16 (the GEMM kernel's instruction) on register operands
+    with the accumulator set of the kernel's wave tile, timed inside the kernel, once with operands
+    from the GEMM's input distribution and once with zeros.  The first figure is what the matrix cores
+    sustain on this device under its power limit -- the practical ceiling for a GEMM on such data; the
     published peak stays the denominator of `roofline.frac`."""
     import subprocess
     exe = os.path.join(ROOT, "swiftrt_amd", "lib", "mfma_ceiling")

@@ -210,8 +210,8 @@ srtStatus srtMatmulBiasActivation(const void* a, const srtTensorDescriptor* aDes
                                   srtActivation activation, double coef,
                                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 
-/* Name of the kernel family the dispatcher selects for this problem ("mfma_256x256",
- * "skinny", "generic", ...), written into `name`; nothing is launched.  Diagnostic only
+/* Name of the kernel family the dispatcher selects for this problem ("mfma_256x256_m16",
+ * "mfma_256x256", "skinny", "generic", ...), written into `name`; nothing is launched.  Diagnostic only
  * (the reference's matmul diagnostic line, CudaMatmul.swift:34-37, has no counterpart for
  * kernel choice). */
 srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transposeA,
@@ -234,8 +234,8 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
  * call's pointers still meet the plan's alignment rules; otherwise, and for keys never tuned, the
  * built-in heuristic decides.  All plans compute the same function to the documented tolerance
  * (sums are fp32; their order differs between plans).
- * chosen (optional): receives the plan's name ("mfma_256x256", "mfma_128x128", "mfma_64x64", "skinny",
- * "f32_mfma_64x64", "f32_mfma_splitk", "generic").
+ * chosen (optional): receives the plan's name ("mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
+ * "mfma_128x128", "mfma_64x64", "skinny", "f32_mfma_64x64", "f32_mfma_splitk", "generic").
  * The cache is thread-safe.  Save / Load use a small text file, one plan per line:
  *   dtype M N K batch layout epilogue plan-name
  * (layout: bit 0 A contiguous along k, 1 A along m, 2 B along k, 3 B along n, 4 result rows
