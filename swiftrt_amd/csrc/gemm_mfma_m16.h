@@ -20,7 +20,7 @@
 // spare registers with v_accvgpr moves between the MFMAs (measured on an MFMA-only loop: 1760
 // instead of 2435 TFLOP/s on zeros).  The compiler does not know the statement is an MFMA, so the
 // wait states the hardware needs between an MFMA and a dependent non-MFMA access of its
-// accumulator are written out where they could matter (after the k loop, after the zero fill).
+// accumulator are written out where they could matter (after the k loop).
 //
 // An MFMA operand is 16 rows x 32 k: lane l holds row l % 16, k = 8 (l / 16) .. + 7 -- one
 // ds_read_b128 from a k-contiguous region, two ds_read_b64_tr_b16 from an mn-contiguous one.
@@ -73,6 +73,19 @@ __device__ __forceinline__ void mfma16<BF16>(f32x4_t& acc, const u32x4_t& b, con
 template <>
 __device__ __forceinline__ void mfma16<F16>(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a) {
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(b), "v"(a));
+}
+
+// acc = b x a: the first MFMA of a tile takes the constant 0 as its addend, which saves zeroing the
+// 256 accumulator registers of every tile (and the wait states between that and the first MFMA)
+template <typename T>
+__device__ __forceinline__ void mfma16_first(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a);
+template <>
+__device__ __forceinline__ void mfma16_first<BF16>(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a));
+}
+template <>
+__device__ __forceinline__ void mfma16_first<F16>(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a) {
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a));
 }
 
 // Ends the life of the register copies the compiler makes of accumulators (see ring::pin).
@@ -439,11 +452,7 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     const TileRef next_tile = ring::locate_tile<A_KC, B_KC>(p, has_next ? vn : v, tiles_m, tiles_n);
     const bool prefetch = overlap && has_next;
 
-    f32x4_t acc[8][8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4_t acc[8][8];   // defined by the MFMAs of the tile's first stage
 
     u32x4_t af[8], bf[8];   // the stage's A and B tiles
 #pragma unroll
@@ -451,8 +460,6 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
       bf[t] = fb.read(cur + REGION, t);
       af[t] = fa.read(cur, t);
     }
-    // wait states between the zero fill above (v_accvgpr_write) and the first MFMA reading it
-    asm volatile("s_nop 3" ::: "memory");
 
     const int limit = prefetch ? KT + NS - 2 : KT;   // requests below this index are real
     auto stage_of = [&](int r) {
@@ -476,8 +483,9 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     // (one every fourth), and the scalar bookkeeping of the requests is dealt out over the odd
     // slots of the second halves, a few instructions each.
     uint32_t b_target = prv + REGION + wave_lds;   // landing address of the next B request
-    auto one_stage = [&](auto ragged_tag, int kt) __attribute__((always_inline)) {
+    auto one_stage = [&](auto ragged_tag, auto first_tag, int kt) __attribute__((always_inline)) {
       constexpr bool RAGGED = decltype(ragged_tag)::value;
+      constexpr bool FIRST = decltype(first_tag)::value;   // the tile's first stage: accumulators start here
       const int kb = kt - 1 + NS;
       const int ka = kt + NS;
       if (RAGGED) {
@@ -498,7 +506,8 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
           if (u == 24) ring::set_lds_target<2048>(b_target);
           if (u == 28) ring::set_lds_target<3072>(b_target);
           if (load_here) SRT_FENCE();
-          mfma16<T>(acc[i][j], bf[j], af[i]);
+          if constexpr (FIRST) mfma16_first<T>(acc[i][j], bf[j], af[i]);
+          else mfma16<T>(acc[i][j], bf[j], af[i]);
           if (load_here) {
             SRT_FENCE();
             ring::load_to_lds_at_m0(rb, lb.voff[(u - 16) >> 2], sob);
@@ -532,7 +541,8 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
           if (u == 24) ring::set_lds_target<2048>(a_target);
           if (u == 28) ring::set_lds_target<3072>(a_target);
           if (load_here) SRT_FENCE();
-          mfma16<T>(acc[4 + i][j], bf[j], af[4 + i]);
+          if constexpr (FIRST) mfma16_first<T>(acc[4 + i][j], bf[j], af[4 + i]);
+          else mfma16<T>(acc[4 + i][j], bf[j], af[4 + i]);
           if (load_here) {
             SRT_FENCE();
             ring::load_to_lds_at_m0(ra, la.voff[(u - 16) >> 2], soa);
@@ -559,14 +569,15 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     // unrolled by two, which halves the loop's own bookkeeping.
     auto k_loop = [&](auto ragged_tag) __attribute__((always_inline)) {
       constexpr bool RAGGED = decltype(ragged_tag)::value;
-      int kt = 0;
+      one_stage(ragged_tag, std::true_type{}, 0);
+      int kt = 1;
       if (!RAGGED) {
         for (; kt + 1 < KT; kt += 2) {
-          one_stage(ragged_tag, kt);
-          one_stage(ragged_tag, kt + 1);
+          one_stage(ragged_tag, std::false_type{}, kt);
+          one_stage(ragged_tag, std::false_type{}, kt + 1);
         }
       }
-      for (; kt < KT; ++kt) one_stage(ragged_tag, kt);
+      for (; kt < KT; ++kt) one_stage(ragged_tag, std::false_type{}, kt);
     };
     if (ragged) k_loop(std::true_type{});
     else k_loop(std::false_type{});
