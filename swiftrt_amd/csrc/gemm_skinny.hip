@@ -16,6 +16,10 @@
 //           vector-memory instructions are global->LDS loads and its only register-producing
 //           loads are LDS reads.
 //   grid    ceil(N / 32) x batch workgroups of 60-72 KiB LDS: two per CU, all resident at once.
+//   M > 16  x is as large per k block as the 32 rows of W it meets, and every workgroup re-reads it
+//           from L2: when N is large enough to keep most CUs busy that way, a workgroup takes 64
+//           rows of W (two output tiles per wave sharing the x fragments): 12 loads per k block and
+//           64 columns instead of 16, x traffic halved.
 #include "gemm_common.h"
 
 namespace srt {
@@ -43,16 +47,18 @@ __device__ __forceinline__ f32x16_t mfma32s<F16>(u32x4_t a, u32x4_t b, f32x16_t 
 
 constexpr int SK_WAVES = 4;
 constexpr int SK_KB = 64;          // k per block step (128 bytes per row)
-constexpr int SK_WBYTES = 32 * 128;   // W part of a ring slot: 32 rows x 128 B
+constexpr int SK_WTILE = 32 * 128;    // one 32-row W tile of a ring slot: 32 rows x 128 B
 constexpr uint32_t SK_OOB = 0x80000000u;
 
-// ring depth per x-row capacity: two workgroups per CU must fit in 160 KiB of LDS
-template <int XR>
+// XR: x rows staged per k block; NW: 32-row W tiles per workgroup.  Ring depth: what fits in
+// 160 KiB of LDS with two workgroups per CU (NW = 1) or one (NW = 2).
+template <int XR, int NW>
 struct SkinnyShape {
-  static constexpr int DEPTH = XR == 32 ? 2 : 3;           // k blocks in flight per wave
-  static constexpr int SLOT = SK_WBYTES + XR * 128;         // W rows + x rows of one k block
-  static constexpr int LOADS = 4 + XR / 8;                  // load instructions per k block
-  static constexpr int LDS = SK_WAVES * DEPTH * SLOT;       // 60 / 72 / 64 KiB
+  static constexpr int DEPTH = NW == 2 ? 3 : (XR == 32 ? 2 : 3);   // k blocks in flight per wave
+  static constexpr int WBYTES = NW * SK_WTILE;                      // W part of a ring slot
+  static constexpr int SLOT = WBYTES + XR * 128;                    // W rows + x rows of one k block
+  static constexpr int LOADS = 4 * NW + XR / 8;                     // load instructions per k block
+  static constexpr int LDS = SK_WAVES * DEPTH * SLOT;               // 60 / 72 / 64 KiB; 144 KiB for NW = 2
 };
 
 // STREAM: the data is read once by the whole grid (the weight), so the load carries the
@@ -78,9 +84,10 @@ __device__ __forceinline__ void sk_load_to_lds(u32x4_t rsrc, uint32_t lds_addr, 
 // Every vector-memory instruction in the k loop is a global->LDS load issued from inline assembly
 // and awaited with explicit s_waitcnt vmcnt; everything that produces registers is an LDS read,
 // which the compiler tracks on its own counter.
-template <typename T, int XR>
+template <typename T, int XR, int NW>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem p) {
-  using Shape = SkinnyShape<XR>;
+  using Shape = SkinnyShape<XR, NW>;
+  constexpr int SK_WBYTES = Shape::WBYTES;
   constexpr int DEPTH = Shape::DEPTH;
   extern __shared__ __attribute__((aligned(1024))) unsigned char sk_lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)sk_lds_raw;
@@ -89,7 +96,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const int n0 = blockIdx.x * 32;
+  const int n0 = blockIdx.x * (32 * NW);
   const int bz = blockIdx.y;
 
   const uint16_t* X = (const uint16_t*)p.A + (long long)bz * p.sab;
@@ -108,10 +115,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   // c ^ ((r >> 1) & 7)).  (row >> 1) & 7 only depends on the lane, not on which group of 8 rows.
   const int lrow = lane >> 3;
   const int lchunk = (lane & 7) ^ ((lrow >> 1) & 3) ^ 0;   // rows 8 i + lrow: ((8 i + lrow) >> 1) & 7 = 4 (i & 1) + (lrow >> 1)
-  uint32_t wvoff[4], xvoff[XR / 8];
-  int wchunk[4], xchunk[XR / 8];
+  uint32_t wvoff[4 * NW], xvoff[XR / 8];
+  int wchunk[4 * NW], xchunk[XR / 8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 4 * NW; ++i) {
     const int row = 8 * i + lrow;
     wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
     const int n = n0 + row;
@@ -140,7 +147,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     const uint32_t base = my_ring + (uint32_t)slot * Shape::SLOT;
     const uint32_t soff = (uint32_t)kb * (SK_KB * 2);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 4 * NW; ++i) {
       const bool in_k = live && (kb * 8 + wchunk[i]) < k_chunks;
       sk_load_to_lds<true>(rw, base + (uint32_t)i * 1024u, in_k ? wvoff[i] : SK_OOB, soff);
     }
@@ -151,9 +158,11 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     }
   };
 
-  f32x16_t acc;
+  f32x16_t acc[NW];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+  for (int t = 0; t < NW; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
 
   // This wave's k blocks are wave, wave + 4, ... (count of them); it walks them in rotated
   // order, starting at a block that depends on the workgroup, so that the workgroups resident at
@@ -180,10 +189,11 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
       const int j = j0 + d;
       asm volatile("s_waitcnt vmcnt(%0)" : : "i"(Shape::LOADS * (DEPTH - 1)) : "memory");
       const uint32_t base = my_ring + (uint32_t)d * Shape::SLOT;
-      u32x4_t wf[4], xf[4];
+      u32x4_t wf[NW][4], xf[4];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        wf[s] = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + rd[s]);
+#pragma unroll
+        for (int t = 0; t < NW; ++t) wf[t][s] = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + t * SK_WTILE + rd[s]);
         u32x4_t x = {0u, 0u, 0u, 0u};
         if (x_lane) x = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + SK_WBYTES + rd[s]);
         xf[s] = x;
@@ -192,52 +202,62 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
       issue(block_at(j + DEPTH), d);
       if (j < count) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) acc = mfma32s<T>(xf[s], wf[s], acc);
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+          for (int t = 0; t < NW; ++t) acc[t] = mfma32s<T>(xf[s], wf[t][s], acc[t]);
       }
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();   // every wave's loads have landed and its ring is idle: reuse LDS for the reduction
 
-  float* red = reinterpret_cast<float*>(sk_lds_raw);   // [4 waves][16][64] = 16 KiB
+  float* red = reinterpret_cast<float*>(sk_lds_raw);   // [NW tiles][4 waves][16][64] = NW x 16 KiB
 #pragma unroll
-  for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[v];
+  for (int t = 0; t < NW; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[((t * SK_WAVES + wave) * 16 + v) * 64 + lane] = acc[t][v];
   __syncthreads();
 
   // wave w finishes accumulator registers 4w .. 4w+3: rows m = 8 w + 4 h + i, column n
-  const int n = n0 + r;
-  if (n >= p.N) return;
   Epilogue<T> ep(p);
   uint16_t* C = (uint16_t*)p.C + (long long)bz * p.scb;
-  const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int v = 4 * wave + i;
-    const int m = 8 * wave + 4 * h + i;
-    if (m >= p.M) continue;
-    float s = 0.0f;
+  for (int t = 0; t < NW; ++t) {
+    const int n = n0 + 32 * t + r;
+    if (n >= p.N) continue;
+    const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
 #pragma unroll
-    for (int w = 0; w < SK_WAVES; ++w) s += red[(w * 16 + v) * 64 + lane];
-    const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
-    C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, bv);
+    for (int i = 0; i < 4; ++i) {
+      const int v = 4 * wave + i;
+      const int m = 8 * wave + 4 * h + i;
+      if (m >= p.M) continue;
+      float s = 0.0f;
+#pragma unroll
+      for (int w = 0; w < SK_WAVES; ++w) s += red[((t * SK_WAVES + w) * 16 + v) * 64 + lane];
+      const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
+      C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, bv);
+    }
   }
 }
 
-template <typename T, int XR>
+template <typename T, int XR, int NW>
 hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
-  auto kernel = gemm_skinny_kernel<T, XR>;
-  constexpr int lds_bytes = SkinnyShape<XR>::LDS;
+  auto kernel = gemm_skinny_kernel<T, XR, NW>;
+  constexpr int lds_bytes = SkinnyShape<XR, NW>::LDS;
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, dim3((p.N + 31) / 32, p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((p.N + 32 * NW - 1) / (32 * NW), p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
   return hipGetLastError();
 }
 
 template <typename T>
 hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
-  if (p.M <= 8) return launch_skinny_shape<T, 8>(p, stream);
-  if (p.M <= 16) return launch_skinny_shape<T, 16>(p, stream);
-  return launch_skinny_shape<T, 32>(p, stream);
+  if (p.M <= 8) return launch_skinny_shape<T, 8, 1>(p, stream);
+  if (p.M <= 16) return launch_skinny_shape<T, 16, 1>(p, stream);
+  // two W tiles per workgroup once that still gives most CUs a workgroup (192 of them)
+  const long long wide_groups = (long long)((p.N + 63) / 64) * p.batch;
+  if (wide_groups >= 192) return launch_skinny_shape<T, 32, 2>(p, stream);
+  return launch_skinny_shape<T, 32, 1>(p, stream);
 }
 
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }

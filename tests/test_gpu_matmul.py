@@ -355,6 +355,31 @@ def test_skinny_ragged_and_integer_exact(dt):
         assert np.array_equal(got.view(np.uint16), H.encode(exact, dt).view(np.uint16)), (M, N, K)
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_skinny_wide_groups_integer_exact_bias_and_batch(dt):
+    """17 <= M <= 32 against a large weight: workgroups take 64 rows of W.  N not a multiple of 64 (nor of
+    32), K ending inside a k block, bias + ReLU, and a strided batch that reaches the threshold together."""
+    r = H.rng(41)
+    for (M, N, K) in [(32, 12328, 200), (17, 12344, 72), (25, 16384, 64)]:
+        x = r.integers(-2, 3, (M, K)).astype(np.float32)
+        w = r.integers(-2, 3, (N, K)).astype(np.float32)
+        b = r.integers(-3, 4, N).astype(np.float32)
+        xt, wt, bt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt)), srt.Tensor(H.encode(b, dt))
+        out = srt.Tensor(shape=[M, N], dtype=xt.dtype)
+        assert query_kernel(xt, False, wt, True, out) == "skinny"
+        srt.current_queue().matmul(xt, False, wt, True, out, bias=bt, activation=srt.ActivationType.relu)
+        exact = np.maximum(x.astype(np.int64) @ w.astype(np.int64).T + b.astype(np.int64)[None, :], 0)
+        assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    B_, M, N, K = 4, 32, 3100, 136        # 4 x 49 workgroups of 64 columns
+    x = r.integers(-2, 3, (B_, M, K)).astype(np.float32)
+    w = r.integers(-2, 3, (B_, N, K)).astype(np.float32)
+    xt, wt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt))
+    out = srt.matmul(xt, wt, transposed_rhs=True)
+    assert query_kernel(xt, False, wt, True, out) == "skinny"
+    exact = x.astype(np.int64) @ np.swapaxes(w, 1, 2).astype(np.int64)
+    assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
+
+
 # ---- layouts: views, column-major, strided output ------------------------------------------------------
 @pytest.mark.parametrize("dt", DTS)
 def test_strided_views_and_column_major(dt):
