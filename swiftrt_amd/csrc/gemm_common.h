@@ -162,6 +162,9 @@ int mfma_select(const GemmProblem& p);
 int mfma_config(const GemmProblem& p, int tile);
 const char* mfma_name(int config);
 hipError_t launch_mfma(const GemmProblem& p, int config, hipStream_t stream);
+// Split-K over the 256 x 256 kernel: number of k parts (0: the problem does not qualify) and launch.
+int mfma_splitk_parts(const GemmProblem& p);
+hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream);
 
 bool skinny_supported(const GemmProblem& p);
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t stream);

@@ -13,4 +13,9 @@ hipError_t SRT_CAT(launch_m16, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const Gem
   return m16::launch<SRT_M16_TYPE, SRT_M16_AKC != 0, SRT_M16_BKC != 0>(p, stream);
 }
 
+// launch_m16_partial_<type>_<akc><bkc>: the split-K pass (fp32 accumulators to a workspace)
+hipError_t SRT_CAT(launch_m16_partial, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const GemmProblem& p, hipStream_t stream) {
+  return m16::launch_partial<SRT_M16_TYPE, SRT_M16_AKC != 0, SRT_M16_BKC != 0>(p, stream);
+}
+
 }  // namespace srt

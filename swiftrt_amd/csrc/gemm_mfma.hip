@@ -45,6 +45,14 @@ SRT_RING_DECL(F16)
 SRT_M16_DECL(BF16)
 SRT_M16_DECL(F16)
 #undef SRT_M16_DECL
+#define SRT_M16P_DECL(T)                                                         \
+  hipError_t launch_m16_partial_##T##_00(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16_partial_##T##_01(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16_partial_##T##_10(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16_partial_##T##_11(const GemmProblem&, hipStream_t);
+SRT_M16P_DECL(BF16)
+SRT_M16P_DECL(F16)
+#undef SRT_M16P_DECL
 
 namespace {
 
@@ -421,6 +429,107 @@ int mfma_select(const GemmProblem& p) {
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
+}
+
+// ---- split-K over the 256 x 256 kernel ----------------------------------------------------------
+// A problem with few 256 x 256 tiles and a long k loop leaves most compute units idle.  Its k range
+// is cut into S equal parts that run as S "batches" of the 16x16x32 ring kernel (operand batch
+// stride = one part's k extent), each writing its fp32 accumulators to a workspace [S][M][N]; a
+// second kernel adds the parts in a fixed order and applies bias, activation and the one rounding.
+// The sums are fp32 throughout, and the result does not depend on timing.
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* part, int parts, GemmProblem p) {
+  using S = typename T::storage;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const int n8 = p.N / 8;   // 8 columns per lane
+  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long long)p.M * n8) return;
+  const int m = (int)(id / n8), n = (int)(id - (long long)m * n8) * 8;
+  const long long mn = (long long)p.M * p.N;
+  const float* src = part + (long long)m * p.N + n;
+  f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = lo;
+  for (int s = 0; s < parts; ++s) {
+    lo += *reinterpret_cast<const f32x4*>(src + s * mn);
+    hi += *reinterpret_cast<const f32x4*>(src + s * mn + 4);
+  }
+  Epilogue<T> ep(p);
+  union { S h[8]; uint4 v; } out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out.h[e] = ep.finish(e < 4 ? lo[e] : hi[e - 4], ep.bias_at(m, n + e));
+  *reinterpret_cast<uint4*>((S*)p.C + (long long)m * p.scm + n) = out.v;
+}
+
+template <typename T>
+hipError_t launch_m16_partial(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream);
+template <>
+hipError_t launch_m16_partial<BF16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_m16_partial_BF16_11(p, stream);
+  if (a_kc) return launch_m16_partial_BF16_10(p, stream);
+  if (b_kc) return launch_m16_partial_BF16_01(p, stream);
+  return launch_m16_partial_BF16_00(p, stream);
+}
+template <>
+hipError_t launch_m16_partial<F16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (a_kc && b_kc) return launch_m16_partial_F16_11(p, stream);
+  if (a_kc) return launch_m16_partial_F16_10(p, stream);
+  if (b_kc) return launch_m16_partial_F16_01(p, stream);
+  return launch_m16_partial_F16_00(p, stream);
+}
+
+}  // namespace
+
+// Number of k parts for the split-K plan, or 0 when the problem does not qualify: one batch,
+// the 256 x 256 kernel's preconditions, parts of equal length that are whole k stages and at least
+// 16 of them (512 k), and no more parts than it takes to give every compute unit a tile.
+int mfma_splitk_parts(const GemmProblem& p) {
+  const int layout = mfma_layout(p);
+  if (layout < 0 || p.batch != 1) return 0;
+  if (!ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
+  if ((reinterpret_cast<uintptr_t>(p.C) & 15u) != 0 || (p.scm % 8) != 0) return 0;
+  const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256);
+  int parts = 0;
+  for (int s = 2; s <= 16; s *= 2) {
+    if (t256 * s > 256) break;
+    if (p.K % (s * 32) != 0 || p.K / s < 512) break;
+    parts = s;
+  }
+  return parts;
+}
+
+hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {
+  const int parts = mfma_splitk_parts(p);
+  if (parts < 2) return hipErrorInvalidValue;
+  const int layout = mfma_layout(p);
+  const bool a_kc = (layout & 2) != 0, b_kc = (layout & 1) != 0;
+  void* workspace = nullptr;
+  const size_t bytes = (size_t)parts * p.M * p.N * sizeof(float);
+  if (srtDeviceAllocate(&workspace, bytes, reinterpret_cast<srtStream>(stream)) != srtSuccess) return hipErrorOutOfMemory;
+  GemmProblem q = p;
+  q.K = p.K / parts;
+  q.batch = parts;
+  q.sab = (long long)q.K * p.sak;   // part s starts q.K further along k
+  q.sbb = (long long)q.K * p.sbk;
+  q.C = workspace;
+  q.scm = p.N;
+  q.scn = 1;
+  q.scb = (long long)p.M * p.N;
+  q.bias = nullptr;
+  q.activation = srtActivationIdentity;
+  hipError_t e = p.dtype == srtReal16BF ? launch_m16_partial<BF16>(q, a_kc, b_kc, stream)
+                                        : launch_m16_partial<F16>(q, a_kc, b_kc, stream);
+  if (e == hipSuccess) {
+    const long long lanes = (long long)p.M * (p.N / 8);
+    const unsigned blocks = (unsigned)((lanes + 255) / 256);
+    if (p.dtype == srtReal16BF)
+      hipLaunchKernelGGL(splitk_reduce_kernel<BF16>, dim3(blocks), dim3(256), 0, stream, (const float*)workspace, parts, p);
+    else
+      hipLaunchKernelGGL(splitk_reduce_kernel<F16>, dim3(blocks), dim3(256), 0, stream, (const float*)workspace, parts, p);
+    e = hipGetLastError();
+  }
+  (void)srtDeviceFree(workspace);   // stream-ordered: reused only by work queued after the kernels above
+  return e;
 }
 
 const char* mfma_name(int config) {

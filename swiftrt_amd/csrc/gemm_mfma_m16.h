@@ -60,6 +60,7 @@ using ring::EPI_RELU;
 using ring::EPI_BIAS_RELU;
 using ring::EPI_CLIPPED;
 using ring::EPI_TRANS;
+constexpr int EPI_PARTIAL = 6;   // fp32 accumulators as they are, for a split-K pass (C is a float workspace)
 
 #define SRT_FENCE() __builtin_amdgcn_sched_barrier(0)
 
@@ -361,6 +362,28 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
   }
 }
 
+// Split-K pass: the fp32 accumulators go to a float workspace as they are ([batch][M][N], row
+// stride scm floats): a lane's four consecutive columns are one 16-byte store, a store instruction
+// writes 16 rows x 64 bytes.  A second kernel adds the passes and applies the epilogue.
+__device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0,
+                                                   int wave_n0, int bz, int lane) {
+  float* C = (float*)p.C + (long long)bz * p.scb;
+  const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
+  const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 4), 0x00020000);
+  const int ldc4 = (int)(p.scm * 4);
+  const int jn = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = wave_m0 + 16 * i + jn;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = wave_n0 + 16 * j + 4 * g;   // N is a multiple of 8: the four columns are in range together
+      const uint32_t off = (m < p.M && n < p.N) ? (uint32_t)(m * ldc4 + n * 4) : OOB;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, acc[i][j]), rc, (int)off, 0, 0);
+    }
+  }
+}
+
 template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
   static_assert(NS == 5, "ring depth");   // slot arithmetic below assumes the staging slots are NS-2, NS-1 ahead
@@ -593,7 +616,9 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
     const int le = lane_id();
 
-    if (EPI == EPI_TRANS) {
+    if (EPI == EPI_PARTIAL) {
+      store_tile_partial(p, acc, em0, en0, bz, le);
+    } else if (EPI == EPI_TRANS) {
       store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
     } else {
       if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
@@ -640,6 +665,12 @@ hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   }
   if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS, NS>(p, stream);
   return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS>(p, stream);
+}
+
+// The split-K pass of `p` (whose C is the float workspace and whose batch counts the k ranges).
+template <typename T, bool A_KC, bool B_KC, int NS = 5>
+hipError_t launch_partial(const GemmProblem& p, hipStream_t stream) {
+  return launch_kernel<T, A_KC, B_KC, EPI_PARTIAL, NS>(p, stream);
 }
 
 }  // namespace m16

@@ -88,11 +88,11 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
 // (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
 // and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
 enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK,
-            kPlanKc64, kPlanM16, kPlanCount };
+            kPlanKc64, kPlanM16, kPlanSplitK, kPlanCount };
 
 const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
                                             "f32_mfma_64x64", "f32_mfma_splitk", "mfma_256x256_k64",
-                                            "mfma_256x256_m16"};
+                                            "mfma_256x256_m16", "mfma_256x256_splitk"};
 
 bool plan_supported(const GemmProblem& p, Plan plan) {
   switch (plan) {
@@ -102,6 +102,7 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
     case kPlanMfma64: return srt::mfma_config(p, 3) != 0;
     case kPlanKc64: return srt::mfma_config(p, 4) != 0;
     case kPlanM16: return srt::mfma_config(p, 5) != 0;
+    case kPlanSplitK: return srt::mfma_splitk_parts(p) >= 2;
     case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
     case kPlanF32SplitK: return srt::f32_mfma_supported(p);
     default: return srt::generic_supported(p);
@@ -110,6 +111,12 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 
 Plan heuristic_plan(const GemmProblem& p) {
   if (srt::skinny_supported(p)) return kPlanSkinny;
+  // Few 256 x 256 tiles and a long k loop: split K over the idle compute units.  The fp32 parts cost
+  // a fixed 25-30 us to write and add up (about 67 MB each way whatever the shape), so this pays
+  // from K = 4096 up (1024 x 4096 x 4096: 55 us against 75 us; 256 x 8192 x 8192: 62 against 129;
+  // 1024 x 1024 x 4096: 34 against 64) and not below (2048^3: 44 us against 41 us).
+  if (p.K >= 4096 && (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) <= 96 && srt::mfma_splitk_parts(p) >= 2)
+    return kPlanSplitK;
   const int c = srt::mfma_select(p);
   if (c) {
     switch (c >> 2) {
@@ -132,6 +139,7 @@ hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
     case kPlanMfma64: return srt::launch_mfma(p, srt::mfma_config(p, 3), stream);
     case kPlanKc64: return srt::launch_mfma(p, srt::mfma_config(p, 4), stream);
     case kPlanM16: return srt::launch_mfma(p, srt::mfma_config(p, 5), stream);
+    case kPlanSplitK: return srt::launch_mfma_splitk(p, stream);
     case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
     case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
     default: return srt::launch_generic(p, stream);

@@ -200,13 +200,17 @@ def test_kernel_selection_is_queryable_without_gpu():
     # short k loops: the 32x32x16 kernels (64-deep stages when both operands are k-contiguous)
     assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256"
     assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_k64"
+    # few tiles and a long k loop: K split over the idle compute units
+    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_256x256_splitk"
     # mid-size problems: the 256 x 256 kernels from 48 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16"             # 144 tiles, long k loop
     assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256"
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_256x256"                 # 64 tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_64x64"
-    assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_64x64"                    # 32 tiles
+    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_64x64"                    # 32 tiles, K too short to split
     assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"

@@ -531,6 +531,75 @@ def test_m16_kernel_batched_short_k_and_nan(tmp_path):
     srt.PlanCache.clear()
 
 
+# ---- split-K over the 256 x 256 kernel --------------------------------------------------------------
+def pin_plan(tmp_path, plan, dt, M, N, K, ta, tb, bias=False, act=srt.ActivationType.identity):
+    layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
+    f = tmp_path / "plan.txt"
+    f.write_text(f"{dt} {M} {N} {K} 1 {layout} {(1 if bias else 0) | (int(act) << 1)} {plan}\n")
+    srt.PlanCache.clear()
+    srt.PlanCache.load(f)
+
+
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_splitk_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
+    """K cut into 2, 4 and 8 parts; ragged M and N edges; every staging layout."""
+    r = H.rng(310)
+    for (M, N, K) in [(512, 520, 1024), (304, 264, 2048), (200, 1032, 4096)]:
+        pin_plan(tmp_path, "mfma_256x256_splitk", dt, M, N, K, ta, tb)
+        a = r.integers(-2, 3, (K, M) if ta else (M, K)).astype(np.float32)
+        b = r.integers(-2, 3, (N, K) if tb else (K, N)).astype(np.float32)
+        got = gpu_matmul(H.encode(a, dt), H.encode(b, dt), ta, tb, want_kernel="mfma_256x256_splitk")
+        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    M, N, K = 520, 776, 2048
+    pin_plan(tmp_path, "mfma_256x256_splitk", dt, M, N, K, ta, tb)
+    a = (r.standard_normal((K, M) if ta else (M, K)) / np.sqrt(K)).astype(np.float32)
+    b = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    a_st, b_st = H.encode(a, dt), H.encode(b, dt)
+    check_against_fp64(gpu_matmul(a_st, b_st, ta, tb, want_kernel="mfma_256x256_splitk"), a_st, b_st, ta, tb, dt)
+    srt.PlanCache.clear()
+
+
+@pytest.mark.parametrize("act", list(srt.ActivationType))
+def test_splitk_epilogues_vs_oracle_and_nan(act, tmp_path):
+    """Bias and every activation are applied once, after the parts are added; a NaN survives."""
+    r = H.rng(311)
+    dt = H.BF16
+    M, N, K = 520, 264, 2048
+    x = H.encode(r.standard_normal((M, K)).astype(np.float32) / 8, dt)
+    w = H.encode((r.standard_normal((K, N)) / 8).astype(np.float32), dt)
+    b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
+    coef = 0.75
+    pin_plan(tmp_path, "mfma_256x256_splitk", dt, M, N, K, False, False, bias=True, act=act)
+    xt, wt, bt = srt.Tensor(x), srt.Tensor(w), srt.Tensor(b)
+    out = srt.Tensor(shape=[M, N], dtype=x.dtype)
+    srt.current_queue().matmul(xt, False, wt, False, out, bias=bt, activation=act, coef=coef)
+    got = H.decode(out.array())
+    rows = np.concatenate([np.arange(0, M, 37), [M - 1]])
+    want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, transpose_w=False,
+                                      acc=ora.ACC_F32, fused=True))
+    assert np.all(np.abs(got[rows] - want) <= 2.0 ** -7 * np.maximum(np.abs(want), 1.0))
+    if act == srt.ActivationType.identity:
+        a = np.zeros((M, K), np.float32)
+        a[:, 0] = 1.0
+        a[5, K - 1] = np.nan                      # lands in the last part only
+        pin_plan(tmp_path, "mfma_256x256_splitk", dt, M, N, K, False, False)
+        got = gpu_matmul(H.encode(a, dt), w, want_kernel="mfma_256x256_splitk")
+        assert np.all(got[5] == 0x7FFF) and not np.any(got[6] == 0x7FFF)
+    srt.PlanCache.clear()
+
+
+def test_splitk_is_the_choice_for_few_tiles_and_long_k():
+    a = srt.Tensor(H.encode(np.zeros((1024, 4096), np.float32), H.BF16))
+    b = srt.Tensor(H.encode(np.zeros((4096, 4096), np.float32), H.BF16))
+    out = srt.Tensor(shape=[1024, 4096], dtype=a.dtype)
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_splitk"
+    a2 = srt.Tensor(H.encode(np.zeros((1024, 2048), np.float32), H.BF16))      # K = 2048: not worth the extra pass
+    b2 = srt.Tensor(H.encode(np.zeros((2048, 4096), np.float32), H.BF16))
+    assert query_kernel(a2, False, b2, False, out) != "mfma_256x256_splitk"
+
+
 def test_m16_kernel_is_the_choice_for_a_full_device_and_long_k():
     a = srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16))
     b = srt.Tensor(H.encode(np.zeros((2048, 4096), np.float32), H.BF16))
