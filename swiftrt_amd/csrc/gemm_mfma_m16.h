@@ -363,24 +363,55 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
 }
 
 // Split-K pass: the fp32 accumulators go to a float workspace as they are ([batch][M][N], row
-// stride scm floats): a lane's four consecutive columns are one 16-byte store, a store instruction
-// writes 16 rows x 64 bytes.  A second kernel adds the passes and applies the epilogue.
+// stride scm floats); a second kernel adds the passes and applies the epilogue.  Staged through
+// the wave's 16 KiB of LDS in four passes of 32 rows ([32 rows][32 chunks of 16 B], chunk c of row
+// r at c ^ (r & 31)) so that a store instruction writes two rows of 512 contiguous bytes: whole
+// cache lines (straight from the accumulator layout an instruction would write 16 rows x 64 bytes,
+// every line in two halves by different instructions; measured, the two take the same time).
 __device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0,
-                                                   int wave_n0, int bz, int lane) {
+                                                   int wave_n0, int bz, int lane, uint32_t stage) {
   float* C = (float*)p.C + (long long)bz * p.scb;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
   const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 4), 0x00020000);
   const int ldc4 = (int)(p.scm * 4);
   const int jn = lane & 15, g = lane >> 4;
+  const int rd_chunk = lane & 31, rd_row = lane >> 5;   // read side: 4 columns of rows rd_row + 2 it
+  const int n_rd = wave_n0 + 4 * rd_chunk;
+  const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8: the four columns are in range together
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int m = wave_m0 + 16 * i + jn;
+  for (int pass = 0; pass < 4; ++pass) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int n = wave_n0 + 16 * j + 4 * g;   // N is a multiple of 8: the four columns are in range together
-      const uint32_t off = (m < p.M && n < p.N) ? (uint32_t)(m * ldc4 + n * 4) : OOB;
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, acc[i][j]), rc, (int)off, 0, 0);
+    for (int ii = 0; ii < 2; ++ii) {
+      const int i = 2 * pass + ii;
+      const int row = 16 * ii + jn;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int c = 4 * j + g;
+        *reinterpret_cast<SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u + (uint32_t)((c ^ (row & 31)) << 4)) = acc[i][j];
+      }
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int it4 = 0; it4 < 4; ++it4) {
+      f32x4_t v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 2 * (4 * it4 + q);
+        v[q] = *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u +
+                                                         (uint32_t)((rd_chunk ^ (row & 31)) << 4));
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 2 * (4 * it4 + q);
+        const int m = wave_m0 + 32 * pass + row;
+        const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc4 + n_rd * 4) : OOB;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v[q]), rc, (int)off, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // the reads of this pass have returned (their data is in the stores above) before the next
+    // pass overwrites the area: LDS operations of a wave execute in order
   }
 }
 
@@ -617,7 +648,7 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     const int le = lane_id();
 
     if (EPI == EPI_PARTIAL) {
-      store_tile_partial(p, acc, em0, en0, bz, le);
+      store_tile_partial(p, acc, em0, en0, bz, le, stage);
     } else if (EPI == EPI_TRANS) {
       store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
     } else {
