@@ -83,6 +83,55 @@ def test_every_plan_is_the_same_function(tmp_path):
         assert np.max(np.abs(r - results["generic"]) / (np.abs(c64) + 1e-3)) <= 2 ** -6, plan
 
 
+ALL_PLANS_16 = ("mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64", "mfma_256x256_splitk", "mfma_128x128",
+                "mfma_64x64", "skinny", "generic")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_shapes_every_qualifying_plan_bit_exact(seed, tmp_path):
+    """Random shapes, layouts, element types, bias and activation: every plan that accepts the problem
+    (asked through the cache, answered by the kernel query) must give the exact integer result.  A
+    plan that claims a problem it mishandles -- a ragged edge, a k tail, a split that does not divide
+    -- shows up here whatever the heuristic would have chosen."""
+    g = H.rng(5000 + seed)
+    ran = set()
+    for case in range(7):
+        dt = (H.BF16, H.F16)[int(g.integers(0, 2))]
+        ta, tb = bool(g.integers(0, 2)), bool(g.integers(0, 2))
+        M = int(g.choice([8, 24, 32, 200, 264, 520, 1032]))
+        N = int(g.choice([8, 40, 256, 264, 776, 1288]))
+        K = int(g.choice([8, 64, 72, 200, 1024, 2048, 4096]))
+        with_bias = bool(g.integers(0, 2))
+        act = (srt.ActivationType.identity, srt.ActivationType.relu)[int(g.integers(0, 2))]
+        a = g.integers(-2, 3, (K, M) if ta else (M, K)).astype(np.float32)
+        b = g.integers(-2, 3, (N, K) if tb else (K, N)).astype(np.float32)
+        bias = g.integers(-3, 4, N).astype(np.float32)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+        if with_bias:
+            exact = exact + bias[None, :]
+        if act == srt.ActivationType.relu:
+            exact = np.maximum(exact, 0.0)
+        want = H.encode(exact.astype(np.float32), dt).view(np.uint16)
+        at, bt, biast = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(b, dt)), srt.Tensor(H.encode(bias, dt))
+        layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
+        for plan in ALL_PLANS_16:
+            # the query has no epilogue argument: ask with the plain key, run with the real one
+            for epilogue in {10, (1 if with_bias else 0) | (int(act) << 1)}:
+                f = tmp_path / "p.txt"
+                f.write_text(f"{dt} {M} {N} {K} 1 {layout} {epilogue} {plan}\n")
+                srt.PlanCache.load(f)
+            out = srt.Tensor(shape=[M, N], dtype=at.dtype)
+            if query_kernel(at, ta, bt, tb, out) != plan:
+                srt.PlanCache.clear()
+                continue
+            srt.current_queue().matmul(at, ta, bt, tb, out, bias=biast if with_bias else None, activation=act)
+            assert np.array_equal(out.array().view(np.uint16), want), (plan, dt, ta, tb, M, N, K, with_bias, act)
+            ran.add(plan)
+            srt.PlanCache.clear()
+    print("plans exercised:", sorted(ran))
+    assert "generic" in ran and len(ran) >= 3
+
+
 def test_cached_plan_is_skipped_when_this_call_does_not_qualify(tmp_path):
     """Alignment is not part of the key: a view that starts off a 16-byte boundary with the same
     shape and layout class falls back to the heuristic (the generic kernel) instead of the cached
