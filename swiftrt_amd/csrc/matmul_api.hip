@@ -251,7 +251,14 @@ Plan select(const GemmProblem& p) {
 srtStatus run(const GemmProblem& p, hipStream_t stream) {
   const Plan plan = select(p);
   if (plan == kPlanGeneric && !srt::generic_supported(p)) return srtErrorNotSupported;
-  return srt::from_hip(launch_plan(p, plan, stream));
+  hipError_t e = launch_plan(p, plan, stream);
+  if (plan == kPlanSplitK && e == hipErrorOutOfMemory) {
+    // no room for the workspace (nothing was launched): the plan that needs none
+    (void)hipGetLastError();
+    const int c = srt::mfma_select(p);
+    e = c ? srt::launch_mfma(p, c, stream) : srt::launch_generic(p, stream);
+  }
+  return srt::from_hip(e);
 }
 
 }  // namespace
