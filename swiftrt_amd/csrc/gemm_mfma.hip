@@ -256,7 +256,7 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<T>(af[i], bf[j], acc[i][j]);
+        for (int j = 0; j < TN; ++j) acc[i][j] = mfma32<T>(bf[j], af[i], acc[i][j]);   // B first: C^T tiles
     }
     if (more) {
       sa.store(nxt, tid);
@@ -265,22 +265,41 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
     __syncthreads();
   }
 
-  // epilogue: lane holds column l % 32 and rows 8*(v/4) + 4*(l/32) + v%4 of each 32 x 32 tile
+  // epilogue: the MFMA took the B fragment first, so each 32 x 32 accumulator tile is C^T: a lane
+  // holds row l % 32 and, per group of four registers, the four consecutive columns
+  // 8 (v / 4) + 4 (l / 32) + 0..3 -- one 8-byte store per group where the row pitch and base of C
+  // keep it aligned and the group lies inside N, element stores otherwise.
   Epilogue<T> ep(p);
   uint16_t* C = (uint16_t*)p.C + (long long)bz * p.scb;
+  const bool wide = (p.scm % 4) == 0 && (reinterpret_cast<uintptr_t>(C) & 7u) == 0;
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn0 + 32 * j + (lane & 31);
-    if (n >= p.N) continue;
-    const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm0 + 32 * i + (lane & 31);
+    if (m >= p.M) continue;
+    const float brow = ep.per_row ? ep.bias_at(m, 0) : 0.0f;
+    uint16_t* crow = C + (long long)m * p.scm;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int j = 0; j < TN; ++j) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm0 + 32 * i + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (m >= p.M) continue;
-        const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
-        C[(long long)m * p.scm + n] = ep.finish(acc[i][j][v], bv);
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn0 + 32 * j + 8 * q + 4 * (lane >> 5);
+        if (n >= p.N) continue;
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float bv = ep.per_row ? brow : (n + e < p.N ? ep.bias_at(0, n + e) : 0.0f);
+          h[e] = ep.finish(acc[i][j][4 * q + e], bv);
+        }
+        if (wide && n + 3 < p.N) {
+          uint2 w;
+          w.x = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+          w.y = (uint32_t)h[2] | ((uint32_t)h[3] << 16);
+          *reinterpret_cast<uint2*>(crow + n) = w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < p.N) crow[n + e] = h[e];
+        }
       }
     }
   }
