@@ -235,7 +235,7 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
  * built-in heuristic decides.  All plans compute the same function to the documented tolerance
  * (sums are fp32; their order differs between plans).
  * chosen (optional): receives the plan's name ("mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
- * "mfma_256x256_splitk", "mfma_128x128", "mfma_64x64", "skinny", "f32_mfma_64x64", "f32_mfma_splitk",
+ * "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "skinny", "f32_mfma_64x64", "f32_mfma_splitk",
  * "generic").
  * The cache is thread-safe.  Save / Load use a small text file, one plan per line:
  *   dtype M N K batch layout epilogue plan-name

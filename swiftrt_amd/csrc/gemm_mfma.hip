@@ -53,6 +53,10 @@ SRT_M16_DECL(F16)
 SRT_M16P_DECL(BF16)
 SRT_M16P_DECL(F16)
 #undef SRT_M16P_DECL
+hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_BF16_11(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_F16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_F16_11(const GemmProblem&, hipStream_t);
 
 namespace {
 
@@ -362,14 +366,22 @@ hipError_t launch_m16<F16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream
   return launch_m16_F16_00(p, stream);
 }
 
-// tile 1 (256 x 256) is the ring kernel, tile 5 the same ring on 16x16x32 MFMAs; tiles 2 and 3 are the
-// register-staged kernels above
+// the 128 x 256 form of the 16x16x32 ring kernel (k-contiguous A)
+template <typename T>
+hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) return b_kc ? launch_m16h_BF16_11(p, stream) : launch_m16h_BF16_10(p, stream);
+  return b_kc ? launch_m16h_F16_11(p, stream) : launch_m16h_F16_10(p, stream);
+}
+
+// tile 1 (256 x 256) is the ring kernel, tile 5 the same ring on 16x16x32 MFMAs, tile 6 its 128 x 256
+// form; tiles 2 and 3 are the register-staged kernels above
 template <typename T>
 hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hipStream_t stream) {
   switch (tile) {
     case 1: return launch_ring<T>(p, a_kc, b_kc, stream);
     case 4: return T::dtype == srtReal16BF ? launch_kc64_BF16(p, stream) : launch_kc64_F16(p, stream);
     case 5: return launch_m16<T>(p, a_kc, b_kc, stream);
+    case 6: return launch_m16h<T>(p, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     default: return launch_layout<T, 64, 64>(p, a_kc, b_kc, stream);
   }
@@ -404,12 +416,13 @@ static int mfma_layout(const GemmProblem& p) {
 }
 
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
-// 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs), or 0
-// when the problem does not qualify for it.
+// 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
+// 128 x 256 form for a k-contiguous A), or 0 when the problem does not qualify for it.
 int mfma_config(const GemmProblem& p, int tile) {
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || tile > 5) return 0;
-  if ((tile == 1 || tile == 4 || tile == 5) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
+  if (layout < 0 || tile < 1 || tile > 6) return 0;
+  if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
+  if (tile == 6 && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
 }
@@ -441,8 +454,16 @@ int mfma_select(const GemmProblem& p) {
   //    the 256 x 256 kernels' preconditions but have at least one such tile per CU.
   const bool big_ok = ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0);
   const long long t256 = tiles(256);
+  //  * with a k-contiguous A the 16x16x32 kernel also comes with 128 x 256 tiles: twice the
+  //    workgroups, which is what a problem that leaves compute units idle needs, as long as they
+  //    all run at once (2048^3: 29 us against 42 us; 512 x 14336 x 4096: 59 against 82;
+  //    2048 x 4096 x 2048, 256 half tiles: 35 against 47; 3072 x 3072 x 1024, 288 half tiles: 32.5
+  //    against 28 for whole tiles).  With a k-contiguous B as well the 64 x 64 kernel is as good
+  //    up to about 96 such tiles (1024 x 1024 x 2048: 20 us against 23 us).
+  const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
   int tile;
-  if (big_ok && t256 >= 128 && p.K >= 2048) tile = 5;
+  if (big_ok && (layout & 2) != 0 && th <= 256 && th >= (layout == 3 ? 96 : 24) && p.K >= 512) tile = 6;
+  else if (big_ok && t256 >= 128 && p.K >= 2048) tile = 5;
   else if (big_ok && layout == 3 && t256 >= 192) tile = 4;
   else if (big_ok && t256 >= (layout == 3 ? 96 : 48)) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
@@ -556,6 +577,7 @@ const char* mfma_name(int config) {
     case 1: return "mfma_256x256";
     case 4: return "mfma_256x256_k64";
     case 5: return "mfma_256x256_m16";
+    case 6: return "mfma_128x256_m16";
     case 2: return "mfma_128x128";
     default: return "mfma_64x64";
   }

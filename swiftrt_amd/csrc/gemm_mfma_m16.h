@@ -47,7 +47,6 @@ using ring::u32x2_t;
 using ring::u32x4_t;
 using ring::s16x4_t;
 using ring::BK;
-using ring::BM;
 using ring::BN;
 using ring::NT;
 using ring::OOB;
@@ -90,9 +89,10 @@ __device__ __forceinline__ void mfma16_first<F16>(f32x4_t& acc, const u32x4_t& b
 }
 
 // Ends the life of the register copies the compiler makes of accumulators (see ring::pin).
-__device__ __forceinline__ void pin_all(f32x4_t (&acc)[8][8]) {
+template <int TM>
+__device__ __forceinline__ void pin_all(f32x4_t (&acc)[TM][8]) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
 }
@@ -106,17 +106,19 @@ __device__ __forceinline__ void pin_all(f32x4_t (&acc)[8][8]) {
 // ds_read_b64_tr_b16, which come from k rows 8 g .. 8 g + 3, on the same banks for every g.
 //   k-contiguous:  [256 rows][4 chunks of 16 B], chunk c of row r at position c ^ ((r >> 1) & 3)
 //   mn-contiguous: [32 k][32 chunks of 16 B], chunk c of k row k at c ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1)
-template <bool KC>
+// LPW: loads per wave, operand and stage -- 4 for a 256-wide region, 2 for a 128-row k-contiguous one.
+template <bool KC, int LPW = 4>
 struct Loader {
-  uint32_t voff[4];
+  static_assert(LPW == 4 || (KC && LPW == 2), "an mn-contiguous region is 256 wide");
+  uint32_t voff[LPW];
 
   // ld: elements between rows (KC) or between k (MN)
   __device__ __forceinline__ void init(int wave, int lane, long long ld) {
     if constexpr (KC) {
-      // load i of this wave covers tile rows (wave*4 + i)*16 .. +15, 4 lanes per 64-byte row
+      // load i of this wave covers tile rows (wave*LPW + i)*16 .. +15, 4 lanes per 64-byte row
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = (wave * 4 + i) * 16 + (lane >> 2);
+      for (int i = 0; i < LPW; ++i) {
+        const int row = (wave * LPW + i) * 16 + (lane >> 2);
         const int chunk = (lane & 3) ^ ((row >> 1) & 3);
         voff[i] = (uint32_t)(((long long)row * ld + chunk * 8) * 2);
       }
@@ -148,13 +150,13 @@ struct Loader {
                                             bool tail, int krem) const {
     uint32_t v = voff[i];
     if (tail && beyond_k(wave, lane, i, krem)) v = OOB;
-    ring::load_to_lds(rsrc, region + (uint32_t)(wave * 4 + i) * 1024u, v, soff);
+    ring::load_to_lds(rsrc, region + (uint32_t)(wave * LPW + i) * 1024u, v, soff);
   }
 
   // aims what lies at or beyond K out of range for good (the state is derived afresh per tile)
   __device__ __forceinline__ void mask_tail(int wave, int lane, int krem) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < LPW; ++i)
       if (beyond_k(wave, lane, i, krem)) voff[i] = OOB;
   }
 };
@@ -199,8 +201,8 @@ struct FragReader {
 // ---- epilogue ------------------------------------------------------------------------------------
 // acc[i][j] is a transposed 16 x 16 tile: lane l owns row m = wave_m0 + 16 i + l % 16 and the
 // columns n = wave_n0 + 16 j + 4 (l / 16) + 0..3.
-template <typename T, bool HAS_BIAS, int CLAMP>
-__device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x4_t (&acc)[8][8], int wave_m0,
+template <typename T, bool HAS_BIAS, int CLAMP, int TM>
+__device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x4_t (&acc)[TM][8], int wave_m0,
                                                       int wave_n0, int lane) {
   using S = typename T::storage;
   const S* bias = (const S*)p.bias;
@@ -218,7 +220,7 @@ __device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x
       }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < TM; ++i) {
       float brow = 0.0f;
       if (HAS_BIAS) {
         const int m = wave_m0 + 16 * i + jn;
@@ -236,15 +238,17 @@ __device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x
   }
 }
 
-// One rounding to the element type, then a trip through the wave's 16 KiB staging area at LDS
-// address `stage` so that global stores are whole 16-byte chunks of 256-byte row segments.  Two
-// halves of 64 rows: [64 rows][16 chunks of 16 B], chunk c of row r at position c ^ (r & 15)
-// (conflict-free on both sides: a write instruction covers 16 rows x 32 B, a read 4 whole rows).
+// One rounding to the element type, then a trip through the wave's staging area at LDS address
+// `stage` so that global stores are whole 16-byte chunks of 256-byte row segments.  Passes of ROWS
+// rows (64: 16 KiB of staging, the 128-row wave tile; 32: 8 KiB, the 64-row one):
+// [ROWS rows][16 chunks of 16 B], chunk c of row r at position c ^ (r & 15) (conflict-free on both
+// sides: a write instruction covers 16 rows x 32 B, a read 4 whole rows).
 // NaN handling as in ring::store_tile: the hardware converter rounds everything, and when any
 // lane of the wave saw a NaN the staged patterns are rewritten to 0x7FFF on the way out.
-template <typename T>
-__device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0, int wave_n0,
+template <typename T, int TM>
+__device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[TM][8], int wave_m0, int wave_n0,
                                            int bz, int lane, uint32_t stage) {
+  constexpr int ROWS = TM == 8 ? 64 : 32;
   using S = typename T::storage;
   constexpr bool FIXUP = T::dtype == srtReal16BF;
   S* C = (S*)p.C + (long long)bz * p.scb;
@@ -257,11 +261,11 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
   const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8 (checked on the host): the chunk is whole
 
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
+  for (int half = 0; half < TM * 16 / ROWS; ++half) {
     bool nan = false;
 #pragma unroll
-    for (int ii = 0; ii < 4; ++ii) {
-      const int i = 4 * half + ii;
+    for (int ii = 0; ii < ROWS / 16; ++ii) {
+      const int i = (ROWS / 16) * half + ii;
       const int row = 16 * ii + jn;
       const uint32_t row_addr = stage + (uint32_t)row * 256u + (uint32_t)(g & 1) * 8u;
       SRT_FENCE();
@@ -278,9 +282,9 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
     }
     SRT_FENCE();
     const bool fix = FIXUP && __builtin_amdgcn_ballot_w64(nan) != 0;
-    // ---- staging -> global: 16 instructions of 4 rows x 256 bytes, read four at a time ----
+    // ---- staging -> global: ROWS / 4 instructions of 4 rows x 256 bytes, read four at a time ----
 #pragma unroll
-    for (int it4 = 0; it4 < 4; ++it4) {
+    for (int it4 = 0; it4 < ROWS / 16; ++it4) {
       u32x4_t v[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -297,7 +301,7 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = rd_row + 4 * (4 * it4 + q);
-        const int m = wave_m0 + 64 * half + row;
+        const int m = wave_m0 + ROWS * half + row;
         const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc2 + n_rd * 2) : OOB;
         __builtin_amdgcn_raw_buffer_store_b128(v[q], rc, (int)off, 0, SRT_STORE_AUX);
       }
@@ -306,11 +310,13 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
   }
 }
 
-// sigmoid / tanh / elu: acc + bias goes to the staging area as fp32 ([32 rows][32 chunks of 16 B],
-// chunk c of row r at c ^ (r & 31)); activation, rounding and store run in a rolled loop.
-template <typename T>
-__device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, const f32x4_t (&acc)[8][8],
+// sigmoid / tanh / elu: acc + bias goes to the staging area as fp32 (passes of ROWS = 32 or 16 rows:
+// [ROWS rows][32 chunks of 16 B], chunk c of row r at c ^ (r & 31)); activation, rounding and store
+// run in a rolled loop.
+template <typename T, int TM>
+__device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, const f32x4_t (&acc)[TM][8],
                                                           int wave_m0, int wave_n0, int bz, int lane, uint32_t stage) {
+  constexpr int ROWS = TM == 8 ? 32 : 16;
   using S = typename T::storage;
   S* C = (S*)p.C + (long long)bz * p.scb;
   const S* bias = (const S*)p.bias;
@@ -323,10 +329,10 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
   const int n_rd = wave_n0 + 4 * rd_chunk;
   const bool n_rd_ok = n_rd < p.N;
 #pragma unroll
-  for (int pass = 0; pass < 4; ++pass) {
+  for (int pass = 0; pass < TM * 16 / ROWS; ++pass) {
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii) {
-      const int i = 2 * pass + ii;
+    for (int ii = 0; ii < ROWS / 16; ++ii) {
+      const int i = (ROWS / 16) * pass + ii;
       const int row = 16 * ii + jn;
       const int m = wave_m0 + 16 * i + jn;
       const float brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
@@ -344,7 +350,7 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
       }
     }
 #pragma unroll 1
-    for (int it = 0; it < 16; ++it) {
+    for (int it = 0; it < ROWS / 2; ++it) {
       const int row = rd_row + 2 * it;
       const f32x4_t x = *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u +
                                                                   (uint32_t)((rd_chunk ^ (row & 31)) << 4));
@@ -353,7 +359,7 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
       uint32_t hi = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[2])) |
                     ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[3])) << 16);
       const u32x2_t w = {lo, hi};
-      const int mm = wave_m0 + 32 * pass + row;
+      const int mm = wave_m0 + ROWS * pass + row;
       const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
       __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, SRT_STORE_AUX);
     }
@@ -364,12 +370,14 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
 
 // Split-K pass: the fp32 accumulators go to a float workspace as they are ([batch][M][N], row
 // stride scm floats); a second kernel adds the passes and applies the epilogue.  Staged through
-// the wave's 16 KiB of LDS in four passes of 32 rows ([32 rows][32 chunks of 16 B], chunk c of row
+// the wave's LDS in passes of ROWS = 32 or 16 rows ([ROWS rows][32 chunks of 16 B], chunk c of row
 // r at c ^ (r & 31)) so that a store instruction writes two rows of 512 contiguous bytes: whole
 // cache lines (straight from the accumulator layout an instruction would write 16 rows x 64 bytes,
 // every line in two halves by different instructions; measured, the two take the same time).
-__device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0,
+template <int TM>
+__device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f32x4_t (&acc)[TM][8], int wave_m0,
                                                    int wave_n0, int bz, int lane, uint32_t stage) {
+  constexpr int ROWS = TM == 8 ? 32 : 16;
   float* C = (float*)p.C + (long long)bz * p.scb;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
   const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 4), 0x00020000);
@@ -379,10 +387,10 @@ __device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f
   const int n_rd = wave_n0 + 4 * rd_chunk;
   const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8: the four columns are in range together
 #pragma unroll
-  for (int pass = 0; pass < 4; ++pass) {
+  for (int pass = 0; pass < TM * 16 / ROWS; ++pass) {
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii) {
-      const int i = 2 * pass + ii;
+    for (int ii = 0; ii < ROWS / 16; ++ii) {
+      const int i = (ROWS / 16) * pass + ii;
       const int row = 16 * ii + jn;
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -393,7 +401,7 @@ __device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int it4 = 0; it4 < 4; ++it4) {
+    for (int it4 = 0; it4 < ROWS / 8; ++it4) {
       f32x4_t v[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
@@ -404,7 +412,7 @@ __device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = rd_row + 2 * (4 * it4 + q);
-        const int m = wave_m0 + 32 * pass + row;
+        const int m = wave_m0 + ROWS * pass + row;
         const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc4 + n_rd * 4) : OOB;
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v[q]), rc, (int)off, 0, 0);
       }
@@ -415,9 +423,66 @@ __device__ __forceinline__ void store_tile_partial(const GemmProblem& p, const f
   }
 }
 
-template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
+// ring::locate_tile for a tile of TILE_M x 256
+template <bool A_KC, bool B_KC, int TILE_M>
+__device__ __forceinline__ TileRef locate_tile(const GemmProblem& p, int v, int tiles_m, int tiles_n) {
+  const int per_batch = tiles_m * tiles_n;
+  const int bz = v / per_batch;
+  int tm, tn;
+  ring::tile_coords(v - bz * per_batch, tiles_m, tiles_n, &tm, &tn);
+  TileRef t;
+  t.m0 = tm * TILE_M;
+  t.n0 = tn * BN;
+  t.bz = bz;
+  const long long lda = A_KC ? p.sam : p.sak;
+  const long long ldb = B_KC ? p.sbn : p.sbk;
+  t.offa = (uint32_t)(((long long)bz * p.sab + (A_KC ? (long long)t.m0 * lda : (long long)t.m0)) * 2);
+  t.offb = (uint32_t)(((long long)bz * p.sbb + (B_KC ? (long long)t.n0 * ldb : (long long)t.n0)) * 2);
+  return t;
+}
+
+// Slot of a phase (MFMA index u) at which an event of the schedule happens, or its index if u is
+// such a slot (-1 otherwise).  TM = 8: phases of 32 MFMAs, TM = 4: of 16.
+template <int TM> constexpr int phase0_b_read(int u) {      // B tiles 4-7, before their first use at u = 2 TM
+  return TM == 8 ? ((u < 8 && (u & 1) == 0) ? u >> 1 : -1) : (u < 4 ? u : -1);
+}
+template <int TM> constexpr int phase0_a_read(int u) {      // A tiles of phase 1
+  return TM == 8 ? ((u >= 8 && u < 16 && (u & 1) == 0) ? (u - 8) >> 1 : -1) : ((u == 4 || u == 5) ? u - 4 : -1);
+}
+template <int TM> constexpr int phase0_b_load(int u) {      // the four B loads of the stage requested
+  return TM == 8 ? ((u >= 16 && (u & 3) == 0) ? (u - 16) >> 2 : -1) : ((u >= 8 && (u & 1) == 0) ? (u - 8) >> 1 : -1);
+}
+template <int TM> constexpr int phase0_scalar(int u) {      // scalar events 0..6 (TM = 4: 0 and 1 share a slot)
+  if (TM == 8) return (u >= 17 && (u & 1) == 1) ? (u - 17) >> 1 : -1;
+  switch (u) { case 6: return 0; case 7: return 2; case 9: return 3; case 11: return 4; case 13: return 5; case 15: return 6; default: return -1; }
+}
+template <int TM> constexpr int phase1_a_load(int u) {      // the TM / 2 A loads of the stage requested
+  return TM == 8 ? ((u >= 16 && (u & 3) == 0) ? (u - 16) >> 2 : -1) : ((u == 8 || u == 12) ? (u - 8) >> 2 : -1);
+}
+template <int TM> constexpr int phase1_a_read(int u) {      // A tiles of the next stage's phase 0
+  return TM == 8 ? ((u < 16 && (u & 3) == 1) ? u >> 2 : -1) : ((u == 0 || u == 2) ? u >> 1 : -1);
+}
+template <int TM> constexpr int phase1_b_read(int u) {      // B tile j < 4, right after its last MFMA of the stage
+  return TM == 8 ? ((u < 16 && (u & 3) == 3) ? u >> 2 : -1) : ((u < 8 && (u & 1) == 1) ? u >> 1 : -1);
+}
+template <int TM> constexpr int phase1_scalar(int u) {      // scalar events 0..3
+  return TM == 8 ? ((u >= 17 && u <= 23 && (u & 1) == 1) ? (u - 17) >> 1 : -1)
+                 : ((u >= 9 && (u & 1) == 1) ? (u - 9) >> 1 : -1);
+}
+
+// TM: 16-row A tiles per wave.  8: the 256 x 256 tile.  4: a 128 x 256 tile (A region of 128 rows,
+// k-contiguous A only), for problems that leave compute units idle with the large tile.
+template <typename T, bool A_KC, bool B_KC, int EPI, int NS, int TM = 8>
 __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
   static_assert(NS == 5, "ring depth");   // slot arithmetic below assumes the staging slots are NS-2, NS-1 ahead
+  static_assert(TM == 8 || (TM == 4 && A_KC), "the 128-row A region is k-contiguous");
+  constexpr int TILE_M = 32 * TM;                 // 256 or 128
+  constexpr int LPW_A = TM / 2;                   // A loads per wave and stage
+  constexpr int REGION_A = TILE_M * BK * 2;       // bytes of the A part of a stage; the B part (REGION) follows it
+  constexpr int STAGE_B = REGION_A + REGION;      // bytes of a stage
+  constexpr int LOADS = LPW_A + 4;                // loads per wave and stage
+  constexpr int HALF = TM / 2;                    // A tiles per phase
+  constexpr int SLOTS = 8 * HALF;                 // MFMAs per phase
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
 
@@ -427,9 +492,9 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     asm volatile("" : "+s"(zero));   // opaque: keeps the two instructions where they are written
     return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
   };
-  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+  const int wm0 = (wave >> 1) * (16 * TM), wn0 = (wave & 1) * 128;
 
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int tiles_m = (p.M + TILE_M - 1) / TILE_M, tiles_n = (p.N + BN - 1) / BN;
   const int total = tiles_m * tiles_n * p.batch;
   const int grid = (int)gridDim.x;
   int v = (int)blockIdx.x;
@@ -454,36 +519,37 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     return e;
   };
 
-  TileRef cur_tile = ring::locate_tile<A_KC, B_KC>(p, v, tiles_m, tiles_n);
+  TileRef cur_tile = locate_tile<A_KC, B_KC, TILE_M>(p, v, tiles_m, tiles_n);
 
   // Requests stages first .. NS-2 of `tile` and the A part of stage NS-1 (its B part is the first
   // thing the loop requests); stage t goes to the slot t places after `slot0`.
-  auto fill_ring = [&](const Loader<A_KC>& la, const Loader<B_KC>& lb, int lane, const TileRef& tile, uint32_t slot0,
-                       int first) {
+  auto fill_ring = [&](const Loader<A_KC, LPW_A>& la, const Loader<B_KC>& lb, int lane, const TileRef& tile,
+                       uint32_t slot0, int first) {
 #pragma unroll
     for (int t = 0; t < NS; ++t) {
       if (t < first) continue;
-      uint32_t slot = slot0 + (uint32_t)t * STAGE;
-      if (slot >= lds + NS * STAGE) slot -= NS * STAGE;
+      uint32_t slot = slot0 + (uint32_t)t * STAGE_B;
+      if (slot >= lds + NS * STAGE_B) slot -= NS * STAGE_B;
       const bool tail = (t == KT - 1) && ragged;
       const uint32_t soa = t < KT ? tile.offa + (uint32_t)stage_at(t) * kstep_a : OOB;
       const uint32_t sob = t < KT ? tile.offb + (uint32_t)stage_at(t) * kstep_b : OOB;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) la.issue_one(ra, slot, wave, lane, soa, i, tail, krem);
+      for (int i = 0; i < LPW_A; ++i) la.issue_one(ra, slot, wave, lane, soa, i, tail, krem);
       if (t < NS - 1) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lb.issue_one(rb, slot + REGION, wave, lane, sob, i, tail, krem);
+        for (int i = 0; i < 4; ++i) lb.issue_one(rb, slot + REGION_A, wave, lane, sob, i, tail, krem);
       }
     }
   };
 
-  uint32_t cur = lds, prv = lds + (NS - 1) * STAGE;
-  const uint32_t wave_lds = (uint32_t)wave * 4096u;   // this wave's 4 KiB share of an operand region
+  uint32_t cur = lds, prv = lds + (NS - 1) * STAGE_B;
+  const uint32_t wave_lds_a = (uint32_t)wave * (LPW_A * 1024u);   // this wave's share of an A region
+  const uint32_t wave_lds_b = (uint32_t)wave * 4096u;              // and of a B region
 
   bool first_tile = true;
   for (;;) {
     // per-lane addressing state, derived per tile and scoped to it (see gemm_ring_kernel)
-    Loader<A_KC> la;
+    Loader<A_KC, LPW_A> la;
     Loader<B_KC> lb;
     FragReader<A_KC> fa;
     FragReader<B_KC> fb;
@@ -494,7 +560,7 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     fb.init(lane, wn0);
     if (first_tile || !overlap) {
       fill_ring(la, lb, lane, cur_tile, cur, 0);
-      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(8 * (NS - 2) + 4) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(LOADS * (NS - 2) + LPW_A) : "memory");
     } else {
       fill_ring(la, lb, lane, cur_tile, cur, NS - 2);
     }
@@ -503,17 +569,16 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
 
     const int vn = v + grid;
     const bool has_next = vn < total;
-    const TileRef next_tile = ring::locate_tile<A_KC, B_KC>(p, has_next ? vn : v, tiles_m, tiles_n);
+    const TileRef next_tile = locate_tile<A_KC, B_KC, TILE_M>(p, has_next ? vn : v, tiles_m, tiles_n);
     const bool prefetch = overlap && has_next;
 
-    f32x4_t acc[8][8];   // defined by the MFMAs of the tile's first stage
+    f32x4_t acc[TM][8];   // defined by the MFMAs of the tile's first stage
 
-    u32x4_t af[8], bf[8];   // the stage's A and B tiles
+    u32x4_t af[TM], bf[8];   // the stage's A and B tiles
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      bf[t] = fb.read(cur + REGION, t);
-      af[t] = fa.read(cur, t);
-    }
+    for (int t = 0; t < 4; ++t) bf[t] = fb.read(cur + REGION_A, t);
+#pragma unroll
+    for (int t = 0; t < HALF; ++t) af[t] = fa.read(cur, t);
 
     const int limit = prefetch ? KT + NS - 2 : KT;   // requests below this index are real
     auto stage_of = [&](int r) {
@@ -536,7 +601,13 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     // reads take the first half of each phase (one every other MFMA), the loads the second half
     // (one every fourth), and the scalar bookkeeping of the requests is dealt out over the odd
     // slots of the second halves, a few instructions each.
-    uint32_t b_target = prv + REGION + wave_lds;   // landing address of the next B request
+    uint32_t b_target = prv + REGION_A + wave_lds_b;   // landing address of the next B request
+    auto set_target = [](int idx, uint32_t base) __attribute__((always_inline)) {
+      if (idx == 0) ring::set_lds_target<0>(base);
+      if (idx == 1) ring::set_lds_target<1024>(base);
+      if (idx == 2) ring::set_lds_target<2048>(base);
+      if (idx == 3) ring::set_lds_target<3072>(base);
+    };
     auto one_stage = [&](auto ragged_tag, auto first_tag, int kt) __attribute__((always_inline)) {
       constexpr bool RAGGED = decltype(ragged_tag)::value;
       constexpr bool FIRST = decltype(first_tag)::value;   // the tile's first stage: accumulators start here
@@ -548,70 +619,72 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
       }
       uint32_t nxt = 0, a_target = 0, sel = 0, sob_next = OOB;
       bool wrap = false;
-      // ---- phase 0: A tiles 0-3 ----
+      // ---- phase 0: the first half of the A tiles ----
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int u = j * 4 + i;   // 0..31
-          const bool load_here = u >= 16 && (u & 3) == 0;   // 16, 20, 24, 28
-          if (u == 16) ring::set_lds_target<0>(b_target);
-          if (u == 20) ring::set_lds_target<1024>(b_target);
-          if (u == 24) ring::set_lds_target<2048>(b_target);
-          if (u == 28) ring::set_lds_target<3072>(b_target);
-          if (load_here) SRT_FENCE();
+        for (int i = 0; i < HALF; ++i) {
+          const int u = j * HALF + i;   // 0 .. SLOTS - 1
+          const int ld = phase0_b_load<TM>(u);
+          if (ld >= 0) {
+            set_target(ld, b_target);
+            SRT_FENCE();
+          }
           if constexpr (FIRST) mfma16_first<T>(acc[i][j], bf[j], af[i]);
           else mfma16<T>(acc[i][j], bf[j], af[i]);
-          if (load_here) {
+          if (ld >= 0) {
             SRT_FENCE();
-            ring::load_to_lds_at_m0(rb, lb.voff[(u - 16) >> 2], sob);
+            ring::load_to_lds_at_m0(rb, lb.voff[ld], sob);
           }
-          // the rest of stage kt: B tiles 4-7 (first used by MFMA 16), A tiles 4-7 (phase 1)
-          if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.read(cur + REGION, 4 + (u >> 1));
-          if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.read(cur, 4 + ((u - 8) >> 1));
-          if (u == 17) nxt = cur + STAGE;
-          if (u == 19) nxt = nxt == lds + NS * STAGE ? lds : nxt;
+          // the rest of stage kt: B tiles 4-7 (first used half way through the phase), the A tiles of phase 1
+          const int rb_ = phase0_b_read<TM>(u), ra_ = phase0_a_read<TM>(u);
+          if (rb_ >= 0) bf[4 + rb_] = fb.read(cur + REGION_A, 4 + rb_);
+          if (ra_ >= 0) af[HALF + ra_] = fa.read(cur, HALF + ra_);
           // request r = ka: its A part goes out in phase 1, its B part in phase 0 of the next stage
-          if (u == 21) sel = ka < KT ? cur_tile.offa : next_tile.offa;
-          if (u == 23) soa = ka < limit ? sel + ea_off : OOB;
-          if (u == 25) sel = ka < KT ? cur_tile.offb : next_tile.offb;
-          if (u == 27) sob_next = ka < limit ? sel + eb_off : OOB;
-          if (u == 29) a_target = cur + wave_lds;
+          const int ev = phase0_scalar<TM>(u);
+          if (ev == 0) nxt = cur + STAGE_B;
+          if (ev == 1 || (TM == 4 && ev == 0)) nxt = nxt == lds + NS * STAGE_B ? lds : nxt;
+          if (ev == 2) sel = ka < KT ? cur_tile.offa : next_tile.offa;
+          if (ev == 3) soa = ka < limit ? sel + ea_off : OOB;
+          if (ev == 4) sel = ka < KT ? cur_tile.offb : next_tile.offb;
+          if (ev == 5) sob_next = ka < limit ? sel + eb_off : OOB;
+          if (ev == 6) a_target = cur + wave_lds_a;
           SRT_FENCE();
         }
       }
       // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
-      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(8 * (NS - 2)) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(LOADS * (NS - 2)) : "memory");
       SRT_FENCE();
-      // ---- phase 1: A tiles 4-7; reads of stage kt+1; A loads of stage kt+NS ----
+      // ---- phase 1: the second half of the A tiles; reads of stage kt+1; A loads of stage kt+NS ----
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int u = j * 4 + i;   // 0..31
-          const bool load_here = u >= 16 && (u & 3) == 0;   // 16, 20, 24, 28
-          if (u == 16) ring::set_lds_target<0>(a_target);
-          if (u == 20) ring::set_lds_target<1024>(a_target);
-          if (u == 24) ring::set_lds_target<2048>(a_target);
-          if (u == 28) ring::set_lds_target<3072>(a_target);
-          if (load_here) SRT_FENCE();
-          if constexpr (FIRST) mfma16_first<T>(acc[4 + i][j], bf[j], af[4 + i]);
-          else mfma16<T>(acc[4 + i][j], bf[j], af[4 + i]);
-          if (load_here) {
+        for (int i = 0; i < HALF; ++i) {
+          const int u = j * HALF + i;   // 0 .. SLOTS - 1
+          const int ld = phase1_a_load<TM>(u);
+          if (ld >= 0) {
+            set_target(ld, a_target);
             SRT_FENCE();
-            ring::load_to_lds_at_m0(ra, la.voff[(u - 16) >> 2], soa);
           }
-          // stage kt+1: A tiles 0-3 (idle since phase 0) and B tiles 0-3, each as it falls free
-          if (u < 16 && i == 1) af[j] = fa.read(nxt, j);
-          if (u < 16 && i == 3) bf[j] = fb.read(nxt + REGION, j);
+          if constexpr (FIRST) mfma16_first<T>(acc[HALF + i][j], bf[j], af[HALF + i]);
+          else mfma16<T>(acc[HALF + i][j], bf[j], af[HALF + i]);
+          if (ld >= 0) {
+            SRT_FENCE();
+            ring::load_to_lds_at_m0(ra, la.voff[ld], soa);
+          }
+          // stage kt+1: the A tiles of phase 0 (idle since then) and B tiles 0-3, each as it falls free
+          const int ra_ = phase1_a_read<TM>(u), rb_ = phase1_b_read<TM>(u);
+          if (ra_ >= 0) af[ra_] = fa.read(nxt, ra_);
+          if (rb_ >= 0) bf[rb_] = fb.read(nxt + REGION_A, rb_);
           // the stage of request r = ka + 1, and where its B part will land
-          if (u == 17) {
+          const int ev = phase1_scalar<TM>(u);
+          if (ev == 0) {
             wrap = e_req + 1 == KT;
             e_req = wrap ? 0 : e_req + 1;
           }
-          if (u == 19) ea_off = wrap ? 0u : ea_off + kstep_a;
-          if (u == 21) eb_off = wrap ? 0u : eb_off + kstep_b;
-          if (u == 23) b_target = cur + REGION + wave_lds;
+          if (ev == 1) ea_off = wrap ? 0u : ea_off + kstep_a;
+          if (ev == 2) eb_off = wrap ? 0u : eb_off + kstep_b;
+          if (ev == 3) b_target = cur + REGION_A + wave_lds_b;
           SRT_FENCE();
         }
       }
@@ -640,24 +713,24 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     // the staging area.  The s_nops are the wait states between the last MFMAs and the first
     // reads of their accumulators by other instructions.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
-    // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1 (16 KiB each)
-    uint32_t pprv = prv - STAGE;
-    if (prv == lds) pprv = lds + (NS - 1) * STAGE;
-    const uint32_t stage = ((wave & 2) ? prv : pprv) + (uint32_t)(wave & 1) * 16384u;
+    // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1 (half a slot each)
+    uint32_t pprv = prv - STAGE_B;
+    if (prv == lds) pprv = lds + (NS - 1) * STAGE_B;
+    const uint32_t stage = ((wave & 2) ? prv : pprv) + (uint32_t)(wave & 1) * (uint32_t)(STAGE_B / 2);
     const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
     const int le = lane_id();
 
     if (EPI == EPI_PARTIAL) {
-      store_tile_partial(p, acc, em0, en0, bz, le, stage);
+      store_tile_partial<TM>(p, acc, em0, en0, bz, le, stage);
     } else if (EPI == EPI_TRANS) {
-      store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
+      store_tile_transcendental<T, TM>(p, acc, em0, en0, bz, le, stage);
     } else {
-      if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
-      else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1>(p, acc, em0, en0, le);
-      else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1>(p, acc, em0, en0, le);
-      else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2>(p, acc, em0, en0, le);
-      if (EPI != EPI_PLAIN) pin_all(acc);
-      store_tile<T>(p, acc, em0, en0, bz, le, stage);
+      if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0, TM>(p, acc, em0, en0, le);
+      else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1, TM>(p, acc, em0, en0, le);
+      else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1, TM>(p, acc, em0, en0, le);
+      else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2, TM>(p, acc, em0, en0, le);
+      if (EPI != EPI_PLAIN) pin_all<TM>(acc);
+      store_tile<T, TM>(p, acc, em0, en0, bz, le, stage);
     }
     if (!has_next) break;
 
@@ -670,13 +743,14 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
 
 #undef SRT_FENCE
 
-template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
+template <typename T, bool A_KC, bool B_KC, int EPI, int NS, int TM = 8>
 hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
-  auto kernel = gemm_m16_kernel<T, A_KC, B_KC, EPI, NS>;
-  constexpr int lds_bytes = NS * STAGE;
+  auto kernel = gemm_m16_kernel<T, A_KC, B_KC, EPI, NS, TM>;
+  constexpr int tile_m = 32 * TM;
+  constexpr int lds_bytes = NS * (tile_m * BK * 2 + REGION);
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
-  const long long tiles = (long long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN) * p.batch;
+  const long long tiles = (long long)((p.M + tile_m - 1) / tile_m) * ((p.N + BN - 1) / BN) * p.batch;
   int grid = ring::compute_units() & ~7;
   if (grid <= 0) grid = 8;
   if (tiles < grid) grid = (int)tiles;
@@ -684,18 +758,18 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <typename T, bool A_KC, bool B_KC, int NS = 5>
+template <typename T, bool A_KC, bool B_KC, int NS = 5, int TM = 8>
 hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
                      p.activation == srtActivationElu;
-  if (trans) return launch_kernel<T, A_KC, B_KC, EPI_TRANS, NS>(p, stream);
-  if (p.activation == srtActivationClippedRelu) return launch_kernel<T, A_KC, B_KC, EPI_CLIPPED, NS>(p, stream);
+  if (trans) return launch_kernel<T, A_KC, B_KC, EPI_TRANS, NS, TM>(p, stream);
+  if (p.activation == srtActivationClippedRelu) return launch_kernel<T, A_KC, B_KC, EPI_CLIPPED, NS, TM>(p, stream);
   if (p.activation == srtActivationRelu) {
-    if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS_RELU, NS>(p, stream);
-    return launch_kernel<T, A_KC, B_KC, EPI_RELU, NS>(p, stream);
+    if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS_RELU, NS, TM>(p, stream);
+    return launch_kernel<T, A_KC, B_KC, EPI_RELU, NS, TM>(p, stream);
   }
-  if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS, NS>(p, stream);
-  return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS>(p, stream);
+  if (p.bias) return launch_kernel<T, A_KC, B_KC, EPI_BIAS, NS, TM>(p, stream);
+  return launch_kernel<T, A_KC, B_KC, EPI_PLAIN, NS, TM>(p, stream);
 }
 
 // The split-K pass of `p` (whose C is the float workspace and whose batch counts the k ranges).

@@ -88,11 +88,11 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
 // (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
 // and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
 enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK,
-            kPlanKc64, kPlanM16, kPlanSplitK, kPlanCount };
+            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanCount };
 
 const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
                                             "f32_mfma_64x64", "f32_mfma_splitk", "mfma_256x256_k64",
-                                            "mfma_256x256_m16", "mfma_256x256_splitk"};
+                                            "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16"};
 
 bool plan_supported(const GemmProblem& p, Plan plan) {
   switch (plan) {
@@ -103,6 +103,7 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
     case kPlanKc64: return srt::mfma_config(p, 4) != 0;
     case kPlanM16: return srt::mfma_config(p, 5) != 0;
     case kPlanSplitK: return srt::mfma_splitk_parts(p) >= 2;
+    case kPlanM16H: return srt::mfma_config(p, 6) != 0;
     case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
     case kPlanF32SplitK: return srt::f32_mfma_supported(p);
     default: return srt::generic_supported(p);
@@ -124,6 +125,7 @@ Plan heuristic_plan(const GemmProblem& p) {
       case 2: return kPlanMfma128;
       case 4: return kPlanKc64;
       case 5: return kPlanM16;
+      case 6: return kPlanM16H;
       default: return kPlanMfma64;
     }
   }
@@ -140,6 +142,7 @@ hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
     case kPlanKc64: return srt::launch_mfma(p, srt::mfma_config(p, 4), stream);
     case kPlanM16: return srt::launch_mfma(p, srt::mfma_config(p, 5), stream);
     case kPlanSplitK: return srt::launch_mfma_splitk(p, stream);
+    case kPlanM16H: return srt::launch_mfma(p, srt::mfma_config(p, 6), stream);
     case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
     case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
     default: return srt::launch_generic(p, stream);

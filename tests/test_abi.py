@@ -171,7 +171,7 @@ def test_plan_cache_file_round_trip_and_rejects_malformed_files(tmp_path):
     srt.PlanCache.clear()
     assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
                                   buf, 64) == 0
-    assert buf.value == b"mfma_256x256"
+    assert buf.value == b"mfma_128x256_m16"
     assert L.srtPlanCacheCount(None) == native.ERROR_INVALID_VALUE
     assert L.srtPlanCacheLoad(None) == native.ERROR_INVALID_VALUE
 
@@ -208,9 +208,14 @@ def test_kernel_selection_is_queryable_without_gpu():
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16"             # 144 tiles, long k loop
     assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256"
-    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_256x256"                 # 64 tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_64x64"
-    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_64x64"                    # 32 tiles, K too short to split
+    # a k-contiguous A and at most one round of 128 x 256 tiles: the half-height form of the 16x16x32 kernel
+    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16"             # 128 half tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16"
+    assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16"             # 256 half tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256"        # A not k-contiguous: whole tiles
+    assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
+    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16"              # K too short to split
+    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_64x64"                     # and too short for the ring
     assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"

@@ -600,6 +600,70 @@ def test_splitk_is_the_choice_for_few_tiles_and_long_k():
     assert query_kernel(a2, False, b2, False, out) != "mfma_256x256_splitk"
 
 
+# ---- the 128 x 256 form of the 16x16x32 kernel ---------------------------------------------------------
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("tb", [False, True])
+def test_m16_half_tile_integer_bit_exact_random_and_batched(dt, tb, tmp_path):
+    """k-contiguous A against both B layouts; ragged edges in M (not a multiple of 128) and N, K below one
+    stage, ending inside a stage, fewer stages than the ring holds; several tiles per workgroup; a batch."""
+    r = H.rng(320)
+    for (M, N, K) in [(128, 256, 32), (136, 264, 8), (1000, 776, 200), (2048, 2056, 328), (4360, 4360, 72)]:
+        pin_plan(tmp_path, "mfma_128x256_m16", dt, M, N, K, False, tb)
+        a = r.integers(-3, 4, (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+        got = gpu_matmul(H.encode(a, dt), H.encode(b, dt), False, tb, want_kernel="mfma_128x256_m16")
+        exact = a.astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+        assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    M, N, K = 1160, 1032, 264
+    pin_plan(tmp_path, "mfma_128x256_m16", dt, M, N, K, False, tb)
+    a = (r.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+    b = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    a_st, b_st = H.encode(a, dt), H.encode(b, dt)
+    check_against_fp64(gpu_matmul(a_st, b_st, False, tb, want_kernel="mfma_128x256_m16"), a_st, b_st, False, tb, dt)
+    srt.PlanCache.clear()
+    # the heuristic's own choice, batched: 3 x 6 x 4 half tiles
+    B_, M, N, K = 3, 768, 1024, 520
+    a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+    w = r.integers(-3, 4, (B_, N, K) if tb else (B_, K, N)).astype(np.float32)
+    at, wt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(w, dt))
+    out = srt.matmul(at, wt, transposed_rhs=tb)
+    if not tb:
+        assert query_kernel(at, False, wt, tb, out) == "mfma_128x256_m16"
+    exact = a.astype(np.float64) @ (np.swapaxes(w, 1, 2) if tb else w).astype(np.float64)
+    assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
+
+
+@pytest.mark.parametrize("act", list(srt.ActivationType))
+def test_m16_half_tile_epilogues_vs_oracle_and_nan(act, tmp_path):
+    r = H.rng(321)
+    dt = H.BF16
+    M, N, K = 1100, 520, 200
+    x = H.encode(r.standard_normal((M, K)).astype(np.float32), dt)
+    w = H.encode((r.standard_normal((K, N)) / 8).astype(np.float32), dt)
+    b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
+    coef = 0.75
+    pin_plan(tmp_path, "mfma_128x256_m16", dt, M, N, K, False, False, bias=True, act=act)
+    xt, wt, bt = srt.Tensor(x), srt.Tensor(w), srt.Tensor(b)
+    out = srt.Tensor(shape=[M, N], dtype=x.dtype)
+    srt.current_queue().matmul(xt, False, wt, False, out, bias=bt, activation=act, coef=coef)
+    got = H.decode(out.array())
+    rows = np.concatenate([np.arange(0, M, 61), [M - 1]])
+    want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, transpose_w=False,
+                                      acc=ora.ACC_F32, fused=True))
+    assert np.all(np.abs(got[rows] - want) <= 2.0 ** -7 * np.maximum(np.abs(want), 1.0))
+    if act == srt.ActivationType.identity:
+        a = np.zeros((M, 64), np.float32)
+        w2 = np.zeros((64, N), np.float32)
+        a[:, 0] = 1.0
+        w2[0, :] = 2.0
+        a[5, 1] = np.nan
+        w2[1, :] = 1.0
+        pin_plan(tmp_path, "mfma_128x256_m16", dt, M, N, 64, False, False)
+        got = gpu_matmul(H.encode(a, dt), H.encode(w2, dt), want_kernel="mfma_128x256_m16")
+        assert np.all(got[5] == 0x7FFF) and np.all(got[6] == H.encode(np.array([2.0], np.float32), dt)[0])
+    srt.PlanCache.clear()
+
+
 def test_m16_kernel_is_the_choice_for_a_full_device_and_long_k():
     a = srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16))
     b = srt.Tensor(H.encode(np.zeros((2048, 4096), np.float32), H.BF16))
