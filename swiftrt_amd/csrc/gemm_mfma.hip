@@ -433,7 +433,7 @@ int mfma_select(const GemmProblem& p) {
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
   // Tile choice, from measurements over mid-size problems (1024^3 .. 4096 x 14336 x 4096):
   //  * the 256 x 256 kernels are so much more efficient per tile (deep prefetch, 4x the arithmetic
-  //    intensity) that they win long before they can fill the device: from 48 tiles up for the
+  //    intensity) that they win long before they can fill the device: from 24 tiles up (48 when K < 1024) for the
   //    ring kernel (3072^3, 144 tiles: 64 us against 143 us with 128 x 128 tiles);
   //  * with both operands k-contiguous the 64 x 64 kernel reads whole lines too and stays ahead up
   //    to about 96 tiles of 256 x 256 (2048^3 NT: 36 us against 44 us); from there the ring kernel
@@ -455,17 +455,27 @@ int mfma_select(const GemmProblem& p) {
   const bool big_ok = ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0);
   const long long t256 = tiles(256);
   //  * with a k-contiguous A the 16x16x32 kernel also comes with 128 x 256 tiles: twice the
-  //    workgroups, which is what a problem that leaves compute units idle needs, as long as they
-  //    all run at once (2048^3: 29 us against 42 us; 512 x 14336 x 4096: 59 against 82;
-  //    2048 x 4096 x 2048, 256 half tiles: 35 against 47; 3072 x 3072 x 1024, 288 half tiles: 32.5
-  //    against 28 for whole tiles).  With a k-contiguous B as well the 64 x 64 kernel is as good
-  //    up to about 96 such tiles (1024 x 1024 x 2048: 20 us against 23 us).
+  //    workgroups, which is what a problem that leaves compute units idle needs (2048^3: 29 us
+  //    against 42 us; 512 x 14336 x 4096: 59 against 82; 256 x 1024 x 1024: 15 against 19 for 64 x 64
+  //    tiles).  On a full device a half tile costs about 0.6 of a whole one (4096^3: 129 us
+  //    against 105 us), so the choice goes by rounds of the persistent grid: half tiles when
+  //    0.6 x their rounds does not exceed the whole tiles' rounds -- always when they fit in one
+  //    round (2048 x 4096 x 2048: 35 us against 47 us), and where whole tiles quantise badly
+  //    (1536 x 11008 x 4096, 258 tiles: 152 us against 171 us; 3072 x 3072 x 1024, 144 tiles
+  //    against 288 halves: 28 us whole, 32.5 us halves).  With a k-contiguous B as well the half
+  //    tile is dearer (0.68: both operands arrive as half cache lines), so there it is taken only
+  //    when it fits in one round (1536 x 11008 x 4096 NT: 190 us against 168 us whole), and the
+  //    64 x 64 kernel is as good up to about 96 half tiles (1024 x 1024 x 2048: 20 us against 23 us).
   const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
+  const long long cus = 256;
+  const long long rounds256 = (t256 + cus - 1) / cus, rounds_h = (th + cus - 1) / cus;
   int tile;
-  if (big_ok && (layout & 2) != 0 && th <= 256 && th >= (layout == 3 ? 96 : 24) && p.K >= 512) tile = 6;
+  if (big_ok && (layout & 2) != 0 && p.K >= 512 && th >= (layout == 3 ? 96 : 8) &&
+      (layout == 3 ? rounds_h == 1 : 6 * rounds_h <= 10 * rounds256))
+    tile = 6;
   else if (big_ok && t256 >= 128 && p.K >= 2048) tile = 5;
   else if (big_ok && layout == 3 && t256 >= 192) tile = 4;
-  else if (big_ok && t256 >= (layout == 3 ? 96 : 48)) tile = 1;
+  else if (big_ok && t256 >= (layout == 3 ? 96 : (p.K >= 1024 ? 24 : 48))) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
@@ -536,6 +546,28 @@ int mfma_splitk_parts(const GemmProblem& p) {
     parts = s;
   }
   return parts;
+}
+
+// Whether the heuristic takes the split-K plan.  The fp32 parts cost a fixed 25-30 us to write and
+// add up (about 67 MB each way whatever the shape), and with a k-contiguous A the 128 x 256 tiles
+// already double the workgroups at no such cost, so the split must buy more than that:
+//   A not k-contiguous      four parts from K = 2048 (256 x 2048 x 2048 TN: 27 us against 45 us for
+//                           64 x 64 tiles), two from K = 4096 (2048 x 4096 x 4096 TN: 77 us against
+//                           87 us; at K = 2048 two parts lose, 1024 x 8192 x 2048: 56 against 47)
+//   A and B k-contiguous    four parts from K = 4096 (768 x 4096 x 4096: 47 us against 52 us for half
+//                           tiles), two from K = 8192 (1536 x 4096 x 11008: 136 us against 168 us)
+//   A k-, B n-contiguous    eight parts from K = 4096 (512 x 4096 x 4096: 43 us against ~50 us for half
+//                           tiles; with four parts the two tie), four from K = 8192 (2048 x 2048 x
+//                           8192: 79 us); two parts lose to half tiles (2048 x 4096 x 11008: 183
+//                           against 154)
+bool mfma_prefers_splitk(const GemmProblem& p) {
+  const int parts = mfma_splitk_parts(p);
+  if (parts < 2) return false;
+  const int layout = mfma_layout(p);
+  if ((layout & 2) == 0) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
+  if (p.K < 4096) return false;
+  if (layout == 3) return parts >= 4 || p.K >= 8192;
+  return parts >= 8 || (parts >= 4 && p.K >= 8192);
 }
 
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {

@@ -112,12 +112,8 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 
 Plan heuristic_plan(const GemmProblem& p) {
   if (srt::skinny_supported(p)) return kPlanSkinny;
-  // Few 256 x 256 tiles and a long k loop: split K over the idle compute units.  The fp32 parts cost
-  // a fixed 25-30 us to write and add up (about 67 MB each way whatever the shape), so this pays
-  // from K = 4096 up (1024 x 4096 x 4096: 55 us against 75 us; 256 x 8192 x 8192: 62 against 129;
-  // 1024 x 1024 x 4096: 34 against 64) and not below (2048^3: 44 us against 41 us).
-  if (p.K >= 4096 && (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) <= 96 && srt::mfma_splitk_parts(p) >= 2)
-    return kPlanSplitK;
+  // few 256 x 256 tiles and a long k loop: K split over the idle compute units
+  if (srt::mfma_prefers_splitk(p)) return kPlanSplitK;
   const int c = srt::mfma_select(p);
   if (c) {
     switch (c >> 2) {

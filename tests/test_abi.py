@@ -200,11 +200,18 @@ def test_kernel_selection_is_queryable_without_gpu():
     # short k loops: the 32x32x16 kernels (64-deep stages when both operands are k-contiguous)
     assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256"
     assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_k64"
-    # few tiles and a long k loop: K split over the idle compute units
-    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_256x256_splitk"
+    # few tiles and a long k loop: K split over the idle compute units -- when that buys more than the
+    # half-height tiles a k-contiguous A allows
+    assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_256x256_splitk"           # eight parts
     assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_128x256_m16"             # four parts: half tiles tie, no workspace
+    assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_256x256_splitk"          # four parts, K = 8192
     assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_256x256_splitk"
-    # mid-size problems: the 256 x 256 kernels from 48 tiles up (96 when both operands are k-contiguous),
+    assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: from K = 2048
+    assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x256"        # 32 tiles: the ring from 24 up
+    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_64x64"          # 16 tiles
+    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x256_m16"    # two parts at K = 2048 do not pay
+    # mid-size problems: the 256 x 256 kernels from 24 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16"             # 144 tiles, long k loop
     assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256"
@@ -212,7 +219,12 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16"             # 128 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16"
     assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16"             # 256 half tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256"        # A not k-contiguous: whole tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: whole tiles, K split
+    assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x256"
+    assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_128x256_m16"            # 258 whole tiles: two rounds for two tiles
+    assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16"   # both k-contiguous: one round of halves or none
+    assert query(native.REAL16BF, 1536, 4096, 11008, tb=True) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16"              # 8 half tiles
     assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
     assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16"              # K too short to split
     assert query(native.REAL16BF, 512, 4096, 256) == "mfma_64x64"                     # and too short for the ring
