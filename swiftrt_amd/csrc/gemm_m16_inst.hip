@@ -19,9 +19,12 @@ hipError_t SRT_CAT(launch_m16_partial, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(c
 }
 
 #if SRT_M16_AKC
-// launch_m16h_<type>_1<bkc>: the 128 x 256 tile (k-contiguous A only)
+// launch_m16h_<type>_1<bkc>: the 128 x 256 tile (k-contiguous A only), and its split-K pass
 hipError_t SRT_CAT(launch_m16h, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const GemmProblem& p, hipStream_t stream) {
   return m16::launch<SRT_M16_TYPE, true, SRT_M16_BKC != 0, 5, 4>(p, stream);
+}
+hipError_t SRT_CAT(launch_m16h_partial, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const GemmProblem& p, hipStream_t stream) {
+  return m16::launch_partial<SRT_M16_TYPE, true, SRT_M16_BKC != 0, 5, 4>(p, stream);
 }
 #endif
 

@@ -57,6 +57,10 @@ hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_F16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_F16_11(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_partial_BF16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_partial_BF16_11(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_partial_F16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16h_partial_F16_11(const GemmProblem&, hipStream_t);
 
 namespace {
 
@@ -538,7 +542,8 @@ int mfma_splitk_parts(const GemmProblem& p) {
   if (layout < 0 || p.batch != 1) return 0;
   if (!ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
   if ((reinterpret_cast<uintptr_t>(p.C) & 15u) != 0 || (p.scm % 8) != 0) return 0;
-  const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256);
+  // a k-contiguous A of at most 128 rows runs the pass on 128 x 256 tiles (half the padding to multiply)
+  const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256);   // also the count of half tiles then
   int parts = 0;
   for (int s = 2; s <= 16; s *= 2) {
     if (t256 * s > 256) break;
@@ -554,20 +559,22 @@ int mfma_splitk_parts(const GemmProblem& p) {
 //   A not k-contiguous      four parts from K = 2048 (256 x 2048 x 2048 TN: 27 us against 45 us for
 //                           64 x 64 tiles), two from K = 4096 (2048 x 4096 x 4096 TN: 77 us against
 //                           87 us; at K = 2048 two parts lose, 1024 x 8192 x 2048: 56 against 47)
+//   A k-contiguous, M <= 128  the same rule (the pass runs on 128 x 256 tiles: 64 x 2048 x 2048: 18 us
+//                           against 25 us for half tiles alone; 64 x 14336 x 4096: 32 us against 46 us)
 //   A and B k-contiguous    four parts from K = 4096 (768 x 4096 x 4096: 47 us against 52 us for half
 //                           tiles), two from K = 8192 (1536 x 4096 x 11008: 136 us against 168 us)
 //   A k-, B n-contiguous    eight parts from K = 4096 (512 x 4096 x 4096: 43 us against ~50 us for half
 //                           tiles; with four parts the two tie), four from K = 8192 (2048 x 2048 x
-//                           8192: 79 us); two parts lose to half tiles (2048 x 4096 x 11008: 183
-//                           against 154)
+//                           8192: 79 us) or when M <= 256 (64 x 14336 x 4096: 37 us against 46 us);
+//                           two parts lose to half tiles (2048 x 4096 x 11008: 183 against 154)
 bool mfma_prefers_splitk(const GemmProblem& p) {
   const int parts = mfma_splitk_parts(p);
   if (parts < 2) return false;
   const int layout = mfma_layout(p);
-  if ((layout & 2) == 0) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
+  if ((layout & 2) == 0 || p.M <= 128) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;
-  return parts >= 8 || (parts >= 4 && p.K >= 8192);
+  return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 256));
 }
 
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {
@@ -589,8 +596,14 @@ hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {
   q.scb = (long long)p.M * p.N;
   q.bias = nullptr;
   q.activation = srtActivationIdentity;
-  hipError_t e = p.dtype == srtReal16BF ? launch_m16_partial<BF16>(q, a_kc, b_kc, stream)
-                                        : launch_m16_partial<F16>(q, a_kc, b_kc, stream);
+  hipError_t e;
+  if (a_kc && p.M <= 128) {
+    if (p.dtype == srtReal16BF) e = b_kc ? launch_m16h_partial_BF16_11(q, stream) : launch_m16h_partial_BF16_10(q, stream);
+    else e = b_kc ? launch_m16h_partial_F16_11(q, stream) : launch_m16h_partial_F16_10(q, stream);
+  } else {
+    e = p.dtype == srtReal16BF ? launch_m16_partial<BF16>(q, a_kc, b_kc, stream)
+                               : launch_m16_partial<F16>(q, a_kc, b_kc, stream);
+  }
   if (e == hipSuccess) {
     const long long lanes = (long long)p.M * (p.N / 8);
     const unsigned blocks = (unsigned)((lanes + 255) / 256);

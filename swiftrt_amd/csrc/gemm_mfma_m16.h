@@ -773,9 +773,9 @@ hipError_t launch(const GemmProblem& p, hipStream_t stream) {
 }
 
 // The split-K pass of `p` (whose C is the float workspace and whose batch counts the k ranges).
-template <typename T, bool A_KC, bool B_KC, int NS = 5>
+template <typename T, bool A_KC, bool B_KC, int NS = 5, int TM = 8>
 hipError_t launch_partial(const GemmProblem& p, hipStream_t stream) {
-  return launch_kernel<T, A_KC, B_KC, EPI_PARTIAL, NS>(p, stream);
+  return launch_kernel<T, A_KC, B_KC, EPI_PARTIAL, NS, TM>(p, stream);
 }
 
 }  // namespace m16

@@ -545,7 +545,7 @@ def pin_plan(tmp_path, plan, dt, M, N, K, ta, tb, bias=False, act=srt.Activation
 def test_splitk_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
     """K cut into 2, 4 and 8 parts; ragged M and N edges; every staging layout."""
     r = H.rng(310)
-    for (M, N, K) in [(512, 520, 1024), (304, 264, 2048), (200, 1032, 4096)]:
+    for (M, N, K) in [(512, 520, 1024), (304, 264, 2048), (200, 1032, 4096), (96, 520, 2048), (128, 264, 4096)]:
         pin_plan(tmp_path, "mfma_256x256_splitk", dt, M, N, K, ta, tb)
         a = r.integers(-2, 3, (K, M) if ta else (M, K)).astype(np.float32)
         b = r.integers(-2, 3, (N, K) if tb else (K, N)).astype(np.float32)
