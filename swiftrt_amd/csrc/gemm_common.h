@@ -168,6 +168,7 @@ bool mfma_prefers_splitk(const GemmProblem& p);
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream);
 
 bool skinny_supported(const GemmProblem& p);
+bool skinny_preferred(const GemmProblem& p);   // the heuristic's choice among the problems it supports
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t stream);
 
 bool f32_mfma_supported(const GemmProblem& p);

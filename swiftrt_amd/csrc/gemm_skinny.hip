@@ -1,4 +1,4 @@
-// Small-M matmul (M <= 32) against a k-contiguous weight: out[m, n] = sum_k x[m, k] * W[n, k].
+// Small-M matmul (M <= 64) against a k-contiguous weight: out[m, n] = sum_k x[m, k] * W[n, k].
 // The shape of single-token / small-batch inference; bound by streaming W from HBM once.
 //
 //   block   4 waves share 32 rows of W (one 32 x 32 output tile; rows m >= M are zero).  Wave w
@@ -16,6 +16,7 @@
 //           vector-memory instructions are global->LDS loads and its only register-producing
 //           loads are LDS reads.
 //   grid    ceil(N / 32) x batch workgroups of 60-72 KiB LDS: two per CU, all resident at once.
+//   M > 32  two 32-row output tiles per 32 rows of W (the x fragments of both meet each W fragment)
 //   M > 16  x is as large per k block as the 32 rows of W it meets, and every workgroup re-reads it
 //           from L2: when N is large enough to keep most CUs busy that way, a workgroup takes 64
 //           rows of W (two output tiles per wave sharing the x fragments): 12 loads per k block and
@@ -54,11 +55,12 @@ constexpr uint32_t SK_OOB = 0x80000000u;
 // 160 KiB of LDS with two workgroups per CU (NW = 1) or one (NW = 2).
 template <int XR, int NW>
 struct SkinnyShape {
-  static constexpr int DEPTH = NW == 2 ? 3 : (XR == 32 ? 2 : 3);   // k blocks in flight per wave
+  static constexpr int MT = (XR + 31) / 32;                          // 32-row output tiles along M
+  static constexpr int DEPTH = XR == 64 ? (NW == 2 ? 2 : 3) : NW == 2 ? 3 : (XR == 32 ? 2 : 3);   // k blocks in flight per wave
   static constexpr int WBYTES = NW * SK_WTILE;                      // W part of a ring slot
   static constexpr int SLOT = WBYTES + XR * 128;                    // W rows + x rows of one k block
   static constexpr int LOADS = 4 * NW + XR / 8;                     // load instructions per k block
-  static constexpr int LDS = SK_WAVES * DEPTH * SLOT;               // 60 / 72 / 64 KiB; 144 KiB for NW = 2
+  static constexpr int LDS = SK_WAVES * DEPTH * SLOT;               // 60 / 72 / 64 KiB; 128-144 KiB for NW = 2 or XR = 64
 };
 
 // STREAM: the data is read once by the whole grid (the weight), so the load carries the
@@ -80,7 +82,7 @@ __device__ __forceinline__ void sk_load_to_lds(u32x4_t rsrc, uint32_t lds_addr, 
   }
 }
 
-// XR = number of x rows staged per k block (8, 16 or 32 >= M).
+// XR = number of x rows staged per k block (8, 16, 32 or 64 >= M).
 // Every vector-memory instruction in the k loop is a global->LDS load issued from inline assembly
 // and awaited with explicit s_waitcnt vmcnt; everything that produces registers is an LDS read,
 // which the compiler tracks on its own counter.
@@ -88,6 +90,7 @@ template <typename T, int XR, int NW>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem p) {
   using Shape = SkinnyShape<XR, NW>;
   constexpr int SK_WBYTES = Shape::WBYTES;
+  constexpr int MT = Shape::MT;
   constexpr int DEPTH = Shape::DEPTH;
   extern __shared__ __attribute__((aligned(1024))) unsigned char sk_lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)sk_lds_raw;
@@ -137,7 +140,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   uint32_t rd[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s) rd[s] = (uint32_t)(r * 128 + (((2 * s + h) ^ ((r >> 1) & 7)) << 4));
-  const bool x_lane = r < XR;   // lanes of rows that are not staged hold zero operands
+  const bool x_lane = XR >= 32 || r < XR;   // lanes of rows that are not staged hold zero operands
 
   const int KB = (p.K + SK_KB - 1) / SK_KB;   // k blocks in total; this wave takes wave, wave + 4, ...
   const int k_chunks = p.K / 8;                // valid 16-byte chunks per row
@@ -158,11 +161,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     }
   };
 
-  f32x16_t acc[NW];
+  f32x16_t acc[NW][MT];
 #pragma unroll
   for (int t = 0; t < NW; ++t)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[t][mt][v] = 0.0f;
 
   // This wave's k blocks are wave, wave + 4, ... (count of them); it walks them in rotated
   // order, starting at a block that depends on the workgroup, so that the workgroups resident at
@@ -189,14 +194,17 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
       const int j = j0 + d;
       asm volatile("s_waitcnt vmcnt(%0)" : : "i"(Shape::LOADS * (DEPTH - 1)) : "memory");
       const uint32_t base = my_ring + (uint32_t)d * Shape::SLOT;
-      u32x4_t wf[NW][4], xf[4];
+      u32x4_t wf[NW][4], xf[MT][4];
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
 #pragma unroll
         for (int t = 0; t < NW; ++t) wf[t][s] = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + t * SK_WTILE + rd[s]);
-        u32x4_t x = {0u, 0u, 0u, 0u};
-        if (x_lane) x = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + SK_WBYTES + rd[s]);
-        xf[s] = x;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          u32x4_t x = {0u, 0u, 0u, 0u};
+          if (x_lane) x = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + SK_WBYTES + mt * 4096 + rd[s]);
+          xf[mt][s] = x;
+        }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // fragments are in registers: the slot is free
       issue(block_at(j + DEPTH), d);
@@ -204,18 +212,22 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-          for (int t = 0; t < NW; ++t) acc[t] = mfma32s<T>(xf[s], wf[t][s], acc[t]);
+          for (int t = 0; t < NW; ++t)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[t][mt] = mfma32s<T>(xf[mt][s], wf[t][s], acc[t][mt]);
       }
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();   // every wave's loads have landed and its ring is idle: reuse LDS for the reduction
 
-  float* red = reinterpret_cast<float*>(sk_lds_raw);   // [NW tiles][4 waves][16][64] = NW x 16 KiB
+  float* red = reinterpret_cast<float*>(sk_lds_raw);   // [NW x MT tiles][4 waves][16][64] = NW x MT x 16 KiB
 #pragma unroll
   for (int t = 0; t < NW; ++t)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) red[((t * SK_WAVES + wave) * 16 + v) * 64 + lane] = acc[t][v];
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) red[(((t * MT + mt) * SK_WAVES + wave) * 16 + v) * 64 + lane] = acc[t][mt][v];
   __syncthreads();
 
   // wave w finishes accumulator registers 4w .. 4w+3: rows m = 8 w + 4 h + i, column n
@@ -227,15 +239,18 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     if (n >= p.N) continue;
     const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int v = 4 * wave + i;
-      const int m = 8 * wave + 4 * h + i;
-      if (m >= p.M) continue;
-      float s = 0.0f;
+    for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-      for (int w = 0; w < SK_WAVES; ++w) s += red[((t * SK_WAVES + w) * 16 + v) * 64 + lane];
-      const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
-      C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, bv);
+      for (int i = 0; i < 4; ++i) {
+        const int v = 4 * wave + i;
+        const int m = 32 * mt + 8 * wave + 4 * h + i;
+        if (m >= p.M) continue;
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) s += red[(((t * MT + mt) * SK_WAVES + w) * 16 + v) * 64 + lane];
+        const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
+        C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, bv);
+      }
     }
   }
 }
@@ -256,8 +271,12 @@ hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
   if (p.M <= 16) return launch_skinny_shape<T, 16, 1>(p, stream);
   // two W tiles per workgroup once that still gives most CUs a workgroup (192 of them)
   const long long wide_groups = (long long)((p.N + 63) / 64) * p.batch;
-  if (wide_groups >= 192) return launch_skinny_shape<T, 32, 2>(p, stream);
-  return launch_skinny_shape<T, 32, 1>(p, stream);
+  if (p.M <= 32) {
+    if (wide_groups >= 192) return launch_skinny_shape<T, 32, 2>(p, stream);
+    return launch_skinny_shape<T, 32, 1>(p, stream);
+  }
+  if (wide_groups >= 192) return launch_skinny_shape<T, 64, 2>(p, stream);
+  return launch_skinny_shape<T, 64, 1>(p, stream);
 }
 
 inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
@@ -266,7 +285,7 @@ inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 
 bool skinny_supported(const GemmProblem& p) {
   if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return false;
-  if (p.M > 32 || p.M < 1 || p.K < 1) return false;
+  if (p.M > 64 || p.M < 1 || p.K < 1) return false;
   if (p.sak != 1 || p.sbk != 1) return false;           // both operands k-contiguous
   if ((p.K % 8) != 0) return false;                     // whole 16-byte chunks
   if ((p.sam % 8) != 0 && p.M > 1) return false;
@@ -279,6 +298,21 @@ bool skinny_supported(const GemmProblem& p) {
   if (((long long)p.N + 32) * p.sbn + p.K >= (0x7fffffffLL / 2 - 4096)) return false;
   // worth it only when the weight dominates the traffic
   return p.N >= 32;
+}
+
+// Whether the heuristic takes this kernel for a problem it supports.  Up to M = 32 always.  With
+// 33..64 rows a workgroup needs 128-144 KiB of LDS, one fits per compute unit, and the kernel pays
+// only when its workgroups run in a single round that keeps most units streaming: 192..256
+// workgroups of 64 weight rows (64 x 14336 x 4096: 26.5 us against 32 us for split-K), or at most
+// 256 of 32 rows unless they are few and the k loop is long (64 x 4096 x 4096, 128 workgroups: 17 us
+// against 21 us; 64 x 4096 x 14336: 51 us against 35 us; 64 x 11008 x 4096, 344 workgroups: 34 us
+// against 29 us; 64 x 32768 x 1024: 22 us against 17 us for 64 x 64 tiles).
+bool skinny_preferred(const GemmProblem& p) {
+  if (p.M <= 32) return true;
+  const long long groups64 = (long long)((p.N + 63) / 64) * p.batch, groups32 = (long long)((p.N + 31) / 32) * p.batch;
+  if (groups64 >= 192) return groups64 <= 256;
+  if (groups32 > 256) return false;
+  return groups32 >= 192 || p.K <= 4096;
 }
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t stream) {

@@ -111,7 +111,7 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 }
 
 Plan heuristic_plan(const GemmProblem& p) {
-  if (srt::skinny_supported(p)) return kPlanSkinny;
+  if (srt::skinny_supported(p) && srt::skinny_preferred(p)) return kPlanSkinny;
   // few 256 x 256 tiles and a long k loop: K split over the idle compute units
   if (srt::mfma_prefers_splitk(p)) return kPlanSplitK;
   const int c = srt::mfma_select(p);

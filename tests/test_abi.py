@@ -231,6 +231,12 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"
+    # 33..64 rows: the streaming kernel when its workgroups make one round that fills the device
+    assert query(native.REAL16BF, 64, 14336, 4096, tb=True) == "skinny"               # 224 workgroups of 64 weight rows
+    assert query(native.REAL16BF, 64, 4096, 4096, tb=True) == "skinny"                # 128 of 32, short enough k loop
+    assert query(native.REAL16BF, 64, 4096, 14336, tb=True) == "mfma_256x256_splitk"  # few workgroups, long k loop
+    assert query(native.REAL16BF, 64, 11008, 4096, tb=True) == "mfma_256x256_splitk"  # 344 workgroups: not one round
+    assert query(native.REAL16BF, 65, 14336, 4096, tb=True) == "mfma_256x256_splitk"
     assert query(native.REAL16BF, 33, 33, 33) == "generic"
     assert query(native.REAL16BF, 64, 64, 64, align=2) == "generic"      # misaligned view
     assert query(native.REAL32F, 512, 512, 512) in ("generic", "f32_mfma")

@@ -380,6 +380,36 @@ def test_skinny_wide_groups_integer_exact_bias_and_batch(dt):
     assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_skinny_up_to_64_rows_integer_exact_bias_and_choice(dt, tmp_path):
+    """33 <= M <= 64: two output tiles along M per workgroup, with 32 and with 64 weight rows; ragged N and K,
+    bias + ReLU, a batch; and the shapes the heuristic gives to this kernel or keeps from it."""
+    r = H.rng(42)
+    for (M, N, K) in [(33, 1000, 520), (64, 12328, 200), (40, 12344, 72), (57, 4096, 64), (64, 264, 4096)]:
+        x = r.integers(-2, 3, (M, K)).astype(np.float32)
+        w = r.integers(-2, 3, (N, K)).astype(np.float32)
+        b = r.integers(-3, 4, N).astype(np.float32)
+        xt, wt, bt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt)), srt.Tensor(H.encode(b, dt))
+        out = srt.Tensor(shape=[M, N], dtype=xt.dtype)
+        f = tmp_path / "plan.txt"
+        f.write_text(f"{dt} {M} {N} {K} 1 85 10 skinny\n{dt} {M} {N} {K} 1 85 3 skinny\n")
+        srt.PlanCache.clear()
+        srt.PlanCache.load(f)
+        assert query_kernel(xt, False, wt, True, out) == "skinny"
+        srt.current_queue().matmul(xt, False, wt, True, out, bias=bt, activation=srt.ActivationType.relu)
+        exact = np.maximum(x.astype(np.float64) @ w.astype(np.float64).T + b[None, :], 0)
+        assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    srt.PlanCache.clear()
+    B_, M, N, K = 3, 48, 2056, 136
+    x = r.integers(-2, 3, (B_, M, K)).astype(np.float32)
+    w = r.integers(-2, 3, (B_, N, K)).astype(np.float32)
+    xt, wt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt))
+    out = srt.matmul(xt, wt, transposed_rhs=True)
+    assert query_kernel(xt, False, wt, True, out) == "skinny"            # 195 workgroups of 32 rows, short k loop
+    exact = x.astype(np.float64) @ np.swapaxes(w, 1, 2).astype(np.float64)
+    assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
+
+
 # ---- layouts: views, column-major, strided output ------------------------------------------------------
 @pytest.mark.parametrize("dt", DTS)
 def test_strided_views_and_column_major(dt):
