@@ -16,6 +16,13 @@
 //           vector-memory instructions are global->LDS loads and its only register-producing
 //           loads are LDS reads.
 //   grid    ceil(N / 32) x batch workgroups of 60-72 KiB LDS: two per CU, all resident at once.
+//   W[K,N]  An n-contiguous weight (x . W, the Dense layer's own layout) streams the same way with 64
+//           columns per workgroup: a k row of the block is then 128 contiguous bytes, one load
+//           instruction fetches 8 k rows, and a k block of 64 rows lands as [64 k][8 chunks of 16 B],
+//           chunk c of k row k at c ^ (((k >> 1) & 1) << 2).  The MFMA operand (lane l: column l % 32,
+//           k = 8 (l / 32) .. + 7) is two ds_read_b64_tr_b16: within 16 lanes the instruction
+//           transposes a 4 (k) x 16 (n) block; the swizzle puts the four k rows a half wave touches
+//           on different banks.
 //   M > 32  two 32-row output tiles per 32 rows of W (the x fragments of both meet each W fragment)
 //   M > 16  x is as large per k block as the 32 rows of W it meets, and every workgroup re-reads it
 //           from L2: when N is large enough to keep most CUs busy that way, a workgroup takes 64
@@ -31,6 +38,8 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
 #define SRT_LDS __attribute__((address_space(3)))
 
 template <typename T>
@@ -86,8 +95,11 @@ __device__ __forceinline__ void sk_load_to_lds(u32x4_t rsrc, uint32_t lds_addr, 
 // Every vector-memory instruction in the k loop is a global->LDS load issued from inline assembly
 // and awaited with explicit s_waitcnt vmcnt; everything that produces registers is an LDS read,
 // which the compiler tracks on its own counter.
-template <typename T, int XR, int NW>
+// W_MN: the weight is n-contiguous ([K, N]); a workgroup takes 32 NW columns, i.e. RB = 64 NW bytes
+// of every k row.
+template <typename T, int XR, int NW, bool W_MN = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem p) {
+  constexpr int RB = 64 * NW;   // W_MN: bytes of a k row in LDS
   using Shape = SkinnyShape<XR, NW>;
   constexpr int SK_WBYTES = Shape::WBYTES;
   constexpr int MT = Shape::MT;
@@ -106,7 +118,8 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   const uint16_t* W = (const uint16_t*)p.B + (long long)bz * p.sbb;
 
   // both operands through bounds-checked buffers: rows >= N (>= M) and k >= K read zero
-  const uint32_t w_bytes = (uint32_t)(((long long)(p.N - 1) * p.sbn + p.K) * 2);
+  const uint32_t w_bytes = W_MN ? (uint32_t)(((long long)(p.K - 1) * p.sbk + p.N) * 2)
+                                : (uint32_t)(((long long)(p.N - 1) * p.sbn + p.K) * 2);
   const uint64_t wp = reinterpret_cast<uint64_t>(W);
   const u32x4_t rw = {(uint32_t)wp, (uint32_t)(wp >> 32) & 0xffffu, w_bytes, 0x00020000u};
   const uint32_t x_bytes = (uint32_t)(((long long)(p.M - 1) * p.sam + p.K) * 2);
@@ -123,9 +136,20 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 #pragma unroll
   for (int i = 0; i < 4 * NW; ++i) {
     const int row = 8 * i + lrow;
-    wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
-    const int n = n0 + row;
-    wvoff[i] = n < p.N ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * 8) * 2) : SK_OOB;
+    if (W_MN) {
+      // load i covers 1024 / RB k rows of the block; the lane fetches the chunk of 8 columns that
+      // belongs at its landing position.  wchunk holds the k row (for the tail test).
+      const int krow = (1024 / RB) * i + lane / (RB / 16);
+      const int pos = lane % (RB / 16);
+      const int c = NW == 2 ? pos ^ (((krow >> 1) & 1) << 2) : pos;
+      const int n = n0 + 8 * c;
+      wchunk[i] = krow;
+      wvoff[i] = n < p.N ? (uint32_t)(((long long)krow * p.sbk + n) * 2) : SK_OOB;
+    } else {
+      wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
+      const int n = n0 + row;
+      wvoff[i] = n < p.N ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * 8) * 2) : SK_OOB;
+    }
   }
 #pragma unroll
   for (int i = 0; i < XR / 8; ++i) {
@@ -141,6 +165,21 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 #pragma unroll
   for (int s = 0; s < 4; ++s) rd[s] = (uint32_t)(r * 128 + (((2 * s + h) ^ ((r >> 1) & 7)) << 4));
   const bool x_lane = XR >= 32 || r < XR;   // lanes of rows that are not staged hold zero operands
+  // n-contiguous weight: the lane's address for the transposing read of column tile t at k slice 0
+  // (k row 8 h + e, columns 32 t + 16 (g & 1) + 4 q .. + 3); k slice s is 16 k rows further, the
+  // second half of the lane's eight k values four k rows.  With 64-byte rows the four k rows a half
+  // wave reads are 256 contiguous bytes and need no swizzle.
+  uint32_t rdw[2];
+  {
+    const int g = lane >> 4, e = (lane >> 2) & 3, q = lane & 3;
+    const int krow = 8 * (g >> 1) + e;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int mn = 32 * t + 16 * (g & 1) + 4 * q;
+      const int chunk = NW == 2 ? (mn >> 3) ^ (((krow >> 1) & 1) << 2) : (mn >> 3);
+      rdw[t] = (uint32_t)(krow * RB + chunk * 16 + ((mn >> 2) & 1) * 8);
+    }
+  }
 
   const int KB = (p.K + SK_KB - 1) / SK_KB;   // k blocks in total; this wave takes wave, wave + 4, ...
   const int k_chunks = p.K / 8;                // valid 16-byte chunks per row
@@ -149,10 +188,11 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     const bool live = kb < KB;
     const uint32_t base = my_ring + (uint32_t)slot * Shape::SLOT;
     const uint32_t soff = (uint32_t)kb * (SK_KB * 2);
+    const uint32_t soff_w = W_MN ? (uint32_t)kb * (uint32_t)(SK_KB * 2) * (uint32_t)p.sbk : soff;
 #pragma unroll
     for (int i = 0; i < 4 * NW; ++i) {
-      const bool in_k = live && (kb * 8 + wchunk[i]) < k_chunks;
-      sk_load_to_lds<true>(rw, base + (uint32_t)i * 1024u, in_k ? wvoff[i] : SK_OOB, soff);
+      const bool in_k = live && (W_MN ? kb * SK_KB + wchunk[i] < p.K : (kb * 8 + wchunk[i]) < k_chunks);
+      sk_load_to_lds<true>(rw, base + (uint32_t)i * 1024u, in_k ? wvoff[i] : SK_OOB, soff_w);
     }
 #pragma unroll
     for (int i = 0; i < XR / 8; ++i) {
@@ -174,7 +214,9 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   // one time are spread over different byte offsets of their rows -- with rows a power of two
   // apart, all workgroups reading the same offset would hammer the same few memory channels.
   const int count = KB > wave ? (KB - wave + SK_WAVES - 1) / SK_WAVES : 0;
-  const int rot = count > 0 ? (int)((blockIdx.x * 7u) % (unsigned)count) : 0;
+  // (An n-contiguous weight is walked in step instead: neighbouring workgroups then read neighbouring
+  // 128-byte pieces of the same k rows at about the same time.)
+  const int rot = (!W_MN && count > 0) ? (int)((blockIdx.x * 7u) % (unsigned)count) : 0;
   auto block_at = [&](int j) {   // j-th block of the walk, or KB (= nothing) past the end
     if (j >= count) return KB;
     int jj = j + rot;
@@ -198,7 +240,18 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
 #pragma unroll
-        for (int t = 0; t < NW; ++t) wf[t][s] = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + t * SK_WTILE + rd[s]);
+        for (int t = 0; t < NW; ++t) {
+          if (W_MN) {
+            const uint32_t a = base + rdw[t & 1] + s * (16 * RB);
+            const u32x2_t lo = __builtin_bit_cast(
+                u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a)));
+            const u32x2_t hi = __builtin_bit_cast(
+                u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a + 4 * RB)));
+            wf[t][s] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+          } else {
+            wf[t][s] = *reinterpret_cast<const SRT_LDS u32x4_t*>(base + t * SK_WTILE + rd[s]);
+          }
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           u32x4_t x = {0u, 0u, 0u, 0u};
@@ -255,9 +308,9 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   }
 }
 
-template <typename T, int XR, int NW>
+template <typename T, int XR, int NW, bool W_MN = false>
 hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
-  auto kernel = gemm_skinny_kernel<T, XR, NW>;
+  auto kernel = gemm_skinny_kernel<T, XR, NW, W_MN>;
   constexpr int lds_bytes = SkinnyShape<XR, NW>::LDS;
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
@@ -267,6 +320,15 @@ hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
 
 template <typename T>
 hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
+  if (p.sbk != 1) {   // n-contiguous weight
+    // Always 64 columns per workgroup, i.e. whole 128-byte lines of a k row.  (With 32 columns the
+    // two workgroups that share a line each pull it from memory: 11008 columns x 4096 took 39 us
+    // instead of 22 us, 8192 x 8192 47 us instead of 40 us.)
+    if (p.M <= 8) return launch_skinny_shape<T, 8, 2, true>(p, stream);
+    if (p.M <= 16) return launch_skinny_shape<T, 16, 2, true>(p, stream);
+    if (p.M <= 32) return launch_skinny_shape<T, 32, 2, true>(p, stream);
+    return launch_skinny_shape<T, 64, 2, true>(p, stream);
+  }
   if (p.M <= 8) return launch_skinny_shape<T, 8, 1>(p, stream);
   if (p.M <= 16) return launch_skinny_shape<T, 16, 1>(p, stream);
   // two W tiles per workgroup once that still gives most CUs a workgroup (192 of them)
@@ -286,16 +348,23 @@ inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 bool skinny_supported(const GemmProblem& p) {
   if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return false;
   if (p.M > 64 || p.M < 1 || p.K < 1) return false;
-  if (p.sak != 1 || p.sbk != 1) return false;           // both operands k-contiguous
+  if (p.sak != 1) return false;                         // x is k-contiguous
   if ((p.K % 8) != 0) return false;                     // whole 16-byte chunks
   if ((p.sam % 8) != 0 && p.M > 1) return false;
-  if ((p.sbn % 8) != 0 && p.N > 1) return false;
   if ((p.sab % 8) != 0 || (p.sbb % 8) != 0) return false;
-  if (p.sam < 0 || p.sbn < 0 || p.scm < 0 || p.scn < 0) return false;
+  if (p.sam < 0 || p.scm < 0 || p.scn < 0) return false;
   if (!aligned16(p.A) || !aligned16(p.B)) return false;
   if (p.batch > 65535) return false;
-  // 32-bit byte offsets must reach every row of W (and stay below the out-of-range marker)
-  if (((long long)p.N + 32) * p.sbn + p.K >= (0x7fffffffLL / 2 - 4096)) return false;
+  if (p.sbk == 1) {                                     // W k-contiguous ([N, K])
+    if ((p.sbn % 8) != 0 && p.N > 1) return false;
+    if (p.sbn < 0) return false;
+    // 32-bit byte offsets must reach every row of W (and stay below the out-of-range marker)
+    if (((long long)p.N + 32) * p.sbn + p.K >= (0x7fffffffLL / 2 - 4096)) return false;
+  } else {                                              // W n-contiguous ([K, N])
+    if (p.sbn != 1 || (p.N % 8) != 0) return false;     // whole 16-byte chunks of a k row
+    if (p.sbk < 8 || (p.sbk % 8) != 0) return false;
+    if (((long long)p.K + 64) * p.sbk + p.N >= (0x7fffffffLL / 2 - 4096)) return false;
+  }
   // worth it only when the weight dominates the traffic
   return p.N >= 32;
 }
@@ -307,7 +376,20 @@ bool skinny_supported(const GemmProblem& p) {
 // 256 of 32 rows unless they are few and the k loop is long (64 x 4096 x 4096, 128 workgroups: 17 us
 // against 21 us; 64 x 4096 x 14336: 51 us against 35 us; 64 x 11008 x 4096, 344 workgroups: 34 us
 // against 29 us; 64 x 32768 x 1024: 22 us against 17 us for 64 x 64 tiles).
+//
+// An n-contiguous weight streams at 4.3-4.8 TB/s at best (x . W with 14336 x 4096: 25-28 us for up
+// to 32 rows, where split-K takes 29 us and the k-contiguous form of this kernel 21 us), always with
+// 64 columns per workgroup, so it needs its workgroups to number at most one round, and a short k
+// loop when they are few; 8192-deep problems go to split-K (8 x 4096 x 8192: 25 us against 37 us)
+// and more than 256 workgroups to the 128 x 256 tiles (8 x 28672 x 1024: 16 us against 19 us).
 bool skinny_preferred(const GemmProblem& p) {
+  if (p.sbk != 1) {
+    const long long groups = (long long)((p.N + 63) / 64) * p.batch;
+    if (groups > 256) return false;
+    if (p.K <= 2048) return true;
+    if (p.K <= 4096) return p.M <= 16 || (p.M <= 32 ? (groups >= 192 || groups <= 32) : groups >= 208);
+    return p.M <= 16 && groups <= 32;
+  }
   if (p.M <= 32) return true;
   const long long groups64 = (long long)((p.N + 63) / 64) * p.batch, groups32 = (long long)((p.N + 31) / 32) * p.batch;
   if (groups64 >= 192) return groups64 <= 256;

@@ -237,6 +237,14 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 64, 4096, 14336, tb=True) == "mfma_256x256_splitk"  # few workgroups, long k loop
     assert query(native.REAL16BF, 64, 11008, 4096, tb=True) == "mfma_256x256_splitk"  # 344 workgroups: not one round
     assert query(native.REAL16BF, 65, 14336, 4096, tb=True) == "mfma_256x256_splitk"
+    # x . W with an n-contiguous W: the streaming kernel within one round of 64-column workgroups and a short k loop
+    assert query(native.REAL16BF, 8, 14336, 4096) == "skinny"
+    assert query(native.REAL16BF, 32, 4096, 2048) == "skinny"
+    assert query(native.REAL16BF, 32, 4096, 4096) == "mfma_256x256_splitk"            # 64 workgroups, 17..32 rows
+    assert query(native.REAL16BF, 8, 4096, 8192) == "mfma_256x256_splitk"             # long k loop
+    assert query(native.REAL16BF, 8, 28672, 1024) == "mfma_128x256_m16"               # 448 workgroups: not one round
+    assert query(native.REAL16BF, 64, 14336, 4096) == "skinny"
+    assert query(native.REAL16BF, 64, 11008, 4096) == "mfma_256x256_splitk"
     assert query(native.REAL16BF, 33, 33, 33) == "generic"
     assert query(native.REAL16BF, 64, 64, 64, align=2) == "generic"      # misaligned view
     assert query(native.REAL32F, 512, 512, 512) in ("generic", "f32_mfma")

@@ -410,6 +410,50 @@ def test_skinny_up_to_64_rows_integer_exact_bias_and_choice(dt, tmp_path):
     assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_skinny_n_contiguous_weight_integer_exact_bias_and_batch(dt, tmp_path):
+    """x[M, K] . W[K, N] (no transposes) with up to 64 rows of x: the streaming kernel reads W through the
+    transposing LDS read.  Every staged row count, N ending inside a 64-column group, K ending inside a k block,
+    bias + ReLU, a batch, and random data against fp64."""
+    r = H.rng(43)
+    relu = srt.ActivationType.relu
+    for (M, N, K) in [(1, 64, 8), (5, 104, 72), (8, 1000, 520), (16, 4096, 64), (17, 12328, 200), (32, 264, 4096),
+                      (33, 1000, 520), (64, 12344, 72), (57, 4096, 192)]:
+        x = r.integers(-2, 3, (M, K)).astype(np.float32)
+        w = r.integers(-2, 3, (K, N)).astype(np.float32)
+        b = r.integers(-3, 4, N).astype(np.float32)
+        xt, wt, bt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt)), srt.Tensor(H.encode(b, dt))
+        out = srt.Tensor(shape=[M, N], dtype=xt.dtype)
+        pin_plan(tmp_path, "skinny", dt, M, N, K, False, False)
+        assert query_kernel(xt, False, wt, False, out) == "skinny"
+        srt.current_queue().matmul(xt, False, wt, False, out)
+        exact = x.astype(np.float64) @ w.astype(np.float64)
+        assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+        pin_plan(tmp_path, "skinny", dt, M, N, K, False, False, bias=True, act=relu)
+        srt.current_queue().matmul(xt, False, wt, False, out, bias=bt, activation=relu)
+        exact = np.maximum(exact + b[None, :], 0)
+        assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    B_, M, N, K = 3, 24, 2056, 136
+    x = r.integers(-2, 3, (B_, M, K)).astype(np.float32)
+    w = r.integers(-2, 3, (B_, K, N)).astype(np.float32)
+    f = tmp_path / "plan.txt"
+    f.write_text(f"{dt} {M} {N} {K} {B_} 89 0 skinny\n")
+    srt.PlanCache.clear()
+    srt.PlanCache.load(f)
+    xt, wt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt))
+    out = srt.matmul(xt, wt)
+    assert query_kernel(xt, False, wt, False, out) == "skinny"
+    exact = x.astype(np.float64) @ w.astype(np.float64)
+    assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
+    M, N, K = 48, 2048, 4096
+    pin_plan(tmp_path, "skinny", dt, M, N, K, False, False)
+    a = (r.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+    w = r.standard_normal((K, N)).astype(np.float32)
+    a_st, w_st = H.encode(a, dt), H.encode(w, dt)
+    check_against_fp64(gpu_matmul(a_st, w_st, want_kernel="skinny"), a_st, w_st, False, False, dt)
+    srt.PlanCache.clear()
+
+
 # ---- layouts: views, column-major, strided output ------------------------------------------------------
 @pytest.mark.parametrize("dt", DTS)
 def test_strided_views_and_column_major(dt):
