@@ -20,7 +20,13 @@
 //       k, written to LDS as they are;
 //   operand stored mn-contiguous (A transposed / B not transposed): each thread loads an
 //       8(k) x 8(mn) block as eight 16-byte rows (coalesced along mn), transposes it in
-//       registers with 32 v_perm_b32 and writes eight k-contiguous chunks.
+//       registers with 32 v_perm_b32 and writes eight k-contiguous chunks;
+//   operand with a unit stride that misses the alignment rules (odd extents or leading strides,
+//       a base that is not 16-byte aligned): the same two loaders with 16-byte loads at 2-byte
+//       alignment (global memory takes them), and element loads for the one chunk per row that
+//       would cross the end of the contiguous dimension;
+//   operand with non-unit strides in both dimensions: 2-byte loads with arbitrary element strides,
+//       eight k-values of a row packed into one chunk in registers.
 #include "gemm_common.h"
 
 namespace srt {
@@ -94,21 +100,51 @@ __device__ __forceinline__ uint32_t lds_off(int row, int chunk) {
 }
 
 // ---- global -> register staging --------------------------------------------------------------
+// Up to 7 elements src[0], src[stride], ... (count of them, 1..7) as the leading halves of a
+// 16-byte chunk, zero behind them: the end of a contiguous dimension that is not a multiple of 8.
+__device__ __forceinline__ u32x4_t load_chunk_tail(const uint16_t* src, int count) {
+  uint32_t h[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) h[j] = (uint32_t)src[min(j, count - 1)] & (uint32_t)((j - count) >> 31);
+  return u32x4_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+}
+
+// 16 bytes from an address with 2-byte alignment: still one global_load_dwordx4 (global memory
+// takes it at any alignment).  Rows that are off by 2 bytes load at well under half the aligned
+// rate (4096 x 4097 x 4096 with such rows of B: 186 TFLOP/s; with rows that merely miss the 16-byte
+// rule: 450-560); fetching aligned dwords plus a fifth and funnel-shifting them into place was
+// tried and is slower still (155 and 360-430).
+__device__ __forceinline__ u32x4_t load_chunk_unaligned(const uint16_t* src) {
+  u32x4_t x;
+  __builtin_memcpy(&x, src, 16);
+  return x;
+}
+
 // K-contiguous operand: R rows x 64 k.  Thread t owns chunk t % 8 of rows t / 8 + 32 i.
-template <int R>
+// ALIGNED: rows start on 16-byte boundaries and K is a multiple of 8.
+template <int R, bool ALIGNED = true>
 struct StageK {
   static constexpr int CH = R * 8 / NT;
   u32x4_t v[CH];
 
-  __device__ __forceinline__ void load(const uint16_t* base, long long ld, int row0, int rows_total, int k0, int K,
-                                       int tid) {
+  __device__ __forceinline__ void load(const uint16_t* base, long long ld, long long, int row0, int rows_total, int k0,
+                                       int K, int tid) {
     const int chunk = tid & 7;
     const int k = k0 + chunk * 8;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int row = row0 + (tid >> 3) + 32 * i;
       u32x4_t x = {0u, 0u, 0u, 0u};
-      if (row < rows_total && k < K) x = *reinterpret_cast<const u32x4_t*>(base + (long long)row * ld + k);
+      if (row < rows_total && k < K) {
+        const uint16_t* src = base + (long long)row * ld + k;
+        if (ALIGNED) {
+          x = *reinterpret_cast<const u32x4_t*>(src);
+        } else if (k + 8 <= K) {
+          x = load_chunk_unaligned(src);
+        } else {
+          x = load_chunk_tail(src, K - k);
+        }
+      }
       v[i] = x;
     }
   }
@@ -125,20 +161,29 @@ struct StageK {
 
 // MN-contiguous operand: 64 k x R mn, element (k, mn) at base[k * ld + mn].  Thread t (< R)
 // owns the 8 x 8 block k-group t / (R/8), mn-group t % (R/8).
-template <int R>
+template <int R, bool ALIGNED = true>
 struct StageMN {
   static constexpr int GROUPS = R / 8;
   u32x4_t v[8];
 
-  __device__ __forceinline__ void load(const uint16_t* base, long long ld, int mn0, int mn_total, int k0, int K,
-                                       int tid) {
+  __device__ __forceinline__ void load(const uint16_t* base, long long, long long ld, int mn0, int mn_total, int k0,
+                                       int K, int tid) {
     if (R < NT && tid >= R) return;
     const int mn = mn0 + (tid % GROUPS) * 8;
     const int kb = k0 + (tid / GROUPS) * 8;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       u32x4_t x = {0u, 0u, 0u, 0u};
-      if (mn < mn_total && kb + j < K) x = *reinterpret_cast<const u32x4_t*>(base + (long long)(kb + j) * ld + mn);
+      if (mn < mn_total && kb + j < K) {
+        const uint16_t* src = base + (long long)(kb + j) * ld + mn;
+        if (ALIGNED) {
+          x = *reinterpret_cast<const u32x4_t*>(src);
+        } else if (mn + 8 <= mn_total) {
+          x = load_chunk_unaligned(src);
+        } else {
+          x = load_chunk_tail(src, mn_total - mn);
+        }
+      }
       v[j] = x;
     }
   }
@@ -167,12 +212,63 @@ struct StageMN {
   }
 };
 
-template <int R, bool KCONTIG>
+// Any strides: element (mn, k) at base[mn * s_mn + k * s_k], 2-byte loads.  A thread fills whole
+// chunks (8 k of one row): thread t owns row t % R and chunks t / R + (256 / R) i, so a wave's
+// loads walk 64 consecutive rows at one k.
+template <int R>
+struct StageAny {
+  static constexpr int CH = R * 8 / NT;
+  u32x4_t v[CH];
+
+  __device__ __forceinline__ void load(const uint16_t* base, long long s_mn, long long s_k, int mn0, int mn_total,
+                                       int k0, int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int row = tid % R;
+      const int chunk = tid / R + (NT / R) * i;
+      const int mn = mn0 + row, k = k0 + chunk * 8;
+      // every load is issued, from an address clamped into the operand, and masked afterwards: no
+      // branches, so the loads of a stage go out back to back and are awaited once (the mask is
+      // arithmetic -- the sign of index - extent -- so that no select invites the compiler to put
+      // the load back under a condition)
+      const uint16_t* src = base + (long long)min(mn, mn_total - 1) * s_mn;
+      const uint32_t row_mask = (uint32_t)((mn - mn_total) >> 31);
+      uint32_t h[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int kc = min(k + j, K - 1);
+        const uint32_t x = src[(long long)kc * s_k];
+        h[j] = x & row_mask & (uint32_t)((k + j - K) >> 31);
+      }
+      v[i] = u32x4_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned char* lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int row = tid % R;
+      const int chunk = tid / R + (NT / R) * i;
+      *reinterpret_cast<u32x4_t*>(lds + lds_off(row, chunk)) = v[i];
+    }
+  }
+};
+
+// staging modes of an operand: contiguous along mn / along k and aligned; the same two without
+// the alignment; any strides
+constexpr int MODE_MN = 0, MODE_K = 1, MODE_UMN = 2, MODE_UK = 3, MODE_ANY = 4;
+template <int R, int MODE>
 struct Stage;
 template <int R>
-struct Stage<R, true> : StageK<R> {};
+struct Stage<R, MODE_K> : StageK<R, true> {};
 template <int R>
-struct Stage<R, false> : StageMN<R> {};
+struct Stage<R, MODE_MN> : StageMN<R, true> {};
+template <int R>
+struct Stage<R, MODE_UK> : StageK<R, false> {};
+template <int R>
+struct Stage<R, MODE_UMN> : StageMN<R, false> {};
+template <int R>
+struct Stage<R, MODE_ANY> : StageAny<R> {};
 
 // XCD-aware remap of the linear workgroup id followed by a grouped tile order.
 // Workgroups are handed to the 8 XCDs round-robin, so ids congruent mod 8 share an L2.  The
@@ -199,7 +295,7 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
   *tn = in_group / gsize;
 }
 
-template <typename T, int BM, int BN, bool A_KC, bool B_KC>
+template <typename T, int BM, int BN, int A_MODE, int B_MODE>
 __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
   constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -220,8 +316,6 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
 
   const uint16_t* A = (const uint16_t*)p.A + (long long)bz * p.sab;
   const uint16_t* B = (const uint16_t*)p.B + (long long)bz * p.sbb;
-  const long long lda = A_KC ? p.sam : p.sak;  // stride of the non-contiguous dimension
-  const long long ldb = B_KC ? p.sbn : p.sbk;
 
   f32x16_t acc[TM][TN];
 #pragma unroll
@@ -231,12 +325,12 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  Stage<BM, A_KC> sa;
-  Stage<BN, B_KC> sb;
+  Stage<BM, A_MODE> sa;
+  Stage<BN, B_MODE> sb;
   const int KT = (p.K + BK - 1) / BK;
 
-  sa.load(A, lda, m0, p.M, 0, p.K, tid);
-  sb.load(B, ldb, n0, p.N, 0, p.K, tid);
+  sa.load(A, p.sam, p.sak, m0, p.M, 0, p.K, tid);
+  sb.load(B, p.sbn, p.sbk, n0, p.N, 0, p.K, tid);
   sa.store(lds, tid);
   sb.store(lds + A_BYTES, tid);
   __syncthreads();
@@ -249,8 +343,8 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
     unsigned char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
     const bool more = kt + 1 < KT;
     if (more) {
-      sa.load(A, lda, m0, p.M, (kt + 1) * BK, p.K, tid);
-      sb.load(B, ldb, n0, p.N, (kt + 1) * BK, p.K, tid);
+      sa.load(A, p.sam, p.sak, m0, p.M, (kt + 1) * BK, p.K, tid);
+      sb.load(B, p.sbn, p.sbk, n0, p.N, (kt + 1) * BK, p.K, tid);
     }
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
@@ -279,7 +373,7 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
   // keep it aligned and the group lies inside N, element stores otherwise.
   Epilogue<T> ep(p);
   uint16_t* C = (uint16_t*)p.C + (long long)bz * p.scb;
-  const bool wide = (p.scm % 4) == 0 && (reinterpret_cast<uintptr_t>(C) & 7u) == 0;
+  const bool wide = p.scn == 1 && (p.scm % 4) == 0 && (reinterpret_cast<uintptr_t>(C) & 7u) == 0;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = m0 + wm0 + 32 * i + (lane & 31);
@@ -306,7 +400,7 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (n + e < p.N) crow[n + e] = h[e];
+            if (n + e < p.N) crow[(long long)(n + e) * p.scn] = h[e];
         }
       }
     }
@@ -314,10 +408,10 @@ __global__ __launch_bounds__(NT) void gemm_mfma_kernel(GemmProblem p) {
 }
 
 // config ids: tile << 2 | a_kc << 1 | b_kc ; tile 1: 256x256, 2: 128x128, 3: 64x64
-template <typename T, int BM, int BN, bool A_KC, bool B_KC>
+template <typename T, int BM, int BN, int A_MODE, int B_MODE>
 hipError_t launch_one(const GemmProblem& p, hipStream_t stream) {
   constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROW_BYTES;
-  auto kernel = gemm_mfma_kernel<T, BM, BN, A_KC, B_KC>;
+  auto kernel = gemm_mfma_kernel<T, BM, BN, A_MODE, B_MODE>;
   if (lds_bytes > 64 * 1024) {
     static std::atomic<uint32_t> configured{0};
     if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), (int)lds_bytes, configured); e != hipSuccess)
@@ -330,10 +424,25 @@ hipError_t launch_one(const GemmProblem& p, hipStream_t stream) {
 
 template <typename T, int BM, int BN>
 hipError_t launch_layout(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
-  if (a_kc && b_kc) return launch_one<T, BM, BN, true, true>(p, stream);
-  if (a_kc && !b_kc) return launch_one<T, BM, BN, true, false>(p, stream);
-  if (!a_kc && b_kc) return launch_one<T, BM, BN, false, true>(p, stream);
-  return launch_one<T, BM, BN, false, false>(p, stream);
+  if (a_kc && b_kc) return launch_one<T, BM, BN, MODE_K, MODE_K>(p, stream);
+  if (a_kc && !b_kc) return launch_one<T, BM, BN, MODE_K, MODE_MN>(p, stream);
+  if (!a_kc && b_kc) return launch_one<T, BM, BN, MODE_MN, MODE_K>(p, stream);
+  return launch_one<T, BM, BN, MODE_MN, MODE_MN>(p, stream);
+}
+
+// operands without the alignment guarantees: per operand, the unaligned form of the loader for
+// its unit stride, or element-wise staging when it has none
+template <typename T, int BM, int BN, int A_MODE>
+hipError_t launch_any_b(const GemmProblem& p, hipStream_t stream) {
+  if (p.sbk == 1) return launch_one<T, BM, BN, A_MODE, MODE_UK>(p, stream);
+  if (p.sbn == 1) return launch_one<T, BM, BN, A_MODE, MODE_UMN>(p, stream);
+  return launch_one<T, BM, BN, A_MODE, MODE_ANY>(p, stream);
+}
+template <typename T, int BM, int BN>
+hipError_t launch_any_layout(const GemmProblem& p, hipStream_t stream) {
+  if (p.sak == 1) return launch_any_b<T, BM, BN, MODE_UK>(p, stream);
+  if (p.sam == 1) return launch_any_b<T, BM, BN, MODE_UMN>(p, stream);
+  return launch_any_b<T, BM, BN, MODE_ANY>(p, stream);
 }
 
 template <typename T>
@@ -378,7 +487,7 @@ hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
 }
 
 // tile 1 (256 x 256) is the ring kernel, tile 5 the same ring on 16x16x32 MFMAs, tile 6 its 128 x 256
-// form; tiles 2 and 3 are the register-staged kernels above
+// form; tiles 2 and 3 are the register-staged kernels above, 7 and 8 the same without alignment rules
 template <typename T>
 hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hipStream_t stream) {
   switch (tile) {
@@ -387,6 +496,8 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 5: return launch_m16<T>(p, a_kc, b_kc, stream);
     case 6: return launch_m16h<T>(p, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
+    case 7: return launch_any_layout<T, 128, 128>(p, stream);
+    case 8: return launch_any_layout<T, 64, 64>(p, stream);
     default: return launch_layout<T, 64, 64>(p, a_kc, b_kc, stream);
   }
 }
@@ -423,6 +534,11 @@ static int mfma_layout(const GemmProblem& p) {
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
 // 128 x 256 form for a k-contiguous A), or 0 when the problem does not qualify for it.
 int mfma_config(const GemmProblem& p, int tile) {
+  if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
+    if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
+    if (p.K < 1 || p.batch > 65535) return 0;
+    return tile << 2;
+  }
   const int layout = mfma_layout(p);
   if (layout < 0 || tile < 1 || tile > 6) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
@@ -433,8 +549,9 @@ int mfma_config(const GemmProblem& p, int tile) {
 
 int mfma_select(const GemmProblem& p) {
   const int layout = mfma_layout(p);
-  if (layout < 0) return 0;
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
+  // operands that miss the alignment rules: unaligned or element-wise staging, 128 x 128 tiles once they fill the device
+  if (layout < 0) return mfma_config(p, tiles(128) >= 256 ? 7 : 8);
   // Tile choice, from measurements over mid-size problems (1024^3 .. 4096 x 14336 x 4096):
   //  * the 256 x 256 kernels are so much more efficient per tile (deep prefetch, 4x the arithmetic
   //    intensity) that they win long before they can fill the device: from 24 tiles up (48 when K < 1024) for the
@@ -624,6 +741,8 @@ const char* mfma_name(int config) {
     case 5: return "mfma_256x256_m16";
     case 6: return "mfma_128x256_m16";
     case 2: return "mfma_128x128";
+    case 7: return "mfma_128x128_any";
+    case 8: return "mfma_64x64_any";
     default: return "mfma_64x64";
   }
 }

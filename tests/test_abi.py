@@ -245,8 +245,10 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 8, 28672, 1024) == "mfma_128x256_m16"               # 448 workgroups: not one round
     assert query(native.REAL16BF, 64, 14336, 4096) == "skinny"
     assert query(native.REAL16BF, 64, 11008, 4096) == "mfma_256x256_splitk"
-    assert query(native.REAL16BF, 33, 33, 33) == "generic"
-    assert query(native.REAL16BF, 64, 64, 64, align=2) == "generic"      # misaligned view
+    # 16-bit operands that miss the 16-byte rules: the matrix-core kernel with element-wise staging
+    assert query(native.REAL16BF, 33, 33, 33) == "mfma_64x64_any"
+    assert query(native.REAL16BF, 64, 64, 64, align=2) == "mfma_64x64_any"            # misaligned view
+    assert query(native.REAL16F, 2048, 50257, 768) == "mfma_128x128_any"              # odd row pitch of B and C
     assert query(native.REAL32F, 512, 512, 512) in ("generic", "f32_mfma")
 
 

@@ -475,6 +475,45 @@ def test_strided_views_and_column_major(dt):
     assert np.array_equal(H.decode(srt.matmul(ta.t, tb.t, transposed_lhs=True, transposed_rhs=True).array()), H.decode(want))
 
 
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+def test_unaligned_operands_run_on_the_matrix_cores(dt):
+    """Operands the 16-byte loaders cannot take -- odd extents and row pitches, views with both strides non-unit
+    or an odd start, a strided result -- go through element-wise staging into the same MFMA tiles: bit-exact on
+    integers for every transpose combination, both tile sizes, bias + ReLU, a batch; fp64 bound on random data."""
+    r = H.rng(130)
+    relu = srt.ActivationType.relu
+    for (M, N, K, ta, tb) in [(33, 33, 33, False, False), (129, 67, 100, True, False), (70, 131, 65, False, True),
+                              (65, 65, 129, True, True), (2049, 2051, 77, False, False), (2050, 2049, 70, True, True)]:
+        a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+        bias = r.integers(-3, 4, N).astype(np.float32)
+        at, bt, biast = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(b, dt)), srt.Tensor(H.encode(bias, dt))
+        out = srt.Tensor(shape=[M, N], dtype=at.dtype)
+        assert query_kernel(at, ta, bt, tb, out) == ("mfma_128x128_any" if M > 2000 else "mfma_64x64_any")
+        srt.current_queue().matmul(at, ta, bt, tb, out, bias=biast, activation=relu)
+        exact = np.maximum((a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64) + bias[None, :], 0)
+        assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K, ta, tb)
+    # views: both strides non-unit, odd starts; then a batch of odd-pitch matrices
+    big_a = r.integers(-3, 4, (300, 200)).astype(np.float32)
+    big_b = r.integers(-3, 4, (200, 400)).astype(np.float32)
+    ta_, tb_ = srt.Tensor(H.encode(big_a, dt)), srt.Tensor(H.encode(big_b, dt))
+    va, vb = ta_[1:291:2, 3:198:3], tb_[5:70, 1:391:3]
+    got = srt.matmul(va, vb)
+    assert query_kernel(va, False, vb, False, got) == "mfma_64x64_any"
+    exact = big_a[1:291:2, 3:198:3].astype(np.float64) @ big_b[5:70, 1:391:3].astype(np.float64)
+    assert np.array_equal(got.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
+    x = r.integers(-3, 4, (3, 70, 45)).astype(np.float32)
+    w = r.integers(-3, 4, (3, 45, 99)).astype(np.float32)
+    got = srt.matmul(srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt)))
+    assert np.array_equal(got.array().view(np.uint16), H.encode((x.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), dt).view(np.uint16))
+    # random data against fp64
+    M, N, K = 515, 1001, 777
+    a = (r.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+    b = r.standard_normal((K, N)).astype(np.float32)
+    a_st, b_st = H.encode(a, dt), H.encode(b, dt)
+    check_against_fp64(gpu_matmul(a_st, b_st, want_kernel="mfma_64x64_any"), a_st, b_st, False, False, dt)
+
+
 def test_column_major_bias_broadcast_direction():
     r = H.rng(14)
     x = r.integers(-3, 4, (24, 16)).astype(np.float32)

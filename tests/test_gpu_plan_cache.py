@@ -13,7 +13,7 @@ from tests.test_gpu_matmul import query_kernel
 
 pytestmark = pytest.mark.gpu
 
-PLANS_16 = {"mfma_256x256", "mfma_256x256_k64", "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "skinny", "generic"}
+PLANS_16 = {"mfma_256x256", "mfma_256x256_k64", "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any", "skinny", "generic"}
 PLANS_32 = {"f32_mfma_64x64", "f32_mfma_splitk", "generic"}
 
 
@@ -67,7 +67,7 @@ def test_every_plan_is_the_same_function(tmp_path):
     br = H.encode(g.standard_normal((k, n)).astype(np.float32), H.BF16)
     want = H.to64(H.encode((H.to64(a_st) @ H.to64(b_st)).astype(np.float32), H.BF16))
     results = {}
-    for plan in ("mfma_256x256", "mfma_128x128", "mfma_64x64", "generic"):
+    for plan in ("mfma_256x256", "mfma_128x128", "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any", "generic"):
         f = tmp_path / f"{plan}.txt"
         f.write_text(f"14 {m} {n} {k} 1 89 10 {plan}\n")
         srt.PlanCache.clear()
@@ -84,7 +84,7 @@ def test_every_plan_is_the_same_function(tmp_path):
 
 
 ALL_PLANS_16 = ("mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64", "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128",
-                "mfma_64x64", "skinny", "generic")
+                "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any", "skinny", "generic")
 
 
 @pytest.mark.parametrize("seed", range(6))
@@ -134,8 +134,8 @@ def test_random_shapes_every_qualifying_plan_bit_exact(seed, tmp_path):
 
 def test_cached_plan_is_skipped_when_this_call_does_not_qualify(tmp_path):
     """Alignment is not part of the key: a view that starts off a 16-byte boundary with the same
-    shape and layout class falls back to the heuristic (the generic kernel) instead of the cached
-    matrix-core plan."""
+    shape and layout class falls back to the heuristic (the kernel with element-wise staging) instead
+    of the cached plan, whose 16-byte loads it does not qualify for."""
     m = k = n = 256
     f = tmp_path / "p.txt"
     f.write_text(f"14 {m} {n} {k} 1 89 10 mfma_64x64\n")
@@ -145,6 +145,7 @@ def test_cached_plan_is_skipped_when_this_call_does_not_qualify(tmp_path):
     b_st = H.encode(g.integers(-3, 4, (k, n)).astype(np.float32), H.BF16)
     a_view = srt.Tensor(big)[:, 1:k + 1]                 # row pitch 264 (16-byte multiple), start misaligned by 2 bytes
     c = srt.matmul(a_view, srt.Tensor(b_st))
+    assert query_kernel(a_view, False, srt.Tensor(b_st), False, c) == "mfma_64x64_any"
     exact = H.to64(big[:, 1:k + 1]) @ H.to64(b_st)
     assert np.array_equal(H.to64(c.array()), H.to64(H.encode(exact.astype(np.float32), H.BF16)))
 
