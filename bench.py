@@ -31,7 +31,7 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFM
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # and scaled by a 256 MiB device copy (profiles/gemm_m16_bf16_8192_counters.txt).
-TRAFFIC_BYTES_8192 = 1.823e9   # 2.000 x FETCH_SIZE (824 491 KiB) + 1.000 x WRITE_SIZE (131 132 KiB)
+TRAFFIC_BYTES_8192 = 1.799e9   # 2.000 x FETCH_SIZE (812 824 KiB) + 1.000 x WRITE_SIZE (131 117 KiB)
 
 
 def rng(seed):
