@@ -387,7 +387,7 @@ bool skinny_preferred(const GemmProblem& p) {
     const long long groups = (long long)((p.N + 63) / 64) * p.batch;
     if (groups > 256) return false;
     if (p.K <= 2048) return true;
-    if (p.K <= 4096) return p.M <= 16 || (p.M <= 32 ? (groups >= 192 || groups <= 32) : groups >= 208);
+    if (p.K <= 4096) return p.M <= 16 || groups <= 32 || groups >= (p.M <= 32 ? 192 : 224);
     return p.M <= 16 && groups <= 32;
   }
   if (p.M <= 32) return true;
