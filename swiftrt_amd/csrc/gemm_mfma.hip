@@ -590,13 +590,30 @@ int mfma_select(const GemmProblem& p) {
   const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
   const long long cus = 256;
   const long long rounds256 = (t256 + cus - 1) / cus, rounds_h = (th + cus - 1) / cus;
+  //  * a problem of a handful of tiles is bound by the latency of its k stages, and the ring's
+  //    deep prefetch beats the 64 x 64 kernel's load-wait-compute stages even on one or two
+  //    workgroups (192 x 128 x 128: 6.5 us against 8.0 us; 96 x 128 x 768: 12.5 against 14.7);
+  //    the same holds for short k loops on many tiles, where the 64 x 64 kernel's 8-byte stores
+  //    of the result also count (512 x 16384 x 128: 9.0 us against 18.3 us; 3072 x 11008 x 64
+  //    with A m-contiguous, whole tiles: 27 us against 71 us);
+  //  * a whole 256 x 256 tile is half padding or more with up to 128 rows or columns: there the
+  //    64 x 64 kernel wins (48 x 16384 x 768 with A m-contiguous: 15.9 us against 20.5 us;
+  //    128 x 14336 x 128: 8.0 against 10.2);
+  //  * on a device at least half full the 16x16x32 ring is ahead of the 32x32x16 one for short
+  //    k loops too (3072 x 8192 x 1024 with A m-contiguous: 56 us against 65 us; 3072 x 16384 x 512:
+  //    60 against 67; 4096 x 4096 x 1024: 34.6 against 36.2) -- except with two k-contiguous
+  //    operands, where the 64-deep kernel keeps short k loops (8192 x 8192 x 1024: 138 us against 146).
+  // (half tiles: with 64 columns or fewer only for longer k loops -- 1536 x 64 x 128: 10.4 us against
+  // 6.7 us for 64 x 64 tiles, 1536 x 64 x 768: 12.8 against 15.1 -- and whatever the rounds when the k
+  // loop is so short that the stores dominate: 6144 x 16384 x 256 80 us against 90 us for whole tiles)
+  const bool half_ok = p.K >= 64 && (p.N > 64 || p.K >= 512) &&
+                       (layout == 3 ? (th >= 96 && rounds_h == 1) : (p.K <= 256 || 6 * rounds_h <= 10 * rounds256));
+  const bool whole_ok = big_ok && p.M > 128 && p.N > 128;
   int tile;
-  if (big_ok && (layout & 2) != 0 && p.K >= 512 && th >= (layout == 3 ? 96 : 8) &&
-      (layout == 3 ? rounds_h == 1 : 6 * rounds_h <= 10 * rounds256))
-    tile = 6;
-  else if (big_ok && t256 >= 128 && p.K >= 2048) tile = 5;
-  else if (big_ok && layout == 3 && t256 >= 192) tile = 4;
-  else if (big_ok && t256 >= (layout == 3 ? 96 : (p.K >= 1024 ? 24 : 48))) tile = 1;
+  if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
+  else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
+  else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
+  else if (whole_ok && t256 >= (layout == 3 ? 96 : (p.K >= 1024 ? 24 : 48))) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
@@ -688,6 +705,12 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   const int parts = mfma_splitk_parts(p);
   if (parts < 2) return false;
   const int layout = mfma_layout(p);
+  // a handful of tiles: nothing else occupies the device (192 x 512 x 2048: 23 us against 32 us for
+  // 64 x 64 tiles; 512 x 512 x 3072: 28 us against 35 us for half tiles; with both operands
+  // k-contiguous the 64 x 64 kernel holds out longer -- 192 x 512 x 2048: 19 us against 22 us, but
+  // 3072 x 128 x 3072: 33 us against 28 us)
+  const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256);
+  if (t256 <= 24 && parts >= 4 && p.K >= (layout == 3 ? 3072 : 2048)) return true;
   if ((layout & 2) == 0 || p.M <= 128) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;

@@ -380,15 +380,19 @@ bool skinny_supported(const GemmProblem& p) {
 // An n-contiguous weight streams at 4.3-4.8 TB/s at best (x . W with 14336 x 4096: 25-28 us for up
 // to 32 rows, where split-K takes 29 us and the k-contiguous form of this kernel 21 us), always with
 // 64 columns per workgroup, so it needs its workgroups to number at most one round, and a short k
-// loop when they are few; 8192-deep problems go to split-K (8 x 4096 x 8192: 25 us against 37 us)
+// loop when they are few; deeper problems go to split-K (8 x 4096 x 8192: 25 us against 37 us; 8 x 1024 x 8192: 21 against 36)
 // and more than 256 workgroups to the 128 x 256 tiles (8 x 28672 x 1024: 16 us against 19 us).
 bool skinny_preferred(const GemmProblem& p) {
+  // more than 32 rows, a k loop of a few blocks and many workgroups: the two-tile form's set-up does
+  // not pay (64 x 14336 x 64: 7.3 us against 5.5 us for 64 x 64 tiles; K = 256: 7.9 against 6.8; but
+  // 64 x 3072 x 256: 5.9 against 6.6)
+  if (p.M > 32 && p.K < 512 && (long long)((p.N + 31) / 32) * p.batch > 128) return false;
   if (p.sbk != 1) {
     const long long groups = (long long)((p.N + 63) / 64) * p.batch;
     if (groups > 256) return false;
     if (p.K <= 2048) return true;
     if (p.K <= 4096) return p.M <= 16 || groups <= 32 || groups >= (p.M <= 32 ? 192 : 224);
-    return p.M <= 16 && groups <= 32;
+    return false;
   }
   if (p.M <= 32) return true;
   const long long groups64 = (long long)((p.N + 63) / 64) * p.batch, groups32 = (long long)((p.N + 31) / 32) * p.batch;

@@ -197,8 +197,8 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256_m16"
     assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256_m16"
     assert query(native.REAL16BF, 8192, 8192, 8192, tb=True) == "mfma_256x256_m16"
-    # short k loops: the 32x32x16 kernels (64-deep stages when both operands are k-contiguous)
-    assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256"
+    # short k loops: the same, except that two k-contiguous operands take the kernel with 64-deep stages
+    assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256_m16"
     assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_k64"
     # few tiles and a long k loop: K split over the idle compute units -- when that buys more than the
     # half-height tiles a k-contiguous A allows
@@ -214,7 +214,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     # mid-size problems: the 256 x 256 kernels from 24 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16"             # 144 tiles, long k loop
-    assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256"
+    assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256_m16"             # and a short one
     # a k-contiguous A and at most one round of 128 x 256 tiles: the half-height form of the 16x16x32 kernel
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16"             # 128 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16"
@@ -227,7 +227,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16"              # 8 half tiles
     assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
     assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16"              # K too short to split
-    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_64x64"                     # and too short for the ring
+    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_128x256_m16"               # short k loops too (8.4 us against 10.0)
     assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"

@@ -20,6 +20,14 @@ pytestmark = pytest.mark.gpu
 DTS = [H.F32, H.F16, H.BF16]
 
 
+@pytest.fixture(autouse=True)
+def clean_plan_cache():
+    """Tests that pin a plan must not leak it into the next test."""
+    srt.PlanCache.clear()
+    yield
+    srt.PlanCache.clear()
+
+
 def query_kernel(a, ta, b, tb, out):
     ad, k1 = a.descriptor()
     bd, k2 = b.descriptor()
@@ -144,21 +152,15 @@ def test_integer_inputs_bit_exact_vs_oracle(dt, ta, tb):
                                           (4000, 3976, 200, "mfma_256x256")])
 def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, kernel, tmp_path):
     """Aligned shapes with ragged edges in M, N and K, every tile config and staging layout."""
-    if kernel == "mfma_128x128":
-        # the heuristic reaches this tile only when the 256 x 256 kernels' preconditions fail: pin it
-        # for this shape through the plan cache instead
-        layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
-        f = tmp_path / "plan.txt"
-        f.write_text(f"{dt} {M} {N} {K} 1 {layout} 10 mfma_128x128\n")
-        srt.PlanCache.clear()
-        srt.PlanCache.load(f)
+    # two k-contiguous operands have a 64-deep variant of the 256 x 256 kernel: cover it in their place
+    if kernel == "mfma_256x256" and not ta and tb:
+        kernel = "mfma_256x256_k64"
+    # which of these the heuristic takes for a shape moves with its tuning: pin the tile under test
+    pin_plan(tmp_path, kernel, dt, M, N, K, ta, tb)
     r = H.rng(100 + M)
     a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
     b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
     a_st, b_st = H.encode(a, dt), H.encode(b, dt)
-    # two k-contiguous operands take the 64-deep variant of the 256 x 256 kernel
-    if kernel == "mfma_256x256" and not ta and tb:
-        kernel = "mfma_256x256_k64"
     got = gpu_matmul(a_st, b_st, ta, tb, want_kernel=kernel)
     exact = (np.swapaxes(a, 0, 1) if ta else a).astype(np.int64) @ (np.swapaxes(b, 0, 1) if tb else b).astype(np.int64)
     assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
@@ -400,7 +402,7 @@ def test_skinny_up_to_64_rows_integer_exact_bias_and_choice(dt, tmp_path):
         exact = np.maximum(x.astype(np.float64) @ w.astype(np.float64).T + b[None, :], 0)
         assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
     srt.PlanCache.clear()
-    B_, M, N, K = 3, 48, 2056, 136
+    B_, M, N, K = 3, 48, 2056, 520
     x = r.integers(-2, 3, (B_, M, K)).astype(np.float32)
     w = r.integers(-2, 3, (B_, N, K)).astype(np.float32)
     xt, wt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt))
@@ -541,10 +543,11 @@ def test_every_activation_vs_oracle(act, dt):
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("act", list(srt.ActivationType))
-def test_ring_kernel_epilogues_vs_oracle(act, dt):
+def test_ring_kernel_epilogues_vs_oracle(act, dt, tmp_path):
     """Every activation (+ bias) through the 256 x 256 ring kernel, ragged M / N / K edges."""
     r = H.rng(16)
     M, N, K = 3600, 3592, 72
+    pin_plan_for_shape(tmp_path, "mfma_256x256", dt, M, N, K)
     x = H.encode(r.standard_normal((M, K)).astype(np.float32), dt)
     w = H.encode((r.standard_normal((K, N)) / 8).astype(np.float32), dt)
     b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
@@ -645,6 +648,16 @@ def test_m16_kernel_batched_short_k_and_nan(tmp_path):
 
 
 # ---- split-K over the 256 x 256 kernel --------------------------------------------------------------
+def pin_plan_for_shape(tmp_path, plan, dt, M, N, K, batch=1):
+    """Pins `plan` for a shape under every layout class and epilogue (and for the transposed problem a
+    column-major call turns into), for tests of one kernel that should not move with the heuristic."""
+    f = tmp_path / "plan_shape.txt"
+    f.write_text("".join(f"{dt} {m} {n} {K} {batch} {layout} {epi} {plan}\n"
+                         for (m, n) in ((M, N), (N, M)) for layout in range(128) for epi in range(14)))
+    srt.PlanCache.clear()
+    srt.PlanCache.load(f)
+
+
 def pin_plan(tmp_path, plan, dt, M, N, K, ta, tb, bias=False, act=srt.ActivationType.identity):
     layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
     f = tmp_path / "plan.txt"
@@ -832,7 +845,7 @@ def test_k64_kernel_batched_short_k_and_nan():
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
-def test_ring_kernel_batched_broadcast_and_column_major(dt):
+def test_ring_kernel_batched_broadcast_and_column_major(dt, tmp_path):
     """Rank-3 operands through the 256 x 256 ring kernel: strided batch, a broadcast (stride 0) weight,
     and a column-major problem (computed as C^T, bias then broadcast along the other dimension)."""
     r = H.rng(17)
@@ -843,6 +856,7 @@ def test_ring_kernel_batched_broadcast_and_column_major(dt):
     at = srt.Tensor(a_st)
     w3 = srt.Tensor(np.broadcast_to(w_st, (B_, K, N)).copy())
     out = srt.Tensor(shape=[B_, M, N], dtype=a_st.dtype)
+    pin_plan_for_shape(tmp_path, "mfma_256x256", dt, M, N, K, batch=B_)
     assert query_kernel(at, False, w3, False, out) == "mfma_256x256"
     got = srt.matmul(at, w3).array()
     exact = H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), dt)
@@ -862,6 +876,7 @@ def test_ring_kernel_batched_broadcast_and_column_major(dt):
     w2 = r.integers(-3, 4, (K2, N2)).astype(np.float32)
     b2 = r.integers(-3, 4, N2).astype(np.float32)
     xc, wc = srt.Tensor(H.encode(x, dt), order=srt.Order.col), srt.Tensor(H.encode(w2, dt), order=srt.Order.col)
+    pin_plan_for_shape(tmp_path, "mfma_256x256", dt, M2, N2, K2)
     yc = srt.matmul(xc, wc, bias=srt.Tensor(H.encode(b2, dt)))
     assert yc.order == srt.Order.col and query_kernel(xc, False, wc, False, yc) == "mfma_256x256"
     want = H.encode((x.astype(np.int64) @ w2.astype(np.int64) + b2.astype(np.int64)[None, :]).astype(np.float32), dt)
@@ -869,12 +884,14 @@ def test_ring_kernel_batched_broadcast_and_column_major(dt):
     # and relu on top (bias per row after the transposition inside the library)
     layer = srt.Dense(wc, srt.Tensor(H.encode(b2, dt)), srt.ActivationType.relu)
     assert np.array_equal(layer(xc).array().view(np.uint16), H.encode(np.maximum(H.decode(want), 0), dt).view(np.uint16))
+    srt.PlanCache.clear()
 
 
-def test_ring_kernel_nan_and_inf_encode_like_the_reference():
+def test_ring_kernel_nan_and_inf_encode_like_the_reference(tmp_path):
     """A NaN anywhere in a tile switches the wave to the exact encoder: NaN -> 0x7FFF, inf stays inf."""
     M = N = 3584
     K = 64
+    pin_plan_for_shape(tmp_path, "mfma_256x256", H.BF16, M, N, K)
     a = np.zeros((M, K), np.float32)
     b = np.zeros((K, N), np.float32)
     a[:, 0] = 1.0
@@ -891,6 +908,7 @@ def test_ring_kernel_nan_and_inf_encode_like_the_reference():
     layer = srt.Dense(srt.Tensor(H.encode(b, H.BF16)), None, srt.ActivationType.relu)
     y = layer(srt.Tensor(H.encode(a, H.BF16))).array()
     assert np.all(y[5] == 0) and np.all(y[300] == 0x7F80)
+    srt.PlanCache.clear()
 
 
 # ---- error behaviour -----------------------------------------------------------------------------
