@@ -603,17 +603,33 @@ int mfma_select(const GemmProblem& p) {
   //    k loops too (3072 x 8192 x 1024 with A m-contiguous: 56 us against 65 us; 3072 x 16384 x 512:
   //    60 against 67; 4096 x 4096 x 1024: 34.6 against 36.2) -- except with two k-contiguous
   //    operands, where the 64-deep kernel keeps short k loops (8192 x 8192 x 1024: 138 us against 146).
-  // (half tiles: with 64 columns or fewer only for longer k loops -- 1536 x 64 x 128: 10.4 us against
-  // 6.7 us for 64 x 64 tiles, 1536 x 64 x 768: 12.8 against 15.1 -- and whatever the rounds when the k
-  // loop is so short that the stores dominate: 6144 x 16384 x 256 80 us against 90 us for whole tiles)
-  const bool half_ok = p.K >= 64 && (p.N > 64 || p.K >= 512) &&
-                       (layout == 3 ? (th >= 96 && rounds_h == 1) : (p.K <= 256 || 6 * rounds_h <= 10 * rounds256));
-  const bool whole_ok = big_ok && p.M > 128 && p.N > 128;
+  // Half tiles: with 64 columns or fewer only for longer k loops and an n-contiguous B (1536 x 64 x 128:
+  // 10.4 us against 6.7 us for 64 x 64 tiles, 1536 x 64 x 768: 12.8 against 15.1; 32 x 1024 x 64 x 4096
+  // with B k-contiguous: 97 against 67).  With two k-contiguous operands a single matrix takes them only
+  // in one round; a batch whenever whole tiles would be padding or the k loop is short (8 x 128 x 4096 x
+  // 1024: 21 us against 28 us; 8 x 512 x 2048 x 256: 10.5 against 14.0; but 16 x 256 x 2048 x 2048: 81 us
+  // against 51 us for whole tiles).
+  const int m_rest = p.M % 256;
+  const bool half_nt = p.batch == 1 ? (th >= 96 && rounds_h == 1) : ((m_rest > 0 && m_rest <= 128) || p.K <= 512);
+  const bool half_ok = p.K >= 64 && (p.N > 64 || (layout == 2 && p.K >= 512)) &&
+                       (layout == 3 ? half_nt : 6 * rounds_h <= 10 * rounds256);
+  // Whole tiles: padding up to 256 rows and columns is affordable when the alternative is the 64 x 64
+  // kernel on two n- / m-contiguous operands, which it transposes in registers, and the device is at
+  // least half full (64 x 8 x 1024 x 256: 13.6 us against 19.6 us), or when the k loop is long, where the
+  // ring's prefetch outruns the 64 x 64 kernel's load-wait-compute stages whatever the tile count
+  // (16 x 128 x 2048 x 2048: 45 us against 110 us; 8 x 32 x 128 x 4096: 72 against 82; at K = 2048 with a
+  // k-contiguous B the 64 x 64 kernel is still ahead: 8 x 512 x 64 x 2048 34 us against 39 us).  With a
+  // short k loop and few tiles, or a k-contiguous B and under 128 rows, it is not (48 x 16384 x 768: 20.5 us
+  // against 15.9 us for 64 x 64 tiles; 128 x 14336 x 128: 10.2 against 8.0; 8 x 32 x 4096 x 64: 8.6 against
+  // 6.6; but 64 x 128 x 1024 x 128: 12.3 against 18.5).
+  const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
+                                   (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
+  const long long ring_from = layout == 3 ? 96 : (p.K >= 1024 ? 24 : 32);
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
   else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
   else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
-  else if (whole_ok && t256 >= (layout == 3 ? 96 : (p.K >= 1024 ? 24 : 48))) tile = 1;
+  else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout & 2) == 0))) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;

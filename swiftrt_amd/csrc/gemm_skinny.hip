@@ -387,6 +387,9 @@ bool skinny_preferred(const GemmProblem& p) {
   // not pay (64 x 14336 x 64: 7.3 us against 5.5 us for 64 x 64 tiles; K = 256: 7.9 against 6.8; but
   // 64 x 3072 x 256: 5.9 against 6.6)
   if (p.M > 32 && p.K < 512 && (long long)((p.N + 31) / 32) * p.batch > 128) return false;
+  // many rounds of workgroups with a short k loop each (a large batch): the per-workgroup set-up and
+  // reduction dominate (32 x 32 x 4096 x 512: 52 us against 28 us for 128 x 256 tiles)
+  if ((long long)((p.N + 31) / 32) * p.batch > 1024 && p.K < 2048) return false;
   if (p.sbk != 1) {
     const long long groups = (long long)((p.N + 63) / 64) * p.batch;
     if (groups > 256) return false;

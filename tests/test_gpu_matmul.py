@@ -822,7 +822,7 @@ def test_k64_kernel_epilogues_vs_oracle(act, dt):
     assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
 
 
-def test_k64_kernel_batched_short_k_and_nan():
+def test_k64_kernel_batched_short_k_and_nan(tmp_path):
     """Strided batch, K shorter than one stage (8) and of one, two and three stages, a NaN row."""
     r = H.rng(18)
     for K in (8, 64, 72, 136, 192):
@@ -830,6 +830,7 @@ def test_k64_kernel_batched_short_k_and_nan():
         a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
         w = r.integers(-3, 4, (B_, N, K)).astype(np.float32)
         at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+        pin_plan_for_shape(tmp_path, "mfma_256x256_k64", H.BF16, M, N, K, batch=B_)
         out = srt.matmul(at, wt, transposed_rhs=True)
         assert query_kernel(at, False, wt, True, out) == "mfma_256x256_k64"
         exact = a.astype(np.int64) @ np.swapaxes(w, 1, 2).astype(np.int64)
@@ -840,6 +841,7 @@ def test_k64_kernel_batched_short_k_and_nan():
     w[:, 0] = 2.0
     a[5, 1] = np.nan
     w[:, 1] = 1.0
+    pin_plan_for_shape(tmp_path, "mfma_256x256_k64", H.BF16, 3584, 3584, 64)
     got = gpu_matmul(H.encode(a, H.BF16), H.encode(w, H.BF16), tb=True, want_kernel="mfma_256x256_k64")
     assert np.all(got[5] == 0x7FFF) and np.all(got[6] == H.encode(np.array([2.0], np.float32), H.BF16)[0])
 
