@@ -715,7 +715,8 @@ int mfma_splitk_parts(const GemmProblem& p) {
 //                           tiles), two from K = 8192 (1536 x 4096 x 11008: 136 us against 168 us)
 //   A k-, B n-contiguous    eight parts from K = 4096 (512 x 4096 x 4096: 43 us against ~50 us for half
 //                           tiles; with four parts the two tie), four from K = 8192 (2048 x 2048 x
-//                           8192: 79 us) or when M <= 256 (64 x 14336 x 4096: 37 us against 46 us);
+//                           8192: 79 us) or when M <= 192 (64 x 14336 x 4096: 37 us against 46 us;
+//                           256 x 14336 x 4096: 54 us against 47 us for half tiles);
 //                           two parts lose to half tiles (2048 x 4096 x 11008: 183 against 154)
 bool mfma_prefers_splitk(const GemmProblem& p) {
   const int parts = mfma_splitk_parts(p);
@@ -730,7 +731,7 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   if ((layout & 2) == 0 || p.M <= 128) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;
-  return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 256));
+  return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 192));
 }
 
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {
