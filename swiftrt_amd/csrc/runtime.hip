@@ -18,15 +18,20 @@ inline hipStream_t hs(srtStream s) { return reinterpret_cast<hipStream_t>(s); }
 inline hipEvent_t he(srtEvent e) { return reinterpret_cast<hipEvent_t>(e); }
 
 // ---- caching allocator ---------------------------------------------------------------------
-// Blocks are binned by rounded size per device.  A free block remembers the stream it was
-// last associated with and an event recorded on that stream at free time; it is handed out
-// again to the same stream at once, to another stream only when the event has completed.
+// Blocks are binned by rounded size per device.  A free block remembers the stream it was last
+// associated with; it is handed out again to the same stream at once (stream order protects it),
+// to another stream only when an event recorded on the first stream has completed.  That event is
+// recorded when the other stream first asks, not at free time: it then covers more work than it
+// needs to, which is safe, and the common allocate / free / allocate cycle of one stream (a
+// workspace per call) queues no event at all -- an event recorded after every free cost each such
+// call about 5 us of idle device between its last kernel and the next call's first.
 struct Block {
   void* ptr;
   size_t size;
   int device;
   hipStream_t stream;
-  hipEvent_t ready;  // recorded at free time; null while live
+  hipEvent_t ready;  // null while live and until another stream asks for the free block
+  bool pending;      // free, possibly still in use by work queued on `stream`, no event recorded yet
 };
 
 const hipStream_t kNoStream = reinterpret_cast<hipStream_t>(~uintptr_t(0));   // matches no real stream
@@ -57,12 +62,26 @@ class CachingAllocator {
       for (auto it = range.first; it != range.second; ++it) {
         Block& b = it->second;
         bool usable = (b.stream == stream);
+        if (!usable && b.pending) {
+          // first request from another stream: mark the point the block's stream has reached
+          hipEvent_t ev = nullptr;
+          if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess &&
+              hipEventRecord(ev, b.stream) == hipSuccess) {
+            b.ready = ev;
+            b.pending = false;
+          } else {
+            if (ev) (void)hipEventDestroy(ev);
+            (void)hipGetLastError();
+            continue;   // cannot be ordered now: leave it to its own stream
+          }
+        }
         if (!usable && b.ready) usable = (hipEventQuery(b.ready) == hipSuccess);
-        if (!usable && !b.ready) usable = true;
+        if (!usable && !b.ready && !b.pending) usable = true;
         if (usable) {
           Block blk = b;
           free_.erase(it);
           if (blk.ready) { (void)hipEventDestroy(blk.ready); blk.ready = nullptr; }
+          blk.pending = false;
           blk.stream = stream;
           live_[blk.ptr] = blk;
           *out = blk.ptr;
@@ -80,7 +99,7 @@ class CachingAllocator {
       if (e != hipSuccess) { (void)hipGetLastError(); return srtErrorOutOfMemory; }
     }
     std::lock_guard<std::mutex> lock(mu_);
-    live_[p] = Block{p, rs, device, stream, nullptr};
+    live_[p] = Block{p, rs, device, stream, nullptr, false};
     *out = p;
     return srtSuccess;
   }
@@ -95,22 +114,18 @@ class CachingAllocator {
       blk = it->second;
       live_.erase(it);
     }
-    int prev = 0;
-    (void)hipGetDevice(&prev);
-    if (prev != blk.device) (void)hipSetDevice(blk.device);
-    hipEvent_t ev = nullptr;
-    // a block whose stream has been destroyed cannot be ordered by an event on it
-    if (blk.stream != kNoStream && hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess) {
-      if (hipEventRecord(ev, blk.stream) != hipSuccess) { (void)hipEventDestroy(ev); ev = nullptr; }
-    }
-    if (!ev) {
-      // could not order the free (e.g. the stream no longer exists): make it safe the slow way
-      (void)hipGetLastError();
+    blk.ready = nullptr;
+    blk.pending = true;
+    if (blk.stream == kNoStream) {
+      // the stream was destroyed while the block was live: nothing can order the free, so make it
+      // safe the slow way
+      int prev = 0;
+      (void)hipGetDevice(&prev);
+      if (prev != blk.device) (void)hipSetDevice(blk.device);
       (void)hipDeviceSynchronize();
-      blk.stream = kNoStream;
+      if (prev != blk.device) (void)hipSetDevice(prev);
+      blk.pending = false;
     }
-    if (prev != blk.device) (void)hipSetDevice(prev);
-    blk.ready = ev;
     std::lock_guard<std::mutex> lock(mu_);
     free_.emplace(Key{blk.device, blk.size}, blk);
     return srtSuccess;
@@ -122,8 +137,27 @@ class CachingAllocator {
   // device-wide synchronisation).
   void forget_stream(hipStream_t stream) {
     std::lock_guard<std::mutex> lock(mu_);
-    for (auto& kv : free_)
-      if (kv.second.stream == stream) kv.second.stream = kNoStream;
+    for (auto& kv : free_) {
+      Block& b = kv.second;
+      if (b.stream != stream) continue;
+      if (b.pending) {
+        // last chance to order the block behind the stream's work: events outlive their stream
+        int prev = 0;
+        (void)hipGetDevice(&prev);
+        if (prev != b.device) (void)hipSetDevice(b.device);
+        hipEvent_t ev = nullptr;
+        if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess && hipEventRecord(ev, stream) == hipSuccess) {
+          b.ready = ev;
+        } else {
+          if (ev) (void)hipEventDestroy(ev);
+          (void)hipGetLastError();
+          (void)hipStreamSynchronize(stream);
+        }
+        if (prev != b.device) (void)hipSetDevice(prev);
+        b.pending = false;
+      }
+      b.stream = kNoStream;
+    }
     for (auto& kv : live_)
       if (kv.second.stream == stream) kv.second.stream = kNoStream;
   }
@@ -140,6 +174,7 @@ class CachingAllocator {
     for (Block& b : blocks) {
       (void)hipSetDevice(b.device);
       if (b.ready) { (void)hipEventSynchronize(b.ready); (void)hipEventDestroy(b.ready); }
+      if (b.pending) (void)hipStreamSynchronize(b.stream);
       (void)hipFree(b.ptr);
     }
     (void)hipSetDevice(prev);

@@ -56,6 +56,38 @@ def test_caching_allocator_reuses_blocks_per_stream():
     native.check(native.lib().srtDeviceEmptyCache())
 
 
+def test_caching_allocator_orders_blocks_across_streams():
+    """A block freed on one stream goes to another stream only when the work the first stream had
+    queued by then has finished; to its own stream it goes back at once."""
+    p = srt.HipPlatform.local()
+    q0, q1 = p.devices[1].queues[0], p.devices[1].queues[1]
+    q0.wait_for_completion()
+    q1.wait_for_completion()
+    native.check(native.lib().srtDeviceEmptyCache())
+    m = q0.allocate(3 << 20)
+    p0 = m.pointer
+    q0.delay(0.2)                  # q0 is busy: work that may still use the block
+    del m                          # freed on q0 while the delay runs
+    other = q1.allocate(3 << 20)   # another stream asks for the same bin: must not get the busy block
+    assert other.pointer != p0
+    same = q0.allocate(3 << 20)    # its own stream gets it back at once (stream order protects it)
+    assert same.pointer == p0
+    del same
+    q0.wait_for_completion()
+    # q0 has drained: now the block may move to q1 -- as soon as the event that the first request from
+    # q1 records on q0 has been processed, which takes the device a moment even on an idle stream
+    for _ in range(200):
+        again = q1.allocate(3 << 20)
+        if again.pointer == p0:
+            break
+        del again
+        time.sleep(0.005)
+    assert again.pointer == p0
+    del other, again
+    q1.wait_for_completion()
+    native.check(native.lib().srtDeviceEmptyCache())
+
+
 def test_events_delay_and_cross_queue_wait():
     p = srt.HipPlatform.local()
     q0, q1 = p.devices[1].queues[0], p.devices[1].queues[1]
