@@ -211,7 +211,9 @@ srtStatus srtMatmulBiasActivation(const void* a, const srtTensorDescriptor* aDes
                                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 
 /* Name of the kernel family the dispatcher selects for this problem ("mfma_256x256_m16",
- * "mfma_256x256", "skinny", "generic", ...), written into `name`; nothing is launched.  Diagnostic only
+ * "mfma_256x256", "skinny", "generic", ...), written into `name`; nothing is launched.  A 16-bit problem
+ * whose operands span 1 Gi elements or more runs as several launches over halves of its batch, M or N;
+ * the name is then that of the first piece's kernel followed by "/pieces".  Diagnostic only
  * (the reference's matmul diagnostic line, CudaMatmul.swift:34-37, has no counterpart for
  * kernel choice). */
 srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transposeA,

@@ -254,7 +254,68 @@ Plan select(const GemmProblem& p) {
   return heuristic_plan(p);
 }
 
+// ---- operands beyond the 256 x 256 kernels' reach -------------------------------------------------
+// The 256 x 256 kernels address every operand through one buffer descriptor and 32-bit byte
+// offsets, so each operand tensor of a launch (all batches) must span less than 1 Gi elements.
+// A device with hundreds of GB holds larger ones (262144 x 8192 activations, 64 batches of
+// 8192 x 8192): rather than hand those to the 128 x 128 kernel at half the rate, the call is cut
+// into pieces that are within reach -- halves of the batch, then of M, then of N, at multiples of
+// the tile size -- and the pieces run back to back on the caller's stream.  A piece is an ordinary
+// problem (its own pointers, the same strides) and goes through the same plan selection.  An
+// operand whose k walk alone exceeds the reach (K x leading stride >= 1 Gi elements when k is not
+// its contiguous dimension) cannot be helped this way and keeps the smaller tiles.
+bool fits_256(const GemmProblem& p) { return srt::mfma_config(p, 1) != 0; }
+
+bool split_for_reach(const GemmProblem& p, GemmProblem* lo, GemmProblem* hi) {
+  if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return false;
+  if (fits_256(p)) return false;
+  const long long tiles = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
+  if (tiles < 128) return false;   // the small tiles are the choice there anyway
+  GemmProblem q = p;
+  q.batch = 1; q.M = p.M < 256 ? p.M : 256; q.N = p.N < 256 ? p.N : 256;
+  if (!fits_256(q)) return false;   // alignment, or a k walk out of reach: not a matter of extent
+  const size_t es = 2;
+  auto at = [es](const void* base, long long elements) {
+    return static_cast<const void*>(static_cast<const char*>(base) + elements * (long long)es);
+  };
+  *lo = p; *hi = p;
+  if (p.batch > 1) {
+    const int h = p.batch / 2;
+    lo->batch = h; hi->batch = p.batch - h;
+    hi->A = at(p.A, h * p.sab); hi->B = at(p.B, h * p.sbb);
+    hi->C = const_cast<void*>(at(p.C, h * p.scb));
+    return true;
+  }
+  GemmProblem qm = p; qm.M = q.M;   // would whole columns of tiles fit?
+  const bool by_m = p.M > 256 && (fits_256(qm) || p.N <= 256);
+  if (by_m) {
+    const int m0 = ((p.M / 2 + 255) / 256) * 256;
+    lo->M = m0; hi->M = p.M - m0;
+    hi->A = at(p.A, m0 * p.sam);
+    hi->C = const_cast<void*>(at(p.C, m0 * p.scm));
+    if (p.bias && p.bias_per_row) hi->bias = at(p.bias, m0 * p.sbias);
+    return true;
+  }
+  if (p.N <= 256) return false;
+  const int n0 = ((p.N / 2 + 255) / 256) * 256;
+  lo->N = n0; hi->N = p.N - n0;
+  hi->B = at(p.B, n0 * p.sbn);
+  hi->C = const_cast<void*>(at(p.C, n0 * p.scn));
+  if (p.bias && !p.bias_per_row) hi->bias = at(p.bias, n0 * p.sbias);
+  return true;
+}
+
+bool has_cached_plan(const GemmProblem& p) {
+  Plan plan;
+  return plan_cache().size() != 0 && plan_cache().find(key_of(p), &plan) && plan_supported(p, plan);
+}
+
 srtStatus run(const GemmProblem& p, hipStream_t stream) {
+  GemmProblem lo, hi;
+  if (!has_cached_plan(p) && split_for_reach(p, &lo, &hi)) {
+    const srtStatus s = run(lo, stream);
+    return s != srtSuccess ? s : run(hi, stream);
+  }
   const Plan plan = select(p);
   if (plan == kPlanGeneric && !srt::generic_supported(p)) return srtErrorNotSupported;
   hipError_t e = launch_plan(p, plan, stream);
@@ -304,9 +365,17 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
   if (s != srtSuccess) return s;
   const char* n = "empty";
   if (!empty) {
-    const Plan plan = select(p);
+    // a call that runs in pieces reports its first piece's kernel, marked "/pieces"
+    GemmProblem piece = p, lo, hi;
+    bool pieces = false;
+    while (!has_cached_plan(piece) && split_for_reach(piece, &lo, &hi)) { piece = lo; pieces = true; }
+    const Plan plan = select(piece);
     n = kPlanNames[plan];
     if (plan == kPlanF32Tile64 || plan == kPlanF32SplitK) n = "f32_mfma";   // one family name for both fp32 tiles
+    if (pieces) {
+      std::snprintf(name, nameCapacity, "%s/pieces", n);
+      return srtSuccess;
+    }
   }
   std::snprintf(name, nameCapacity, "%s", n);
   return srtSuccess;
@@ -325,6 +394,14 @@ srtStatus srtMatmulTune(const void* a, const srtTensorDescriptor* aDesc, int32_t
                               out, oDesc, &p, &empty);
   if (s != srtSuccess || empty) return s;
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+  {
+    // a problem that runs in pieces has no single plan to record: its pieces keep the heuristic
+    GemmProblem lo, hi;
+    if (!has_cached_plan(p) && split_for_reach(p, &lo, &hi)) {
+      if (chosen && chosenCapacity) std::snprintf(chosen, chosenCapacity, "pieces");
+      return run(p, hs);
+    }
+  }
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess) return srtErrorUnknown;
   if (hipEventCreate(&e1) != hipSuccess) { (void)hipEventDestroy(e0); return srtErrorUnknown; }

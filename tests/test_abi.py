@@ -250,6 +250,14 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 64, 64, 64, align=2) == "mfma_64x64_any"            # misaligned view
     assert query(native.REAL16F, 2048, 50257, 768) == "mfma_128x128_any"              # odd row pitch of B and C
     assert query(native.REAL32F, 512, 512, 512) in ("generic", "f32_mfma")
+    # operands of 1 Gi elements or more: halves of M (N for a k-contiguous B, the batch first) that the
+    # 256 x 256 kernels' 32-bit offsets reach; a k walk out of reach keeps the small tiles
+    assert query(native.REAL16BF, 32768, 32768, 8192) == "mfma_256x256_m16/pieces"           # C alone is 1 Gi
+    assert query(native.REAL16BF, 262144, 8192, 8192) == "mfma_256x256_m16/pieces"           # A and C
+    assert query(native.REAL16BF, 8192, 262144, 8192, tb=True) == "mfma_256x256_m16/pieces"  # B [N, K] and C
+    assert query(native.REAL16BF, 8192, 8192, 262144, ta=True) == "mfma_128x128"             # k walk of A and B
+    assert query(native.REAL16BF, 32768, 32512, 8192) == "mfma_256x256_m16"                  # just within reach
+    assert query(native.REAL16BF, 8, 65664, 32768, tb=True) == "skinny/pieces"
 
 
 def test_tensor_layout_and_views():

@@ -936,3 +936,85 @@ def test_empty_extents_launch_nothing():
     a = srt.Tensor(shape=[3, 0], dtype=np.float32)
     b = srt.Tensor(shape=[0, 4], dtype=np.float32)
     assert np.array_equal(srt.matmul(a, b).array(), np.zeros((3, 4), np.float32))
+
+
+# ---- operands of 1 Gi elements and more (byte offsets beyond 32 bits) ---------------------------------
+def _periodic(block, reps, axis):
+    """`reps` copies of `block` along `axis`: a > 4 GB operand whose product is known from one block."""
+    return np.ascontiguousarray(np.concatenate([block] * reps, axis=axis))
+
+
+@pytest.mark.parametrize("case", ["nn_big_a", "nt_big_w", "tn_big_a", "skinny_big_w"])
+def test_bf16_operands_beyond_4_gib_bit_exact(case):
+    """An operand of 2.15 Gi bf16 elements (4.3 GB).  Where halves of M or N bring it within the 256 x 256
+    kernels' 32-bit offsets the call runs in pieces; an m-contiguous A whose k walk alone is out of reach
+    runs on the 128 x 128 tiles with 64-bit addressing.  Sparse {-1, 0, 1} operands: exact in any order;
+    the big operand repeats a 1152-row block (4.5 tiles, so no piece boundary falls on a block boundary)."""
+    r = H.rng(400)
+    P, reps, K = 1152, 57, 32768                 # 57 x 1152 = 65664 rows
+    big0 = (r.integers(-1, 2, (P, K)) * (r.random((P, K)) < 0.25)).astype(np.float32)
+    small_rows = 8 if case == "skinny_big_w" else 512
+    small = (r.integers(-1, 2, (small_rows, K)) * (r.random((small_rows, K)) < 0.25)).astype(np.float32)
+    block = big0.astype(np.float64) @ small.astype(np.float64).T          # [P, small_rows], exact integers
+    if case == "nn_big_a":      # A [65664, K] . B [K, 512]
+        a, b, ta, tb = _periodic(H.encode(big0, H.BF16), reps, 0), H.encode(np.ascontiguousarray(small.T), H.BF16), False, False
+        want, kernel = np.concatenate([block] * reps, 0), "mfma_256x256_m16/pieces"
+    elif case == "tn_big_a":    # A stored [K, 65664], transposed
+        a, b, ta, tb = _periodic(H.encode(np.ascontiguousarray(big0.T), H.BF16), reps, 1), H.encode(np.ascontiguousarray(small.T), H.BF16), True, False
+        want, kernel = np.concatenate([block] * reps, 0), "mfma_128x128"
+    else:                       # x [512 or 8, K] . W [65664, K]^T
+        a, b, ta, tb = H.encode(small, H.BF16), _periodic(H.encode(big0, H.BF16), reps, 0), False, True
+        want = np.concatenate([block.T] * reps, 1)
+        kernel = "skinny/pieces" if case == "skinny_big_w" else "mfma_256x256_m16/pieces"
+    assert max(a.size, b.size) > 2 ** 31
+    got = gpu_matmul(a, b, ta, tb, want_kernel=kernel)
+    assert np.array_equal(got, H.encode(want.astype(np.float32), H.BF16))
+
+
+def test_bf16_batches_beyond_reach_run_in_pieces_bit_exact():
+    """72 batches of 2048 x 8192 (1.2 Gi elements of A): the batch is halved until a piece is within reach;
+    every batch must land in its own slab of the result.  Bias and ReLU go with every piece."""
+    r = H.rng(401)
+    nb, M, N, K = 72, 2048, 2048, 8192
+    a0 = (r.integers(-1, 2, (3, M, K)) * (r.random((3, M, K)) < 0.25)).astype(np.float32)
+    b0 = (r.integers(-1, 2, (3, K, N)) * (r.random((3, K, N)) < 0.25)).astype(np.float32)
+    bias = r.integers(-4, 5, N).astype(np.float32)
+    a = np.ascontiguousarray(np.concatenate([H.encode(a0, H.BF16)] * (nb // 3), 0))
+    b = np.ascontiguousarray(np.concatenate([H.encode(b0, H.BF16)] * (nb // 3), 0))
+    at, bt = srt.Tensor(a), srt.Tensor(b)
+    out = srt.Tensor(shape=[nb, M, N], dtype=a.dtype)
+    assert query_kernel(at, False, bt, False, out) == "mfma_256x256_m16/pieces"
+    srt.current_queue().matmul(at, False, bt, False, out, bias=srt.Tensor(H.encode(bias, H.BF16)),
+                               activation=srt.ActivationType.relu)
+    block = np.maximum(a0.astype(np.float64) @ b0.astype(np.float64) + bias, 0.0)
+    want = H.encode(np.concatenate([block] * (nb // 3), 0).astype(np.float32), H.BF16)
+    assert np.array_equal(out.array(), want)
+
+
+def test_bias_follows_the_pieces_along_n():
+    """x . W^T + bias with a W of 65664 x 16384 (1 Gi elements and 128 columns more): the pieces along N take
+    their own part of the bias."""
+    r = H.rng(402)
+    P, reps, K, M = 1152, 57, 16384, 300
+    w0 = (r.integers(-1, 2, (P, K)) * (r.random((P, K)) < 0.25)).astype(np.float32)
+    x = (r.integers(-1, 2, (M, K)) * (r.random((M, K)) < 0.25)).astype(np.float32)
+    bias = r.integers(-64, 65, P * reps).astype(np.float32)
+    xt, wt = srt.Tensor(H.encode(x, H.BF16)), srt.Tensor(_periodic(H.encode(w0, H.BF16), reps, 0))
+    out = srt.Tensor(shape=[M, P * reps], dtype=np.uint16)
+    assert query_kernel(xt, False, wt, True, out).endswith("/pieces")
+    srt.current_queue().matmul(xt, False, wt, True, out, bias=srt.Tensor(H.encode(bias, H.BF16)),
+                               activation=srt.ActivationType.identity)
+    block = x.astype(np.float64) @ w0.astype(np.float64).T
+    want = np.concatenate([block] * reps, 1) + bias
+    assert np.array_equal(out.array(), H.encode(want.astype(np.float32), H.BF16))
+
+
+def test_fp32_operand_beyond_4_gib_vs_exact():
+    """fp32 A of 33408 x 32768 (4.4 GB): the fp32 kernels address with 64-bit offsets."""
+    r = H.rng(403)
+    P, reps, K, N = 1152, 29, 32768, 256
+    a0 = (r.integers(-2, 3, (P, K)) * (r.random((P, K)) < 0.25)).astype(np.float32)
+    b = (r.integers(-2, 3, (K, N)) * (r.random((K, N)) < 0.25)).astype(np.float32)
+    got = gpu_matmul(_periodic(a0, reps, 0), b)
+    block = (a0.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(got, np.concatenate([block] * reps, 0))
