@@ -191,17 +191,16 @@ __global__ __launch_bounds__(NT) void gemm_kc64_kernel(GemmProblem p) {
   }
   // all LDS traffic of the main loop has retired in every wave before the slots become the
   // epilogue's staging area
+  constexpr bool LINEAR_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED;
+  u32x2_t bias_regs[16];
+  if (LINEAR_BIAS) load_bias<T>(p, m0 + wm0, n0 + wn0, lane, bias_regs);   // lands during the wait below
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   const uint32_t stage = lds + (uint32_t)wave * 16384u;
 
   if (EPI == EPI_TRANS) {
     store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
   } else {
-    if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1>(p, acc, m0 + wm0, n0 + wn0, lane);
-    else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2>(p, acc, m0 + wm0, n0 + wn0, lane);
-    store_tile<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+    store_tile_linear<T, EPI>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage, bias_regs);
   }
 }
 

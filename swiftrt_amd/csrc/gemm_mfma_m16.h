@@ -201,39 +201,46 @@ struct FragReader {
 // ---- epilogue ------------------------------------------------------------------------------------
 // acc[i][j] is a transposed 16 x 16 tile: lane l owns row m = wave_m0 + 16 i + l % 16 and the
 // columns n = wave_n0 + 16 j + 4 (l / 16) + 0..3.
-template <typename T, bool HAS_BIAS, int CLAMP, int TM>
-__device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x4_t (&acc)[TM][8], int wave_m0,
-                                                      int wave_n0, int lane) {
+//
+// The bias values a lane adds -- 32 per-column ones (or TM per-row ones after a C^T flip) -- are
+// requested in one batch right after the k loop, ahead of the wait and barrier that end it, so
+// their latency passes while the matrix pipe drains.  Read where they are used, inside the pass
+// over the accumulators, they came in eight dependent rounds of a global load's latency each
+// (5.5 us of a 95 us tile at K = 4096).  A dense, 8-byte-aligned bias is read as eight 8-byte loads.
+// They wait in their stored 16-bit form, two to a register (16 registers per lane): b[j] holds the four
+// per-column values of column tile j; in the per-row case b[i].x holds row tile i's value.
+template <typename T, int TM>
+__device__ __forceinline__ void load_bias(const GemmProblem& p, int wave_m0, int wave_n0, int lane, u32x2_t (&b)[8]) {
   using S = typename T::storage;
+  static_assert(sizeof(S) == 2 && TM <= 8, "16-bit element types, at most 8 row tiles");
   const S* bias = (const S*)p.bias;
-  const bool per_row = p.bias_per_row != 0;
-  const float ceiling = p.coef;
   const int jn = lane & 15, g = lane >> 4;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    float bcol[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (HAS_BIAS) {
+  for (int j = 0; j < 8; ++j) b[j] = u32x2_t{0u, 0u};
+  if (!bias) return;
+  if (p.bias_per_row) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = wave_m0 + 16 * i + jn;
+      if (m < p.M) b[i].x = bias[(long long)m * p.sbias];
+    }
+  } else if (p.sbias == 1 && (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) {
+    // N is a multiple of 8 and n of 4: a lane's four columns are all inside or all outside
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = wave_n0 + 16 * j + 4 * g;
+      if (n < p.N) b[j] = *reinterpret_cast<const u32x2_t*>(bias + n);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      uint32_t h[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int n = wave_n0 + 16 * j + 4 * g + e;
-        bcol[e] = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
+        if (n < p.N) h[e] = bias[(long long)n * p.sbias];
       }
-    }
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      float brow = 0.0f;
-      if (HAS_BIAS) {
-        const int m = wave_m0 + 16 * i + jn;
-        brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float x = acc[i][j][e];
-        if (HAS_BIAS) x += per_row ? brow : bcol[e];
-        if (CLAMP >= 1) x = __builtin_fmaxf(x, 0.0f);
-        if (CLAMP == 2) x = __builtin_fminf(x, ceiling);
-        acc[i][j][e] = x;
-      }
+      b[j] = u32x2_t{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
     }
   }
 }
@@ -245,11 +252,15 @@ __device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x
 // sides: a write instruction covers 16 rows x 32 B, a read 4 whole rows).
 // NaN handling as in ring::store_tile: the hardware converter rounds everything, and when any
 // lane of the wave saw a NaN the staged patterns are rewritten to 0x7FFF on the way out.
-template <typename T, int TM>
+// Bias and the clamps (CLAMP 1: relu, 2: clipped relu) are applied to the copy that leaves the
+// accumulator registers, so the accumulators themselves are only read.
+template <typename T, int TM, bool HAS_BIAS, int CLAMP>
 __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[TM][8], int wave_m0, int wave_n0,
-                                           int bz, int lane, uint32_t stage) {
+                                           int bz, int lane, uint32_t stage, const u32x2_t (&b)[8]) {
   constexpr int ROWS = TM == 8 ? 64 : 32;
   using S = typename T::storage;
+  const bool per_row = p.bias_per_row != 0;
+  const float ceiling = p.coef;
   constexpr bool FIXUP = T::dtype == srtReal16BF;
   S* C = (S*)p.C + (long long)bz * p.scb;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
@@ -274,6 +285,21 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
         float a0 = acc[i][j][0], a1 = acc[i][j][1], a2 = acc[i][j][2], a3 = acc[i][j][3];
         // one copy out of the accumulator registers, here, for both the test and the conversion
         asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+        if (HAS_BIAS) {
+          const float br = T::to_float((S)(b[i].x & 0xffffu));
+          a0 += per_row ? br : T::to_float((S)(b[j].x & 0xffffu));
+          a1 += per_row ? br : T::to_float((S)(b[j].x >> 16));
+          a2 += per_row ? br : T::to_float((S)(b[j].y & 0xffffu));
+          a3 += per_row ? br : T::to_float((S)(b[j].y >> 16));
+        }
+        if (CLAMP >= 1) {
+          a0 = __builtin_fmaxf(a0, 0.0f); a1 = __builtin_fmaxf(a1, 0.0f);
+          a2 = __builtin_fmaxf(a2, 0.0f); a3 = __builtin_fmaxf(a3, 0.0f);
+        }
+        if (CLAMP == 2) {
+          a0 = __builtin_fminf(a0, ceiling); a1 = __builtin_fminf(a1, ceiling);
+          a2 = __builtin_fminf(a2, ceiling); a3 = __builtin_fminf(a3, ceiling);
+        }
         if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
         const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};
         const int c = 2 * j + (g >> 1);
@@ -712,25 +738,27 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     // Every load in flight must have landed, in every wave, before the slots vacated last become
     // the staging area.  The s_nops are the wait states between the last MFMAs and the first
     // reads of their accumulators by other instructions.
+    const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
+    const int le = lane_id();
+    constexpr bool LINEAR_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED;
+    u32x2_t bias_regs[8];
+    if (LINEAR_BIAS) load_bias<T, TM>(p, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
     // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1 (half a slot each)
     uint32_t pprv = prv - STAGE_B;
     if (prv == lds) pprv = lds + (NS - 1) * STAGE_B;
     const uint32_t stage = ((wave & 2) ? prv : pprv) + (uint32_t)(wave & 1) * (uint32_t)(STAGE_B / 2);
-    const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
-    const int le = lane_id();
 
     if (EPI == EPI_PARTIAL) {
       store_tile_partial<TM>(p, acc, em0, en0, bz, le, stage);
     } else if (EPI == EPI_TRANS) {
       store_tile_transcendental<T, TM>(p, acc, em0, en0, bz, le, stage);
     } else {
-      if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0, TM>(p, acc, em0, en0, le);
-      else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1, TM>(p, acc, em0, en0, le);
-      else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1, TM>(p, acc, em0, en0, le);
-      else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2, TM>(p, acc, em0, en0, le);
-      if (EPI != EPI_PLAIN) pin_all<TM>(acc);
-      store_tile<T, TM>(p, acc, em0, en0, bz, le, stage);
+      if (EPI == EPI_BIAS) store_tile<T, TM, true, 0>(p, acc, em0, en0, bz, le, stage, bias_regs);
+      else if (EPI == EPI_RELU) store_tile<T, TM, false, 1>(p, acc, em0, en0, bz, le, stage, bias_regs);
+      else if (EPI == EPI_BIAS_RELU) store_tile<T, TM, true, 1>(p, acc, em0, en0, bz, le, stage, bias_regs);
+      else if (EPI == EPI_CLIPPED) store_tile<T, TM, true, 2>(p, acc, em0, en0, bz, le, stage, bias_regs);
+      else store_tile<T, TM, false, 0>(p, acc, em0, en0, bz, le, stage, bias_regs);
     }
     if (!has_next) break;
 

@@ -254,52 +254,52 @@ __device__ __forceinline__ void pin_all(f32x16_t (&acc)[4][4]) {
 // acc[i][j] is a transposed 32 x 32 tile: lane l owns row m = wave_m0 + 32 i + l % 32 and, in
 // registers 4 g .. 4 g + 3, the columns n = wave_n0 + 32 j + 8 g + 4 (l / 32) + 0..3.
 //
-// Step 1 for identity / relu / clippedRelu (apply_linear_epilogue): bias, then the activation as
-// one or two min/max instructions, in place and in straight-line code (the accumulators never
-// cross a branch); HAS_BIAS and CLAMP are compile-time so each variant carries only the
-// instructions it needs (with HAS_BIAS a null bias pointer adds nothing).  CLAMP: 0 none,
+// Step 1 for identity / relu / clippedRelu (load_bias): the bias values a lane adds -- 64
+// per-column ones, or 4 per-row ones after a C^T flip -- are requested in one batch right after
+// the k loop, ahead of the wait and barrier that end it, so their latency passes while the matrix
+// pipe drains (read where they are used they came in sixteen dependent rounds of a global load's
+// latency each).  They wait in their stored 16-bit form, two to a register: b[4 j + g] holds the
+// four values of column group (j, g); in the per-row case b[i].x holds row tile i's value.  A
+// dense, 8-byte-aligned bias is read as sixteen 8-byte loads.  Bias, then the activation as one or
+// two min/max instructions, are applied in store_tile to the copy that leaves the accumulator
+// registers, in straight-line code; HAS_BIAS and CLAMP are compile-time so each variant carries
+// only the instructions it needs (with HAS_BIAS a null bias pointer adds nothing).  CLAMP: 0 none,
 // 1 relu = max(x, 0), 2 clippedRelu = min(max(x, 0), coef).  max(NaN, 0) is 0 on this hardware,
 // which is also what x > 0 ? x : 0 gives.
-template <typename T, bool HAS_BIAS, int CLAMP>
-__device__ __forceinline__ void apply_linear_epilogue(const GemmProblem& p, f32x16_t (&acc)[4][4], int wave_m0,
-                                                      int wave_n0, int lane) {
+template <typename T>
+__device__ __forceinline__ void load_bias(const GemmProblem& p, int wave_m0, int wave_n0, int lane, u32x2_t (&b)[16]) {
   using S = typename T::storage;
+  static_assert(sizeof(S) == 2, "16-bit element types");
   const S* bias = (const S*)p.bias;
-  const bool per_row = p.bias_per_row != 0;
-  const float ceiling = p.coef;
   const int r = lane & 31, h = lane >> 5;
-  float brow[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  if (HAS_BIAS) {
+#pragma unroll
+  for (int c = 0; c < 16; ++c) b[c] = u32x2_t{0u, 0u};
+  if (!bias) return;
+  if (p.bias_per_row) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = wave_m0 + 32 * i + r;
-      brow[i] = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+      if (m < p.M) b[i].x = bias[(long long)m * p.sbias];
+    }
+  } else if (p.sbias == 1 && (reinterpret_cast<uintptr_t>(bias) & 7u) == 0) {
+    // N is a multiple of 8 and n of 4: a lane's four columns are all inside or all outside
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const int n = wave_n0 + 8 * c + 4 * h;
+      if (n < p.N) b[c] = *reinterpret_cast<const u32x2_t*>(bias + n);
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      uint32_t v[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int n = wave_n0 + 8 * c + 4 * h + e;
+        if (n < p.N) v[e] = bias[(long long)n * p.sbias];
+      }
+      b[c] = u32x2_t{v[0] | (v[1] << 16), v[2] | (v[3] << 16)};
     }
   }
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      float bcol[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (HAS_BIAS) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
-          bcol[e] = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float x = acc[i][j][4 * g + e];
-          if (HAS_BIAS) x += per_row ? brow[i] : bcol[e];
-          if (CLAMP >= 1) x = __builtin_fmaxf(x, 0.0f);
-          if (CLAMP == 2) x = __builtin_fminf(x, ceiling);
-          acc[i][j][4 * g + e] = x;
-        }
-      }
-    }
 }
 
 // Step 2 (store_tile): one rounding to the element type, then a trip through LDS so that global
@@ -319,10 +319,12 @@ __device__ __forceinline__ uint32_t canonical_nans_bf16x2(uint32_t w) {
   const uint32_t u = (hi & 0x7fffu) > 0x7f80u ? 0x7fffu : hi;
   return l | (u << 16);
 }
-template <typename T>
+template <typename T, bool HAS_BIAS, int CLAMP>
 __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t (&acc)[4][4], int wave_m0, int wave_n0,
-                                           int bz, int lane, uint32_t stage) {
+                                           int bz, int lane, uint32_t stage, const u32x2_t (&b)[16]) {
   using S = typename T::storage;
+  const bool per_row = p.bias_per_row != 0;
+  const float ceiling = p.coef;
   constexpr bool FIXUP = T::dtype == srtReal16BF;   // the fp16 converter already encodes NaNs as required
   S* C = (S*)p.C + (long long)bz * p.scb;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;   // elements spanned by C (< 2^30, checked on the host)
@@ -352,9 +354,24 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t 
           float a0 = acc[i][j][4 * g], a1 = acc[i][j][4 * g + 1], a2 = acc[i][j][4 * g + 2], a3 = acc[i][j][4 * g + 3];
           // one copy out of the accumulator registers, here, for both the test and the conversion
           asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+          const int c = 4 * j + g;
+          if (HAS_BIAS) {
+            const float br = T::to_float((S)(b[i].x & 0xffffu));
+            a0 += per_row ? br : T::to_float((S)(b[c].x & 0xffffu));
+            a1 += per_row ? br : T::to_float((S)(b[c].x >> 16));
+            a2 += per_row ? br : T::to_float((S)(b[c].y & 0xffffu));
+            a3 += per_row ? br : T::to_float((S)(b[c].y >> 16));
+          }
+          if (CLAMP >= 1) {
+            a0 = __builtin_fmaxf(a0, 0.0f); a1 = __builtin_fmaxf(a1, 0.0f);
+            a2 = __builtin_fmaxf(a2, 0.0f); a3 = __builtin_fmaxf(a3, 0.0f);
+          }
+          if (CLAMP == 2) {
+            a0 = __builtin_fminf(a0, ceiling); a1 = __builtin_fminf(a1, ceiling);
+            a2 = __builtin_fminf(a2, ceiling); a3 = __builtin_fminf(a3, ceiling);
+          }
           if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
           const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};
-          const int c = 4 * j + g;
           *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
         }
       }
@@ -448,6 +465,17 @@ constexpr int EPI_RELU = 2;        // relu
 constexpr int EPI_BIAS_RELU = 3;   // bias, relu (the Dense configuration)
 constexpr int EPI_CLIPPED = 4;     // clippedRelu, bias optional (a null bias adds nothing)
 constexpr int EPI_TRANS = 5;       // sigmoid / tanh / elu (+ bias)
+
+template <typename T, int EPI>
+__device__ __forceinline__ void store_tile_linear(const GemmProblem& p, const f32x16_t (&acc)[4][4], int wave_m0,
+                                                  int wave_n0, int bz, int lane, uint32_t stage, const u32x2_t (&b)[16]) {
+  if (EPI == EPI_BIAS) store_tile<T, true, 0>(p, acc, wave_m0, wave_n0, bz, lane, stage, b);
+  else if (EPI == EPI_RELU) store_tile<T, false, 1>(p, acc, wave_m0, wave_n0, bz, lane, stage, b);
+  else if (EPI == EPI_BIAS_RELU) store_tile<T, true, 1>(p, acc, wave_m0, wave_n0, bz, lane, stage, b);
+  else if (EPI == EPI_CLIPPED) store_tile<T, true, 2>(p, acc, wave_m0, wave_n0, bz, lane, stage, b);   // a null bias adds nothing
+  else store_tile<T, false, 0>(p, acc, wave_m0, wave_n0, bz, lane, stage, b);
+}
+
 
 // One tile as the loads see it: the byte offsets of its first row (column) inside the operand
 // tensors, batch offset included.  All scalar.
@@ -726,26 +754,24 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
     // Every load in flight must have landed, in every wave, before the slots vacated last become
     // the staging area (the out-of-range fillers write zeros there); with the overlap on this
     // also covers the next tile's first stages.
+    const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
+    // the epilogue's per-lane address arithmetic starts from a lane id the compiler cannot see
+    // through: otherwise it is hoisted out of the tile loop and held (spilled) across the k loop
+    const int le = lane_id();
+    constexpr bool LINEAR_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED;
+    u32x2_t bias_regs[16];
+    if (LINEAR_BIAS) load_bias<T>(p, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1
     uint32_t pprv = prv - STAGE;
     if (prv == lds) pprv = lds + (NS - 1) * STAGE;
     const uint32_t stage = ((wave & 2) ? prv : pprv) + (uint32_t)(wave & 1) * 16384u;
-    const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
-    // the epilogue's per-lane address arithmetic starts from a lane id the compiler cannot see
-    // through: otherwise it is hoisted out of the tile loop and held (spilled) across the k loop
-    const int le = lane_id();
 
     // ---- epilogue ----
     if (EPI == EPI_TRANS) {
       store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
     } else {
-      if (EPI == EPI_BIAS) apply_linear_epilogue<T, true, 0>(p, acc, em0, en0, le);
-      else if (EPI == EPI_RELU) apply_linear_epilogue<T, false, 1>(p, acc, em0, en0, le);
-      else if (EPI == EPI_BIAS_RELU) apply_linear_epilogue<T, true, 1>(p, acc, em0, en0, le);
-      else if (EPI == EPI_CLIPPED) apply_linear_epilogue<T, true, 2>(p, acc, em0, en0, le);   // a null bias adds nothing
-      if (EPI != EPI_PLAIN) pin_all(acc);   // ends the life of the copies made above
-      store_tile<T>(p, acc, em0, en0, bz, le, stage);
+      store_tile_linear<T, EPI>(p, acc, em0, en0, bz, le, stage, bias_regs);
     }
     if (!has_next) break;
 

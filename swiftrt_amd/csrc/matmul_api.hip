@@ -274,9 +274,8 @@ bool split_for_reach(const GemmProblem& p, GemmProblem* lo, GemmProblem* hi) {
   GemmProblem q = p;
   q.batch = 1; q.M = p.M < 256 ? p.M : 256; q.N = p.N < 256 ? p.N : 256;
   if (!fits_256(q)) return false;   // alignment, or a k walk out of reach: not a matter of extent
-  const size_t es = 2;
-  auto at = [es](const void* base, long long elements) {
-    return static_cast<const void*>(static_cast<const char*>(base) + elements * (long long)es);
+  auto at = [](const void* base, long long elements) {
+    return static_cast<const void*>(static_cast<const char*>(base) + elements * 2);   // 16-bit elements
   };
   *lo = p; *hi = p;
   if (p.batch > 1) {
