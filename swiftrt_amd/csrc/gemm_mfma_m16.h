@@ -779,9 +779,7 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
   const long long tiles = (long long)((p.M + tile_m - 1) / tile_m) * ((p.N + BN - 1) / BN) * p.batch;
-  int grid = ring::compute_units() & ~7;
-  if (grid <= 0) grid = 8;
-  if (tiles < grid) grid = (int)tiles;
+  const int grid = ring::persistent_grid(tiles);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return hipGetLastError();
 }

@@ -816,6 +816,21 @@ inline int compute_units() {
   return n;
 }
 
+// Workgroups of the persistent grid: one per compute unit (a workgroup takes a whole unit's LDS),
+// a multiple of 8 because the XCD-aware tile order wants the stride between a workgroup's tiles
+// to be one -- and, when the tiles do not fill the last round, only as many as spread them evenly
+// over the same number of rounds (688 tiles: 232 workgroups of 3 tiles instead of 176 with 3 and
+// 80 with 2).  Worth 2 % on that shape (276 -> 271 us): units that idle through a ragged last
+// round give nothing back, and fewer units per round contend less for L2 and fabric.
+inline int persistent_grid(long long tiles) {
+  int grid = compute_units() & ~7;
+  if (grid <= 0) grid = 8;
+  if (tiles < grid) return (int)tiles;
+  const long long rounds = (tiles + grid - 1) / grid;
+  const long long even = ((tiles + rounds - 1) / rounds + 7) & ~7LL;
+  return even < grid ? (int)even : grid;
+}
+
 template <typename T, bool A_KC, bool B_KC, int EPI, int NS>
 hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   auto kernel = gemm_ring_kernel<T, A_KC, B_KC, EPI, NS>;
@@ -825,9 +840,7 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   const long long tiles = (long long)((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN) * p.batch;
   // one workgroup per compute unit (a workgroup takes a whole unit's LDS); the XCD-aware tile
   // order wants the stride between a workgroup's tiles to be a multiple of 8
-  int grid = compute_units() & ~7;
-  if (grid <= 0) grid = 8;
-  if (tiles < grid) grid = (int)tiles;
+  const int grid = persistent_grid(tiles);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return hipGetLastError();
 }
