@@ -195,6 +195,7 @@ __global__ __launch_bounds__(NT) void gemm_kc64_kernel(GemmProblem p) {
   u32x2_t bias_regs[16];
   if (LINEAR_BIAS) load_bias<T>(p, m0 + wm0, n0 + wn0, lane, bias_regs);   // lands during the wait below
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  if (LINEAR_BIAS) pin_all(acc);   // no copy out of the accumulators is scheduled ahead of the wait
   const uint32_t stage = lds + (uint32_t)wave * 16384u;
 
   if (EPI == EPI_TRANS) {

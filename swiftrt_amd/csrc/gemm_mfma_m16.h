@@ -88,7 +88,8 @@ __device__ __forceinline__ void mfma16_first<F16>(f32x4_t& acc, const u32x4_t& b
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(acc) : "v"(b), "v"(a));
 }
 
-// Ends the life of the register copies the compiler makes of accumulators (see ring::pin).
+// An empty statement that "rewrites" every accumulator tile: reads of the accumulators that follow it in
+// the source cannot be scheduled ahead of it (see ring::pin).
 template <int TM>
 __device__ __forceinline__ void pin_all(f32x4_t (&acc)[TM][8]) {
 #pragma unroll
@@ -744,6 +745,9 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     u32x2_t bias_regs[8];
     if (LINEAR_BIAS) load_bias<T, TM>(p, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+    // with the bias loads ahead of the wait the compiler pulled every accumulator read up there too: the
+    // accumulators are "rewritten" here so that no read of them is scheduled above the wait states
+    if (LINEAR_BIAS) pin_all<TM>(acc);
     // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1 (half a slot each)
     uint32_t pprv = prv - STAGE_B;
     if (prv == lds) pprv = lds + (NS - 1) * STAGE_B;

@@ -762,6 +762,7 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
     u32x2_t bias_regs[16];
     if (LINEAR_BIAS) load_bias<T>(p, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (LINEAR_BIAS) pin_all(acc);   // no copy out of the accumulators is scheduled ahead of the wait (registers stay free for the bias)
     // staging: waves 0, 1 share the slot of stage KT-2, waves 2, 3 the slot of stage KT-1
     uint32_t pprv = prv - STAGE;
     if (prv == lds) pprv = lds + (NS - 1) * STAGE;
