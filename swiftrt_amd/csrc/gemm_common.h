@@ -99,6 +99,39 @@ __device__ __forceinline__ float apply_activation(int activation, float coef, fl
   }
 }
 
+// The same for results stored in a 16-bit type: the hardware exponential and reciprocal (a few
+// fp32 ulps: 2^-13 of a half's rounding step, 2^-16 of a bfloat16's) instead of libm's expf / tanhf,
+// whose range reduction and branches cost ten times the instructions -- fused into a 256 x 256
+// tile's epilogue, libm's tanh took longer than the whole k loop at K = 4096.  Where the closed
+// forms cancel (tanh and exp(x) - 1 near 0) a short series takes over, so the relative error stays
+// at fp32 rounding level everywhere.  NaN in, NaN out; +-inf give the limits.
+template <int ACT>
+__device__ __forceinline__ float activation16_ct(float coef, float x) {
+  if (ACT == srtActivationSigmoid) return __fdividef(1.0f, 1.0f + __expf(-x));
+  if (ACT == srtActivationTanh) {
+    // tanh|x| = 1 - 2 / (exp(2|x|) + 1): exp overflows to +inf for large |x|, giving exactly 1
+    const float a = fabsf(x), x2 = x * x;
+    const float big = 1.0f - __fdividef(2.0f, __expf(2.0f * a) + 1.0f);
+    const float small = a * (1.0f + x2 * (-0.33333334f + x2 * 0.13333334f));   // next term 17 x^7 / 315
+    return copysignf(a < 0.125f ? small : big, x);
+  }
+  if (ACT == srtActivationElu) {
+    const float x2 = x * x;
+    const float series = x + x2 * (0.5f + x * (0.16666667f + x * (0.041666668f + x * 0.008333334f)));
+    const float em1 = x > -0.125f ? series : __expf(x) - 1.0f;
+    return x > 0.0f ? x : coef * em1;
+  }
+  return x;
+}
+__device__ __forceinline__ float apply_activation_16(int activation, float coef, float x) {
+  switch (activation) {
+    case srtActivationSigmoid: return activation16_ct<srtActivationSigmoid>(coef, x);
+    case srtActivationTanh: return activation16_ct<srtActivationTanh>(coef, x);
+    case srtActivationElu: return activation16_ct<srtActivationElu>(coef, x);
+    default: return apply_activation(activation, coef, x);
+  }
+}
+
 // Same with the activation fixed at compile time: kernels switch on the activation once per
 // workgroup and run an epilogue specialised for it, so the unrolled store code of the common
 // cases (identity, relu) carries no transcendental code and no per-element branches.
@@ -132,7 +165,8 @@ struct Epilogue {
   }
   __device__ __forceinline__ typename T::storage finish(float acc, float b) const {
     float v = acc + b;
-    if (activation != srtActivationIdentity) v = apply_activation(activation, coef, v);
+    if (activation != srtActivationIdentity)
+      v = sizeof(typename T::storage) == 2 ? apply_activation_16(activation, coef, v) : apply_activation(activation, coef, v);
     return T::from_float(v);
   }
 };

@@ -199,7 +199,8 @@ __global__ __launch_bounds__(NT) void gemm_kc64_kernel(GemmProblem p) {
   const uint32_t stage = lds + (uint32_t)wave * 16384u;
 
   if (EPI == EPI_TRANS) {
-    store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage);
+    load_bias<T>(p, m0 + wm0, n0 + wn0, lane, bias_regs);   // one round of latency, before any store is in flight
+    store_tile_transcendental<T>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage, bias_regs);
   } else {
     store_tile_linear<T, EPI>(p, acc, m0 + wm0, n0 + wn0, bz, lane, stage, bias_regs);
   }

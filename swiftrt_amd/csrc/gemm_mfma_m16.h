@@ -342,11 +342,11 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
 // run in a rolled loop.
 template <typename T, int TM>
 __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, const f32x4_t (&acc)[TM][8],
-                                                          int wave_m0, int wave_n0, int bz, int lane, uint32_t stage) {
+                                                          int wave_m0, int wave_n0, int bz, int lane, uint32_t stage,
+                                                          const u32x2_t (&b)[8]) {
   constexpr int ROWS = TM == 8 ? 32 : 16;
   using S = typename T::storage;
   S* C = (S*)p.C + (long long)bz * p.scb;
-  const S* bias = (const S*)p.bias;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
   const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
   const int ldc2 = (int)(p.scm * 2);
@@ -361,35 +361,42 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
     for (int ii = 0; ii < ROWS / 16; ++ii) {
       const int i = (ROWS / 16) * pass + ii;
       const int row = 16 * ii + jn;
-      const int m = wave_m0 + 16 * i + jn;
-      const float brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+      // bias from the registers load_bias filled before the tile's first store was issued: a global load
+      // in here would wait, with its vmcnt(0), for every store of the previous pass as well
+      const float brow = T::to_float((S)(b[i].x & 0xffffu));
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
+        const float bcol[4] = {T::to_float((S)(b[j].x & 0xffffu)), T::to_float((S)(b[j].x >> 16)),
+                               T::to_float((S)(b[j].y & 0xffffu)), T::to_float((S)(b[j].y >> 16))};
         f32x4_t x;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int n = wave_n0 + 16 * j + 4 * g + e;
-          const float bcol = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
-          x[e] = acc[i][j][e] + (per_row ? brow : bcol);
-        }
+        for (int e = 0; e < 4; ++e) x[e] = acc[i][j][e] + (per_row ? brow : bcol[e]);
         const int c = 4 * j + g;
         *reinterpret_cast<SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u + (uint32_t)((c ^ (row & 31)) << 4)) = x;
       }
     }
-#pragma unroll 1
-    for (int it = 0; it < ROWS / 2; ++it) {
-      const int row = rd_row + 2 * it;
-      const f32x4_t x = *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u +
-                                                                  (uint32_t)((rd_chunk ^ (row & 31)) << 4));
-      uint32_t lo = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[0])) |
-                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[1])) << 16);
-      uint32_t hi = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[2])) |
-                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[3])) << 16);
-      const u32x2_t w = {lo, hi};
-      const int mm = wave_m0 + ROWS * pass + row;
-      const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
-      __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, SRT_STORE_AUX);
-    }
+    // the staged values' activation, rounding and store: one copy of the loop per activation, chosen by a
+    // uniform branch (a switch per element inside the loop costs a chain of branches each)
+    auto tail = [&](auto act) __attribute__((always_inline)) {
+      constexpr int ACT = decltype(act)::value;
+#pragma unroll 4
+      for (int it = 0; it < ROWS / 2; ++it) {
+        const int row = rd_row + 2 * it;
+        const f32x4_t x = *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u +
+                                                                    (uint32_t)((rd_chunk ^ (row & 31)) << 4));
+        uint32_t lo = (uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[0])) |
+                      ((uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[1])) << 16);
+        uint32_t hi = (uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[2])) |
+                      ((uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[3])) << 16);
+        const u32x2_t w = {lo, hi};
+        const int mm = wave_m0 + ROWS * pass + row;
+        const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
+        __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, SRT_STORE_AUX);
+      }
+    };
+    if (p.activation == srtActivationSigmoid) tail(std::integral_constant<int, srtActivationSigmoid>{});
+    else if (p.activation == srtActivationTanh) tail(std::integral_constant<int, srtActivationTanh>{});
+    else tail(std::integral_constant<int, srtActivationElu>{});
     // the rolled loop's reads must have returned before the next pass overwrites the area
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
@@ -756,7 +763,8 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
     if (EPI == EPI_PARTIAL) {
       store_tile_partial<TM>(p, acc, em0, en0, bz, le, stage);
     } else if (EPI == EPI_TRANS) {
-      store_tile_transcendental<T, TM>(p, acc, em0, en0, bz, le, stage);
+      load_bias<T, TM>(p, em0, en0, le, bias_regs);   // one round of latency, before any store is in flight
+      store_tile_transcendental<T, TM>(p, acc, em0, en0, bz, le, stage, bias_regs);
     } else {
       if (EPI == EPI_BIAS) store_tile<T, TM, true, 0>(p, acc, em0, en0, bz, le, stage, bias_regs);
       else if (EPI == EPI_RELU) store_tile<T, TM, false, 1>(p, acc, em0, en0, bz, le, stage, bias_regs);

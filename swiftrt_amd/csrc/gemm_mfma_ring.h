@@ -411,10 +411,10 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x16_t 
 // Four passes of 32 rows: staging is [32 rows][32 chunks of 16 B], chunk c of row r at c ^ r.
 template <typename T>
 __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, const f32x16_t (&acc)[4][4],
-                                                          int wave_m0, int wave_n0, int bz, int lane, uint32_t stage) {
+                                                          int wave_m0, int wave_n0, int bz, int lane, uint32_t stage,
+                                                          const u32x2_t (&b)[16]) {
   using S = typename T::storage;
   S* C = (S*)p.C + (long long)bz * p.scb;
-  const S* bias = (const S*)p.bias;
   const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
   const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
   const int ldc2 = (int)(p.scm * 2);
@@ -425,36 +425,44 @@ __device__ __forceinline__ void store_tile_transcendental(const GemmProblem& p, 
   const bool n_rd_ok = n_rd < p.N;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int m = wave_m0 + 32 * i + r;
-    const float brow = (bias && per_row && m < p.M) ? T::to_float(bias[(long long)m * p.sbias]) : 0.0f;
+    // bias from the registers load_bias filled before the tile's first store was issued: a global load in
+    // here would wait, with its vmcnt(0), for every store of the previous pass as well
+    const float brow = T::to_float((S)(b[i].x & 0xffffu));
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        const u32x2_t bw = b[4 * j + g];
+        const float bcol[4] = {T::to_float((S)(bw.x & 0xffffu)), T::to_float((S)(bw.x >> 16)),
+                               T::to_float((S)(bw.y & 0xffffu)), T::to_float((S)(bw.y >> 16))};
         f32x4_t x;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int n = wave_n0 + 32 * j + 8 * g + 4 * h + e;
-          const float bcol = (bias && !per_row && n < p.N) ? T::to_float(bias[(long long)n * p.sbias]) : 0.0f;
-          x[e] = acc[i][j][4 * g + e] + (per_row ? brow : bcol);
-        }
+        for (int e = 0; e < 4; ++e) x[e] = acc[i][j][4 * g + e] + (per_row ? brow : bcol[e]);
         const int c = 8 * j + 2 * g + h;
         *reinterpret_cast<SRT_LDS f32x4_t*>(stage + (uint32_t)r * 512u + (uint32_t)((c ^ r) << 4)) = x;
       }
-#pragma unroll 1
-    for (int it = 0; it < 16; ++it) {
-      const int row = rd_row + 2 * it;
-      const f32x4_t x =
-          *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u + (uint32_t)((rd_chunk ^ row) << 4));
-      uint32_t lo = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[0])) |
-                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[1])) << 16);
-      uint32_t hi = (uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[2])) |
-                    ((uint32_t)T::from_float(apply_activation(p.activation, p.coef, x[3])) << 16);
-      const u32x2_t w = {lo, hi};
-      const int mm = wave_m0 + 32 * i + row;
-      const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
-      __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, SRT_STORE_AUX);
-    }
+    // the staged values' activation, rounding and store: one copy of the loop per activation, chosen by a
+    // uniform branch (a switch per element inside the loop costs a chain of branches each)
+    auto tail = [&](auto act) __attribute__((always_inline)) {
+      constexpr int ACT = decltype(act)::value;
+#pragma unroll 4
+      for (int it = 0; it < 16; ++it) {
+        const int row = rd_row + 2 * it;
+        const f32x4_t x =
+            *reinterpret_cast<const SRT_LDS f32x4_t*>(stage + (uint32_t)row * 512u + (uint32_t)((rd_chunk ^ row) << 4));
+        uint32_t lo = (uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[0])) |
+                      ((uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[1])) << 16);
+        uint32_t hi = (uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[2])) |
+                      ((uint32_t)T::from_float(activation16_ct<ACT>(p.coef, x[3])) << 16);
+        const u32x2_t w = {lo, hi};
+        const int mm = wave_m0 + 32 * i + row;
+        const uint32_t off = (n_rd_ok && mm < p.M) ? (uint32_t)(mm * ldc2 + n_rd * 2) : OOB;
+        __builtin_amdgcn_raw_buffer_store_b64(w, rc, (int)off, 0, SRT_STORE_AUX);
+      }
+    };
+    if (p.activation == srtActivationSigmoid) tail(std::integral_constant<int, srtActivationSigmoid>{});
+    else if (p.activation == srtActivationTanh) tail(std::integral_constant<int, srtActivationTanh>{});
+    else tail(std::integral_constant<int, srtActivationElu>{});
   }
 }
 
@@ -770,7 +778,8 @@ __global__ __launch_bounds__(NT) void gemm_ring_kernel(GemmProblem p) {
 
     // ---- epilogue ----
     if (EPI == EPI_TRANS) {
-      store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage);
+      load_bias<T>(p, em0, en0, le, bias_regs);   // one round of latency, before any store is in flight
+      store_tile_transcendental<T>(p, acc, em0, en0, bz, le, stage, bias_regs);
     } else {
       store_tile_linear<T, EPI>(p, acc, em0, en0, bz, le, stage, bias_regs);
     }
