@@ -39,12 +39,9 @@ struct SigmoidFast {
   static __device__ __forceinline__ float apply(float a, float) { return __fdividef(1.0f, 1.0f + __expf(-a)); }
 };
 struct TanhFast {
-  // tanh(a) = sign(a) (1 - 2 / (exp(2|a|) + 1)); exp overflows to +inf for large |a|, giving exactly 1
-  static __device__ __forceinline__ float apply(float a, float) {
-    const float e = __expf(2.0f * fabsf(a));
-    const float t = 1.0f - __fdividef(2.0f, e + 1.0f);
-    return copysignf(t, a);
-  }
+  // 1 - 2 / (exp(2|a|) + 1) away from 0, a short series below 0.125 where that form cancels
+  // (at a = 1e-6 it is 6 % off, 15 rounding steps of a bfloat16)
+  static __device__ __forceinline__ float apply(float a, float) { return srt::activation16_ct<srtActivationTanh>(0.0f, a); }
 };
 struct Copy { static __device__ __forceinline__ float apply(float a, float) { return a; } };
 

@@ -27,10 +27,10 @@ def rand_storage(g, shape, dt, scale=2.0):
     return H.encode((g.standard_normal(shape) * scale).astype(np.float32), dt)
 
 
-def close_transcendental(got_st, want_st, dt):
+def close_transcendental(got_st, want_st, dt, floor=1e-7):
     got, want = H.decode(got_st).astype(np.float64), H.decode(want_st).astype(np.float64)
     tol = 2 * (2.0 ** -23 if dt == H.F32 else 2 * H.ULP[dt])
-    return np.all(np.abs(got - want) <= tol * np.abs(want) + 1e-7)
+    return np.all(np.abs(got - want) <= tol * np.abs(want) + floor)
 
 
 # ---- tensor-tensor, dense: the vector path --------------------------------------------------------
@@ -118,6 +118,9 @@ def test_transcendentals(op, dt):
     a_st = rand_storage(g, (48, 160), dt, scale=3.0)
     got = getattr(srt, op)(srt.Tensor(a_st)).array()
     assert close_transcendental(got, ora.elementwise(op, a_st), dt)
+    # small arguments, where 1 - 2 / (exp(2a) + 1) and 1 / (1 + exp(-a)) - 1/2 lose their digits
+    tiny = H.encode((np.logspace(-9, -0.5, 512) * np.where(np.arange(512) % 2, -1.0, 1.0)).astype(np.float32).reshape(8, 64), dt)
+    assert close_transcendental(getattr(srt, op)(srt.Tensor(tiny)).array(), ora.elementwise(op, tiny), dt, floor=1e-12)
     # closed forms on exact inputs
     z = H.encode(np.zeros((1, 8), np.float32), dt)
     want = {"exp": 1.0, "sigmoid": 0.5, "tanh": 0.0}[op]
