@@ -1018,3 +1018,35 @@ def test_fp32_operand_beyond_4_gib_vs_exact():
     got = gpu_matmul(_periodic(a0, reps, 0), b)
     block = (a0.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
     assert np.array_equal(got, np.concatenate([block] * reps, 0))
+
+
+# ---- fused sigmoid / tanh / elu near zero -----------------------------------------------------------
+@pytest.mark.parametrize("dt", [H.F16, H.BF16])
+@pytest.mark.parametrize("act", [srt.ActivationType.sigmoid, srt.ActivationType.tanh, srt.ActivationType.elu])
+@pytest.mark.parametrize("plan,M,N", [(None, 64, 96), ("mfma_256x256_m16", 512, 512), ("mfma_256x256", 512, 512)])
+def test_fused_transcendentals_keep_their_digits_near_zero(act, dt, plan, M, N, tmp_path):
+    """Pre-activations from 1e-7 to 0.4 in magnitude, both signs (K = 8 with a single non-zero term, so the
+    accumulator is exact): the fused epilogues use the hardware exponential, whose closed forms for tanh and
+    exp(x) - 1 cancel near 0; every result must be within two rounding steps of the stored type, relative."""
+    K = 8
+    mags = np.logspace(-7, -0.4, N) * np.where(np.arange(N) % 2, -1.0, 1.0)
+    x = np.zeros((M, K), np.float32)
+    x[:, 0] = np.exp2(-(np.arange(M) % 12)).astype(np.float32)          # row scales, exact powers of two
+    w = np.zeros((K, N), np.float32)
+    w[0] = mags
+    xs, ws = H.encode(x, dt), H.encode(w, dt)
+    if plan is not None:
+        pin_plan_for_shape(tmp_path, plan, dt, M, N, K)
+    xt, wt = srt.Tensor(xs), srt.Tensor(ws)
+    out = srt.Tensor(shape=[M, N], dtype=xs.dtype)
+    srt.current_queue().matmul(xt, False, wt, False, out, activation=act, coef=1.0)
+    if plan is not None:
+        assert query_kernel(xt, False, wt, False, out) == plan
+    got = H.decode(out.array()).astype(np.float64)
+    pre = H.decode(xs)[:, :1].astype(np.float64) * H.decode(ws)[:1].astype(np.float64)     # exact in fp32
+    want = {srt.ActivationType.sigmoid: lambda v: 1.0 / (1.0 + np.exp(-v)),
+            srt.ActivationType.tanh: np.tanh,
+            srt.ActivationType.elu: lambda v: np.where(v > 0, v, np.expm1(v))}[act](pre)
+    floor = 2.0 ** -24 if dt == H.F16 else 1e-30          # a half's subnormal step
+    assert np.all(np.abs(got - want) <= 2 * H.ULP[dt] * np.abs(want) + floor)
+    srt.PlanCache.clear()
