@@ -1,24 +1,31 @@
 #!/usr/bin/env python3
 """Benchmark of the matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-configs] [--no-cpu] [--no-ceiling]
 
 A step is one bf16 GEMM C = A.B with M = N = K = 8192 (row-major, no transposes, fp32
 accumulation, bf16 output) -- the configuration the headline metric is quoted on -- launched
-through the C ABI (srtMatmul) on the library's own stream, inputs resident in HBM.
+through the C ABI (srtMatmulBiasActivation) on the library's own stream, inputs resident in HBM.
 Inputs: A, B ~ N(0,1)/sqrt(K), seed 2 (Philox), rounded once to bf16.
 
-Prints ONE JSON line on stdout.  `value` is TFLOP/s over the K timed steps (wall clock between
-two stream synchronisations); `roofline.achieved` uses the average kernel duration measured
-with events recorded on the stream the kernel runs on.  `cpu_baseline` times the CPU oracle
-(the restated reference cpu_matmul, one thread) on a slab of rows of the same problem.
---all additionally reports the other configurations (transposed lhs, Dense, skinny, batched
-fp16, fp32) on stderr.
+Protocol: a time-bounded settle phase of the same launch (an idle device raises its clocks over a few
+hundred milliseconds of load; reported as `settle_launches` / `settle_ms`, never counted), then W
+untimed warm-up steps, then exactly K timed steps between two stream synchronisations.
+
+Prints ONE JSON line on stdout.  `value` is TFLOP/s over the K timed steps (wall clock);
+`roofline.achieved` uses the average kernel duration measured with events recorded on the stream
+the kernel runs on, over the same K steps; `launch_ms` gives min / median / max per launch from a
+second pass with an event after every launch.  `configs` lists the other configurations
+(transposed lhs, Dense, skinny M = 1 / 8 / 32, batched fp16, fp32, and the element-wise neighbours of
+the Dense layer at its shape), each settled and timed the same
+way with its own bound and roofline fraction.  `cpu_baseline` times the CPU oracle (the restated
+reference cpu_matmul, one thread) on a slab of rows of the headline problem.
 """
 import argparse
 import ctypes
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -29,9 +36,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# and scaled by a 256 MiB device copy (profiles/gemm_m16_bf16_8192_counters.txt).
-TRAFFIC_BYTES_8192 = 1.799e9   # 2.000 x FETCH_SIZE (812 824 KiB) + 1.000 x WRITE_SIZE (131 117 KiB)
+# HBM-side bytes per launch of the headline kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled
+# by a device copy of known size; the file names the kernel it was measured on
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "gemm_bf16_8192_traffic.txt")
 
 
 def rng(seed):
@@ -49,40 +56,66 @@ def bf16_decode(h):
     return (h.astype(np.uint32) << 16).view(np.float32)
 
 
-class Timer:
-    """Event pair on a queue's stream."""
-
-    def __init__(self, queue):
-        self.q = queue
-
-    def run(self, fn, steps):
-        start = self.q.record_event(timing=True)
-        for i in range(steps):
-            fn(i)
-        stop = self.q.record_event(timing=True)
-        stop.wait()
-        return stop.elapsed_ms_since(start)
+def event_ms(q, fn, launches, first=0):
+    """Elapsed time of `launches` back-to-back calls, between two events on the queue's stream."""
+    start = q.record_event(timing=True)
+    for i in range(launches):
+        fn(first + i)
+    stop = q.record_event(timing=True)
+    stop.wait()
+    return stop.elapsed_ms_since(start)
 
 
-def time_steps(queue, fn, steps, warmup):
-    for i in range(warmup):
-        fn(i)
-    queue.wait_for_completion()
+def settle(q, fn, budget_s=1.0, group=10):
+    """Runs groups of `group` launches until three consecutive group averages agree to 1 % or the
+    time budget is spent.  Returns (launches, elapsed ms, last group average in ms)."""
     t0 = time.perf_counter()
-    ev_ms = Timer(queue).run(fn, steps)
-    queue.wait_for_completion()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    return wall_ms, ev_ms
+    avgs, launches = [], 0
+    while True:
+        avgs.append(event_ms(q, fn, group, launches) / group)
+        launches += group
+        if len(avgs) >= 3:
+            lo, hi = min(avgs[-3:]), max(avgs[-3:])
+            if hi <= 1.01 * lo:
+                break
+        if time.perf_counter() - t0 >= budget_s:
+            break
+    return launches, (time.perf_counter() - t0) * 1e3, avgs[-1]
+
+
+def per_launch_ms(q, fn, launches):
+    """Per-launch durations from an event after every launch (the events add a little to each)."""
+    events = [q.record_event(timing=True)]
+    for i in range(launches):
+        fn(i)
+        events.append(q.record_event(timing=True))
+    events[-1].wait()
+    return [events[i + 1].elapsed_ms_since(events[i]) for i in range(launches)]
+
+
+def read_traffic(kernel_name):
+    """roofline.traffic: the measured HBM-side bytes per launch, or None when the kernel that ran is not
+    the one the figure was measured on."""
+    try:
+        fields = {}
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if ":" in line and not line.startswith("#"):
+                    k, v = line.split(":", 1)
+                    fields[k.strip()] = v.strip()
+        if fields.get("kernel") != kernel_name:
+            return None
+        return float(fields["traffic_bytes"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=300,
-                    help="untimed launches before the timed ones; the memory and fabric clocks of an idle device take "
-                         "a few hundred milliseconds of load to settle (10 warm-up launches read 3 %% low)")
-    ap.add_argument("--all", action="store_true", help="also report the other configurations on stderr")
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-configs", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the register-only MFMA loop that measures what the matrix cores sustain on this "
@@ -90,6 +123,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three 256 MiB device-to-device copies (known traffic, for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--only", default=None,
+                    help="run one configuration alone, a few launches, and exit (for profilers): headline, cfg3_tn, "
+                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, dense_backward, add, add_bias, tanh, cast")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the single-GPU matmul path; run it with --gpus 1 "
@@ -109,46 +145,66 @@ def main():
         print(json.dumps({"copy_calibration_bytes": nbytes, "copies": 3}))
         return
     props = srt.HipPlatform.local().devices[1].properties
+    bench = Bench(srt, native, q)
+
+    if args.only:
+        name = args.only
+        cfg = bench.headline() if name == "headline" else bench.secondary(name)
+        for i in range(args.warmup + args.steps):
+            cfg["call"](i)
+        q.wait_for_completion()
+        print(json.dumps({"only": name, "launches": args.warmup + args.steps, "kernel": cfg["kernel"]}))
+        return
+
+    head = bench.headline()
+    step = head["call"]
     n = 8192
+    settle_launches, settle_ms, _ = settle(q, step)
+    for i in range(args.warmup):
+        step(i)
+    q.wait_for_completion()
+    t0 = time.perf_counter()
+    ev_ms = event_ms(q, step, args.steps)
+    q.wait_for_completion()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    launches = per_launch_ms(q, step, min(args.steps, 100))
 
-    g = rng(2)
-    a_st = bf16_encode(g.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n)))
-    b_st = bf16_encode(g.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n)))
-    a, b = srt.Tensor(a_st), srt.Tensor(b_st)
-    c = srt.Tensor(shape=[n, n], dtype=np.uint16)
-    a.device_read(q), b.device_read(q), c.device_read_write(q)
-
-    def step(_i):
-        q.matmul(a, False, b, False, c)
-
-    wall_ms, ev_ms = time_steps(q, step, args.steps, args.warmup)
-    flops = 2.0 * n * n * n
+    flops = head["flops"]
     ms_per_step = wall_ms / args.steps
     kernel_ms = ev_ms / args.steps
     value = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (kernel_ms * 1e-3) / 1e12
 
     # parity spot check of what was just timed: sampled rows against the fp64 GEMM
-    got = c.array()
+    got = head["out"].array()
     rows = np.arange(0, n, 1024)
-    c64 = bf16_decode(a_st[rows]).astype(np.float64) @ bf16_decode(b_st).astype(np.float64)
+    c64 = bf16_decode(head["a_st"][rows]).astype(np.float64) @ bf16_decode(head["b_st"]).astype(np.float64)
     max_rel = float(np.max(np.abs(bf16_decode(got[rows]).astype(np.float64) - c64)) / np.max(np.abs(c64)))
     if not max_rel <= 2e-2:
         sys.exit(f"parity check failed: max-norm relative error {max_rel} > 2e-2")
 
+    name = props.name.decode() or props.archName.decode()
     result = {
         "metric": "bf16 GEMM TFLOP/s (8192^3, 1 MI355X)", "value": round(value, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=8192, row-major, no transposes, fp32 accumulate, bf16 out; "
                                "A,B ~ N(0,1)/sqrt(K) seed 2; inputs resident in HBM",
-                   "entry_point": "srtMatmul", "kernel": "gemm_m16_kernel<BF16> 256x256x32, v_mfma_f32_16x16x32, 5-stage LDS ring, persistent (one workgroup per CU)"},
+                   "entry_point": "srtMatmulBiasActivation", "kernel": head["kernel"]},
+        "settle_launches": settle_launches, "settle_ms": round(settle_ms, 1),
+        "launch_ms": {"mean": round(kernel_ms, 5), "min": round(min(launches), 5),
+                      "median": round(statistics.median(launches), 5), "max": round(max(launches), 5),
+                      "note": "mean: event pair around the timed steps; min / median / max: a second pass with an "
+                              "event after every launch"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": TRAFFIC_BYTES_8192},
+                     "frac": round(achieved / PEAK_TFLOPS["bf16"], 4), "traffic": read_traffic(head["kernel"])},
         "max_rel_err_vs_fp64": max_rel,
-        "device": {"name": props.name.decode(), "arch": props.archName.decode(), "cus": props.multiProcessorCount,
+        "device": {"name": name, "arch": props.archName.decode(), "cus": props.multiProcessorCount,
                    "peak_clock_mhz": props.clockRateKHz // 1000},
     }
+
+    if not args.no_configs:
+        result["configs"] = bench.run_secondary()
 
     if not args.no_ceiling:
         q.wait_for_completion()
@@ -158,12 +214,178 @@ def main():
             result["roofline"]["frac_of_sustained"] = round(achieved / ceiling["normal_operands"]["tflops"], 4)
 
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(a_st, b_st, n)
-
-    if args.all:
-        report_other_configs(srt, q, a_st, b_st, n, args)
+        result["cpu_baseline"] = cpu_baseline(head["a_st"], head["b_st"], n)
 
     print(json.dumps(result), flush=True)
+
+
+class Bench:
+    """The configurations, each as one prepared foreign call per step."""
+
+    SECONDARY = ("cfg3_tn", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1")
+
+    def __init__(self, srt, native, q):
+        self.srt, self.native, self.q = srt, native, q
+        self._head = None
+
+    def prepared(self, a, ta, b, tb, out, bias=None, act=None):
+        """One matmul with descriptors and pointers marshalled once, so that the per-step host cost is a
+        single foreign call (the small configurations finish faster than Python can build descriptors).
+        Returns (call, kernel name)."""
+        srt, native, q = self.srt, self.native, self.q
+        act = srt.ActivationType.identity if act is None else act
+        ptrs = [a.device_read(q), b.device_read(q), out.device_read_write(q)]
+        descs = [t.descriptor() for t in (a, b, out)]
+        bptr = bias.device_read(q) if bias is not None else None
+        bdesc = bias.descriptor() if bias is not None else (None, None)
+        fn = native.lib().srtMatmulBiasActivation
+        argv = (ptrs[0], ctypes.byref(descs[0][0]), int(ta), ptrs[1], ctypes.byref(descs[1][0]), int(tb),
+                bptr, ctypes.byref(bdesc[0]) if bias is not None else None, int(act), 0.0,
+                ptrs[2], ctypes.byref(descs[2][0]), q.stream)
+
+        def call(_i):
+            native.check(fn(*argv))
+        call.keep = (descs, bdesc)
+        buf = ctypes.create_string_buffer(64)
+        native.check(native.lib().srtMatmulQueryKernel(ctypes.byref(descs[0][0]), int(ta), ctypes.byref(descs[1][0]),
+                                                       int(tb), ctypes.byref(descs[2][0]), ptrs[0], ptrs[1], ptrs[2],
+                                                       buf, 64))
+        return call, buf.value.decode()
+
+    def headline(self):
+        if self._head is None:
+            srt, q = self.srt, self.q
+            n = 8192
+            g = rng(2)
+            a_st = bf16_encode(g.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n)))
+            b_st = bf16_encode(g.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n)))
+            a, b = srt.Tensor(a_st), srt.Tensor(b_st)
+            c = srt.Tensor(shape=[n, n], dtype=np.uint16)
+            call, kernel = self.prepared(a, False, b, False, c)
+            self._head = {"call": call, "kernel": kernel, "flops": 2.0 * n ** 3, "bytes": 3 * n * n * 2,
+                          "a_st": a_st, "b_st": b_st, "a": a, "b": b, "out": c}
+        return self._head
+
+    def secondary(self, name):
+        """Builds one secondary configuration: call, kernel, flops, algorithmic bytes, bound, peak key."""
+        srt, q = self.srt, self.q
+        if name == "cfg3_tn":
+            h = self.headline()
+            n = 8192
+            at = srt.Tensor(np.ascontiguousarray(h["a_st"].T))
+            c = srt.Tensor(shape=[n, n], dtype=np.uint16)
+            call, kernel = self.prepared(at, True, h["b"], False, c)
+            return {"name": "cfg3 bf16 8192^3 transposeLhs", "call": call, "kernel": kernel, "flops": 2.0 * n ** 3,
+                    "bytes": 3 * n * n * 2, "bound": "mfma", "dtype": "bf16", "steps": 40}
+        if name == "cfg4_dense":
+            g = rng(3)
+            x = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))
+            w = srt.Tensor(bf16_encode(g.standard_normal((4096, 11008), dtype=np.float32) / np.float32(64)))
+            bias = srt.Tensor(bf16_encode(g.uniform(-0.1, 0.1, 11008).astype(np.float32)))
+            y = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+            call, kernel = self.prepared(x, False, w, False, y, bias=bias, act=srt.ActivationType.relu)
+            return {"name": "cfg4 Dense bf16 4096x4096x11008 +bias +relu", "call": call, "kernel": kernel,
+                    "flops": 2.0 * 4096 * 4096 * 11008, "bytes": (4096 * 4096 + 4096 * 11008 * 2 + 11008) * 2,
+                    "bound": "mfma", "dtype": "bf16", "steps": 100}
+        if name.startswith("cfg5_m"):
+            m = int(name[6:])
+            g = rng(4)
+            # four weight buffers in rotation so that the weight is not served from the last-level cache
+            wbase = bf16_encode(g.standard_normal((14336, 4096), dtype=np.float32) / np.float32(64))
+            ws = [srt.Tensor(wbase.copy()) for _ in range(4)]
+            xs = srt.Tensor(bf16_encode(g.standard_normal((m, 4096), dtype=np.float32)))
+            o = srt.Tensor(shape=[m, 14336], dtype=np.uint16)
+            prepared = [self.prepared(xs, False, w_, True, o) for w_ in ws]
+            calls = [p[0] for p in prepared]
+            return {"name": f"cfg5 skinny bf16 M={m} K=4096 N=14336 transposeRhs", "call": lambda i: calls[i % 4](i),
+                    "kernel": prepared[0][1], "flops": 2.0 * m * 4096 * 14336,
+                    "bytes": 2 * (m * 4096 + 14336 * 4096 + m * 14336), "bound": "hbm", "dtype": "bf16", "steps": 200,
+                    "keep": (ws, calls)}
+        if name == "cfg2":
+            g = rng(1)
+            a2 = srt.Tensor((g.standard_normal((32, 256, 256)) * 0.1).astype(np.float16))
+            b2 = srt.Tensor((g.standard_normal((32, 256, 256)) * 0.1).astype(np.float16))
+            c2 = srt.Tensor(shape=[32, 256, 256], dtype=np.float16)
+            call, kernel = self.prepared(a2, False, b2, True, c2)
+            return {"name": "cfg2 fp16 batch 32 x 256^3 transposeRhs", "call": call, "kernel": kernel,
+                    "flops": 2.0 * 32 * 256 ** 3, "bytes": 32 * 3 * 256 * 256 * 2, "bound": "mfma", "dtype": "f16",
+                    "steps": 200}
+        if name == "cfg1":
+            g = rng(0)
+            a1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
+            b1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
+            c1 = srt.Tensor(shape=[512, 512], dtype=np.float32)
+            call, kernel = self.prepared(a1, False, b1, False, c1)
+            return {"name": "cfg1 fp32 512^3", "call": call, "kernel": kernel, "flops": 2.0 * 512 ** 3,
+                    "bytes": 3 * 512 * 512 * 4, "bound": "mfma", "dtype": "f32", "steps": 200}
+        if name in self.NEIGHBOURS:
+            return self.neighbour(name)
+        raise SystemExit(f"unknown configuration {name}")
+
+    NEIGHBOURS = ("dense_backward", "add", "add_bias", "tanh", "cast")
+
+    def neighbour(self, name):
+        """The element-wise neighbours of the Dense layer at its shape (bandwidth-bound; bytes = what each must
+        move once).  Two buffer sets in rotation: 3 x 90 MB per call would otherwise partly live in the
+        last-level cache."""
+        srt, q = self.srt, self.q
+        if not hasattr(self, "_nb"):
+            m_, n_ = 4096, 11008
+            g = rng(5)
+            self._nb = {
+                "ys": [srt.Tensor(bf16_encode(np.maximum(g.standard_normal((m_, n_), dtype=np.float32), 0))) for _ in range(2)],
+                "dys": [srt.Tensor(bf16_encode(g.standard_normal((m_, n_), dtype=np.float32))) for _ in range(2)],
+                "outs": [srt.Tensor(shape=[m_, n_], dtype=np.uint16) for _ in range(2)],
+                "db": srt.Tensor(shape=[n_], dtype=np.uint16),
+                "bias": srt.Tensor(bf16_encode(g.uniform(-0.1, 0.1, n_).astype(np.float32))),
+                "f32out": srt.Tensor(shape=[m_, n_], dtype=np.float32)}
+        nb = self._nb
+        ys, dys, outs, db = nb["ys"], nb["dys"], nb["outs"], nb["db"]
+        m_, n_ = 4096, 11008
+        e = m_ * n_ * 2
+        relu = srt.ActivationType.relu
+        if name == "dense_backward":
+            call, nbytes = (lambda i: q.activation_backward(ys[i % 2], dys[i % 2], relu, 0.0, outs[i % 2], db)), 3 * e + n_ * 2
+            label, kernel = "Dense backward epilogue bf16 4096x11008: dz = dy*relu'(y), dbias (fused)", "activation_backward"
+        elif name == "add":
+            call, nbytes = (lambda i: q.add(ys[i % 2], dys[i % 2], outs[i % 2])), 3 * e
+            label, kernel = "add bf16 4096x11008 (dense, tensor + tensor)", "map"
+        elif name == "add_bias":
+            bias_row = srt.Tensor.repeating(nb["bias"], (m_, n_))
+            call, nbytes = (lambda i: q.add(ys[i % 2], bias_row, outs[i % 2])), 2 * e + n_ * 2
+            label, kernel = "add bf16 4096x11008 + bias[11008] (stride-0 broadcast)", "map"
+        elif name == "tanh":
+            call, nbytes = (lambda i: q.tanh(ys[i % 2], outs[i % 2])), 2 * e
+            label, kernel = "tanh bf16 4096x11008", "map"
+        else:
+            call, nbytes = (lambda i: q.copy(ys[i % 2], nb["f32out"])), e + 2 * e
+            label, kernel = "cast bf16 -> fp32 4096x11008", "map"
+        return {"name": label, "call": call, "kernel": kernel, "flops": 0.0, "bytes": nbytes, "bound": "hbm",
+                "dtype": "bf16", "steps": 40}
+
+    def run_secondary(self):
+        out = []
+        for name in self.SECONDARY + self.NEIGHBOURS:
+            cfg = self.secondary(name)
+            call, steps = cfg["call"], cfg["steps"]
+            settle_launches, settle_ms, _ = settle(self.q, call, budget_s=0.5)
+            groups = [event_ms(self.q, call, steps // 5, g * (steps // 5)) / (steps // 5) for g in range(5)]
+            ms = statistics.median(groups)
+            tflops = cfg["flops"] / (ms * 1e-3) / 1e12
+            gbs = cfg["bytes"] / (ms * 1e-3) / 1e9
+            entry = {"name": cfg["name"], "kernel": cfg["kernel"], "ms": round(ms, 5), "ms_min": round(min(groups), 5),
+                     "launches": 5 * (steps // 5), "settle_launches": settle_launches, "tflops": round(tflops, 2),
+                     "algorithmic_gbs": round(gbs, 1), "bound": cfg["bound"]}
+            if cfg["bound"] == "hbm":
+                entry.update({"achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                              "frac": round(gbs / PEAK_HBM_GBS, 4)})
+            else:
+                peak = PEAK_TFLOPS[cfg["dtype"]]
+                entry.update({"achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",
+                              "frac": round(tflops / peak, 4)})
+            out.append(entry)
+            del cfg
+        return out
 
 
 def mfma_ceiling():
@@ -214,122 +436,6 @@ def cpu_baseline(a_st, b_st, n):
     dt2 = time.perf_counter() - t0
     out["host_blas_fp32_tflops"] = round(2.0 * m * n * n / dt2 / 1e12, 4)
     return out
-
-
-def report_other_configs(srt, q, a_st, b_st, n, args):
-    """Secondary configurations, human-readable on stderr."""
-    from swiftrt_amd import native
-
-    def line(name, ms, flops, nbytes, peak_key):
-        tf = flops / (ms * 1e-3) / 1e12
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        print(f"[bench] {name}: {ms * 1e3:.1f} us  {tf:.1f} TFLOP/s ({100 * tf / PEAK_TFLOPS[peak_key]:.1f}% of "
-              f"{peak_key} MFMA peak)  {gbs:.0f} GB/s algorithmic ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM peak)",
-              file=sys.stderr, flush=True)
-
-    def timed(fn, steps=args.steps, warmup=args.warmup):
-        _, ev = time_steps(q, fn, steps, warmup)
-        return ev / steps
-
-    def prepared(a, ta, b, tb, out, bias=None, act=srt.ActivationType.identity):
-        """One matmul with descriptors and pointers marshalled once, so that the per-step host cost is
-        a single foreign call (the small configurations finish faster than Python can build descriptors)."""
-        ptrs = [a.device_read(q), b.device_read(q), out.device_read_write(q)]
-        descs = [t.descriptor() for t in (a, b, out)]
-        bptr = bias.device_read(q) if bias is not None else None
-        bdesc = bias.descriptor() if bias is not None else (None, None)
-        fn = native.lib().srtMatmulBiasActivation
-        argv = (ptrs[0], ctypes.byref(descs[0][0]), int(ta), ptrs[1], ctypes.byref(descs[1][0]), int(tb),
-                bptr, ctypes.byref(bdesc[0]) if bias is not None else None, int(act), 0.0,
-                ptrs[2], ctypes.byref(descs[2][0]), q.stream)
-
-        def call(_i):
-            native.check(fn(*argv))
-        call.keep = (descs, bdesc)
-        return call
-
-    # cfg3 with transposeLhs: A stored K x M
-    at = srt.Tensor(np.ascontiguousarray(a_st.T))
-    b = srt.Tensor(b_st)
-    c = srt.Tensor(shape=[n, n], dtype=np.uint16)
-    at.device_read(q), b.device_read(q), c.device_read_write(q)
-    line("cfg3 bf16 8192^3 transposeLhs", timed(prepared(at, True, b, False, c)), 2.0 * n ** 3, 3 * n * n * 2, "bf16")
-    del at, c
-
-    # cfg4 Dense
-    g = rng(3)
-    x = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))
-    w = srt.Tensor(bf16_encode(g.standard_normal((4096, 11008), dtype=np.float32) / np.float32(64)))
-    bias = srt.Tensor(bf16_encode(g.uniform(-0.1, 0.1, 11008).astype(np.float32)))
-    y = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
-    for t in (x, w, bias):
-        t.device_read(q)
-    y.device_read_write(q)
-    line("cfg4 Dense bf16 4096x4096x11008 +bias +relu",
-         timed(prepared(x, False, w, False, y, bias=bias, act=srt.ActivationType.relu)),
-         2.0 * 4096 * 4096 * 11008, (4096 * 4096 + 4096 * 11008 * 2 + 11008) * 2, "bf16")
-    del x, w, y
-
-    # cfg5 skinny: rotate 4 weight buffers so the weight is not served from the last-level cache
-    g = rng(4)
-    wbase = bf16_encode(g.standard_normal((14336, 4096), dtype=np.float32) / np.float32(64))
-    ws = [srt.Tensor(wbase.copy()) for _ in range(4)]
-    for t in ws:
-        t.device_read(q)
-    for m in (1, 8, 32):
-        xs = srt.Tensor(bf16_encode(g.standard_normal((m, 4096), dtype=np.float32)))
-        o = srt.Tensor(shape=[m, 14336], dtype=np.uint16)
-        xs.device_read(q), o.device_read_write(q)
-        calls = [prepared(xs, False, w_, True, o) for w_ in ws]
-        line(f"cfg5 skinny bf16 M={m} K=4096 N=14336 transposeRhs",
-             timed(lambda i: calls[i % 4](i), steps=200, warmup=20),
-             2.0 * m * 4096 * 14336, 2 * (m * 4096 + 14336 * 4096 + m * 14336), "bf16")
-    del ws
-
-    # cfg2 batched fp16
-    g = rng(1)
-    a2 = srt.Tensor((g.standard_normal((32, 256, 256)) * 0.1).astype(np.float16))
-    b2 = srt.Tensor((g.standard_normal((32, 256, 256)) * 0.1).astype(np.float16))
-    c2 = srt.Tensor(shape=[32, 256, 256], dtype=np.float16)
-    a2.device_read(q), b2.device_read(q), c2.device_read_write(q)
-    line("cfg2 fp16 batch 32 x 256^3 transposeRhs", timed(prepared(a2, False, b2, True, c2), steps=200, warmup=20),
-         2.0 * 32 * 256 ** 3, 32 * 3 * 256 * 256 * 2, "f16")
-
-    # cfg1 fp32
-    g = rng(0)
-    a1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
-    b1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
-    c1 = srt.Tensor(shape=[512, 512], dtype=np.float32)
-    a1.device_read(q), b1.device_read(q), c1.device_read_write(q)
-    line("cfg1 fp32 512^3", timed(prepared(a1, False, b1, False, c1), steps=200, warmup=20),
-         2.0 * 512 ** 3, 3 * 512 * 512 * 4, "f32")
-    del a1, b1, c1, a2, b2, c2
-
-    # the neighbours of the Dense layer at its shape (bandwidth-bound: bytes = what each must move once)
-    def bw_line(name, ms, nbytes):
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        print(f"[bench] {name}: {ms * 1e3:.1f} us  {gbs:.0f} GB/s algorithmic ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM "
-              f"peak)", file=sys.stderr, flush=True)
-
-    m_, n_ = 4096, 11008
-    g = rng(5)
-    e = m_ * n_ * 2
-    ys = [srt.Tensor(bf16_encode(np.maximum(g.standard_normal((m_, n_), dtype=np.float32), 0))) for _ in range(2)]
-    dys = [srt.Tensor(bf16_encode(g.standard_normal((m_, n_), dtype=np.float32))) for _ in range(2)]
-    outs = [srt.Tensor(shape=[m_, n_], dtype=np.uint16) for _ in range(2)]
-    db = srt.Tensor(shape=[n_], dtype=np.uint16)
-    # two buffer sets in rotation: 3 x 90 MB per call would otherwise partly live in the last-level cache
-    bw_line("Dense backward epilogue bf16 4096x11008: dz = dy*relu'(y), dbias (fused)",
-            timed(lambda i: q.activation_backward(ys[i % 2], dys[i % 2], srt.ActivationType.relu, 0.0, outs[i % 2], db),
-                  steps=40, warmup=6), 3 * e + n_ * 2)
-    bw_line("add bf16 4096x11008 (dense, tensor + tensor)",
-            timed(lambda i: q.add(ys[i % 2], dys[i % 2], outs[i % 2]), steps=40, warmup=6), 3 * e)
-    bias_row = srt.Tensor.repeating(bias, (m_, n_))
-    bw_line("add bf16 4096x11008 + bias[11008] (stride-0 broadcast)",
-            timed(lambda i: q.add(ys[i % 2], bias_row, outs[i % 2]), steps=40, warmup=6), 2 * e + n_ * 2)
-    bw_line("tanh bf16 4096x11008", timed(lambda i: q.tanh(ys[i % 2], outs[i % 2]), steps=40, warmup=6), 2 * e)
-    f32out = srt.Tensor(shape=[m_, n_], dtype=np.float32)
-    bw_line("cast bf16 -> fp32 4096x11008", timed(lambda i: q.copy(ys[i % 2], f32out), steps=40, warmup=6), e + 2 * e)
 
 
 if __name__ == "__main__":

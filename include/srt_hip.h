@@ -185,7 +185,9 @@ srtStatus srtMemsetAsync(void* dst, int32_t value, size_t byteCount, srtStream s
  * (Sources/SwiftRTCore/platform/cpu/functions/CpuMath.swift:1141-1161, :1164-1186).
  * Elements: srtReal32F, srtReal16F, srtReal16BF, all three tensors the same type.  Products
  * are accumulated in fp32 and rounded once (nearest even) to the element type.
- * Operands may be any strided view; `out` may have any strides that do not alias.
+ * Operands may be any strided view; `out` may have any strides, but the span of storage it covers
+ * (first to last element) must not overlap the span of `a`, `b` or the bias: srtErrorInvalidValue
+ * otherwise (tiles are stored while other tiles are still being read).
  *
  * Returns srtErrorNotSupported (caller falls back to the CPU) for other element types,
  * orders other than row/col, or rank other than 2/3; srtErrorInvalidValue when extents do not
@@ -290,7 +292,9 @@ srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yD
  * Strided forms: all tensors the same rank and shape; an input broadcasts along a dimension by
  * giving it stride 0 there (Tensor(repeating:to:)); `out` may be any non-aliasing strided view.
  * TE forms: `element` points to ONE host-side element of the tensors' type, read during the call.
- * Flat forms: dense buffers of `count` elements.
+ * Flat forms: dense buffers of `count` elements -- what CudaQueue calls when canFlatten holds
+ * (CudaMath.swift:103-113); every binary operator has a tensor-tensor (Flat) and a tensor-element
+ * (TEFlat) form.
  * Element types 32F, 16F, 16BF (srtCopy / srtCopyFlat also convert between any two of them,
  * rounding to nearest even); arithmetic is fp32 with one rounding to the element type, i.e. the
  * reference's CPU definitions evaluated in E.Value (CpuMath.swift:646-662, :1189-1256,
@@ -303,26 +307,48 @@ srtStatus srtAdd(const void* a, const srtTensorDescriptor* aDesc, const void* b,
 srtStatus srtAddTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtAddFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+/* Tensor-element on a dense buffer: replaces srtAddTEFlat (math_api.h:95-100), argument order as there. */
+srtStatus srtAddTEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count,
+                       srtStream stream);
 srtStatus srtSub(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtSubTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtSubFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+srtStatus srtSubTEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count,
+                       srtStream stream);
 srtStatus srtMul(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtMulTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMulFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+srtStatus srtMulTEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count,
+                       srtStream stream);
 srtStatus srtDiv(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtDivTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtDivFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+srtStatus srtDivTEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count,
+                       srtStream stream);
 srtStatus srtMax(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtMaxTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMaxFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+srtStatus srtMaxTEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count,
+                       srtStream stream);
 srtStatus srtMin(const void* a, const srtTensorDescriptor* aDesc, const void* b, const srtTensorDescriptor* bDesc,
                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtMinTE(const void* a, const srtTensorDescriptor* aDesc, const void* element,
                    void* out, const srtTensorDescriptor* oDesc, srtStream stream);
+srtStatus srtMinFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream);
+srtStatus srtMinTEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count,
+                       srtStream stream);
+/* The reference's comparison family spells its dense tensor-element form with the type first
+ * (srtMinFlatTE, compare_api.h:160-167); both spellings are exported for max and min. */
+srtStatus srtMinFlatTE(srtDataType type, const void* a, const void* element, void* out, size_t count, srtStream stream);
+srtStatus srtMaxFlatTE(srtDataType type, const void* a, const void* element, void* out, size_t count, srtStream stream);
 srtStatus srtNeg(const void* a, const srtTensorDescriptor* aDesc,
                  void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 srtStatus srtExp(const void* a, const srtTensorDescriptor* aDesc,

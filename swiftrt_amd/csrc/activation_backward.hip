@@ -190,11 +190,11 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
   const dim3 grid(strips, chunks);
   if (vec) hipLaunchKernelGGL((activation_backward_kernel<T, VEC>), grid, dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((activation_backward_kernel<T, 1>), grid, dim3(256), 0, stream, p);
-  hipError_t e = hipGetLastError();
+  hipError_t e = launch_status(stream);
   if (e == hipSuccess && dbias) {
     hipLaunchKernelGGL((bias_gradient_finish_kernel<T>), dim3((p.N + 63) / 64), dim3(256), 0, stream,
                        (const float*)workspace, chunks, p.N, (typename T::storage*)dbias, dbias_stride);
-    e = hipGetLastError();
+    e = launch_status(stream);
   }
   // stream-ordered: the block becomes reusable for other streams only after the work queued so
   // far on `stream` has finished

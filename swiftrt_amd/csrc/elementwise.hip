@@ -159,7 +159,7 @@ hipError_t launch_v(const Map& m, hipStream_t stream) {
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   hipLaunchKernelGGL((map_kernel<TI, TO, Op, V>), dim3((unsigned)blocks), dim3(256), 0, stream, m);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 // Vector width the layout allows: the innermost dimension must be contiguous in the result and
@@ -433,15 +433,47 @@ SRT_UNARY(Sigmoid, kSigmoid)
 SRT_UNARY(Tanh, kTanh)
 SRT_UNARY(Copy, kCopy)
 
-srtStatus srtAddFlat(srtDataType type, const void* a, const void* b, void* out, size_t count, srtStream stream) {
+// Dense tensor-tensor and tensor-element forms of the six binary operators: what CudaQueue calls when
+// canFlatten holds (Sources/SwiftRTCore/platform/cuda/functions/CudaMath.swift:103-113).
+static srtStatus binary_flat(int op, srtDataType type, const void* a, const void* b, const void* element, void* out,
+                             size_t count, srtStream stream) {
   if (!float_type(type)) return srtErrorNotSupported;
   if (count == 0) return srtSuccess;
-  if (!a || !b || !out) return srtErrorInvalidValue;
+  if (!a || !out || (!b && !element)) return srtErrorInvalidValue;
   Map m{};
   m.a = a; m.b = b; m.o = out;
+  if (!b) {
+    m.b_is_element = 1;
+    m.element = host_element(type, element);
+  }
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
   return flat_pieces(count, type_size(type), type_size(type), m,
-                     [&](const Map& p) { return launch_op(kAdd, type, p, hs); });
+                     [&](const Map& p) { return launch_op(op, type, p, hs); });
+}
+
+#define SRT_BINARY_FLAT(Name, code)                                                                          \
+  srtStatus srt##Name##Flat(srtDataType type, const void* a, const void* b, void* out, size_t count,          \
+                            srtStream stream) {                                                               \
+    return binary_flat(code, type, a, b, nullptr, out, count, stream);                                       \
+  }                                                                                                           \
+  srtStatus srt##Name##TEFlat(const void* a, srtDataType atype, const void* element, void* out, size_t count, \
+                              srtStream stream) {                                                             \
+    return binary_flat(code, atype, a, nullptr, element, out, count, stream);                                \
+  }
+
+SRT_BINARY_FLAT(Add, kAdd)
+SRT_BINARY_FLAT(Sub, kSub)
+SRT_BINARY_FLAT(Mul, kMul)
+SRT_BINARY_FLAT(Div, kDiv)
+SRT_BINARY_FLAT(Max, kMax)
+SRT_BINARY_FLAT(Min, kMin)
+
+// the reference spells the comparison family's tensor-element form the other way round, with the type first
+srtStatus srtMinFlatTE(srtDataType type, const void* a, const void* element, void* out, size_t count, srtStream stream) {
+  return binary_flat(kMin, type, a, nullptr, element, out, count, stream);
+}
+srtStatus srtMaxFlatTE(srtDataType type, const void* a, const void* element, void* out, size_t count, srtStream stream) {
+  return binary_flat(kMax, type, a, nullptr, element, out, count, stream);
 }
 
 srtStatus srtCopyFlat(srtDataType atype, const void* a, srtDataType otype, void* out, size_t count,

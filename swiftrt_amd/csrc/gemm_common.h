@@ -7,6 +7,7 @@
 #include <atomic>
 
 #include "../../include/srt_hip.h"
+#include "status.h"
 
 namespace srt {
 

@@ -271,7 +271,7 @@ hipError_t launch_mfma128_vec(const GemmProblem& p, hipStream_t stream) {
   else if (a_kf) hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<true, false>), grid, dim3(256), 0, stream, p);
   else if (b_kf) hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<false, true>), grid, dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((gemm_f32_mfma128_vec_kernel<false, false>), grid, dim3(256), 0, stream, p);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 // ---- 32 x 32 tiles, the 4 waves split K ---------------------------------------------------------
@@ -501,7 +501,7 @@ hipError_t launch_f32_mfma_variant(const GemmProblem& p, bool splitk, hipStream_
       hipLaunchKernelGGL(gemm_f32_mfma_kernel<1>, grid, dim3(256), 0, stream, p);
     }
   }
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 hipError_t launch_f32_mfma(const GemmProblem& p, hipStream_t stream) {

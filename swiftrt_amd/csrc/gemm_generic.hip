@@ -104,7 +104,7 @@ hipError_t launch_generic(const GemmProblem& p, hipStream_t stream) {
     case srtReal16BF: hipLaunchKernelGGL(gemm_generic_kernel<BF16>, grid, block, 0, stream, p); break;
     default: return hipErrorNotSupported;
   }
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 }  // namespace srt

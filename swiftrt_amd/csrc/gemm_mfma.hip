@@ -419,7 +419,7 @@ hipError_t launch_one(const GemmProblem& p, hipStream_t stream) {
   }
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 template <typename T, int BM, int BN>
@@ -768,7 +768,7 @@ hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {
       hipLaunchKernelGGL(splitk_reduce_kernel<BF16>, dim3(blocks), dim3(256), 0, stream, (const float*)workspace, parts, p);
     else
       hipLaunchKernelGGL(splitk_reduce_kernel<F16>, dim3(blocks), dim3(256), 0, stream, (const float*)workspace, parts, p);
-    e = hipGetLastError();
+    e = launch_status(stream);
   }
   (void)srtDeviceFree(workspace);   // stream-ordered: reused only by work queued after the kernels above
   return e;

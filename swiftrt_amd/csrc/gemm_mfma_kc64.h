@@ -220,7 +220,7 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
   const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
   hipLaunchKernelGGL(kernel, dim3(tiles, p.batch), dim3(NT), lds_bytes, stream, p);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 template <typename T>

@@ -793,7 +793,7 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   const long long tiles = (long long)((p.M + tile_m - 1) / tile_m) * ((p.N + BN - 1) / BN) * p.batch;
   const int grid = ring::persistent_grid(tiles);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 template <typename T, bool A_KC, bool B_KC, int NS = 5, int TM = 8>

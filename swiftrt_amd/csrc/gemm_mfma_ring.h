@@ -852,7 +852,7 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   // order wants the stride between a workgroup's tiles to be a multiple of 8
   const int grid = persistent_grid(tiles);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 template <typename T, bool A_KC, bool B_KC, int NS = 5>

@@ -315,7 +315,7 @@ hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
   hipLaunchKernelGGL(kernel, dim3((p.N + 32 * NW - 1) / (32 * NW), p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
-  return hipGetLastError();
+  return launch_status(stream);
 }
 
 template <typename T>
@@ -355,6 +355,8 @@ bool skinny_supported(const GemmProblem& p) {
   if (p.sam < 0 || p.scm < 0 || p.scn < 0) return false;
   if (!aligned16(p.A) || !aligned16(p.B)) return false;
   if (p.batch > 65535) return false;
+  // 32-bit byte offsets must reach every row of x too (a row view of a wide tensor has a large pitch)
+  if (((long long)p.M + 8) * p.sam + p.K >= (0x7fffffffLL / 2 - 4096)) return false;
   if (p.sbk == 1) {                                     // W k-contiguous ([N, K])
     if ((p.sbn % 8) != 0 && p.N > 1) return false;
     if (p.sbn < 0) return false;

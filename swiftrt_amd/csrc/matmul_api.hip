@@ -20,7 +20,8 @@ bool supported_type(srtDataType t) { return t == srtReal32F || t == srtReal16F |
 srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
                         const void* b, const srtTensorDescriptor* bd, int tB,
                         const void* bias, const srtTensorDescriptor* biasd, int activation, double coef,
-                        void* out, const srtTensorDescriptor* od, GemmProblem* p, bool* empty) {
+                        void* out, const srtTensorDescriptor* od, GemmProblem* p, bool* empty,
+                        bool check_alias = true) {
   *empty = false;
   if (!ad || !bd || !od) return srtErrorInvalidValue;
   if (!ad->shape || !ad->strides || !bd->shape || !bd->strides || !od->shape || !od->strides)
@@ -66,6 +67,29 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
   }
   if (M == 0 || N == 0 || batch == 0) { *empty = true; return srtSuccess; }
   if (!a || !b || !out) return srtErrorInvalidValue;
+
+  // The kernels read operand tiles while other workgroups already store results: a result whose
+  // storage span overlaps the span of an input is refused (the Swift side always hands in a freshly
+  // allocated dense result, operators/Matmul.swift:38-39).
+  if (check_alias) {   // (the kernel query takes placeholder pointers and launches nothing)
+    const size_t es = od->type == srtReal32F ? 4 : 2;
+    auto span = [&](const void* base, long long e0, long long s0, long long e1, long long s1, long long e2, long long s2,
+                    uintptr_t* lo, uintptr_t* hi) {
+      const long long last = (e0 - 1) * s0 + (e1 - 1) * s1 + (e2 - 1) * s2;   // strides are non-negative (size_t)
+      *lo = reinterpret_cast<uintptr_t>(base);
+      *hi = *lo + (uintptr_t)(last + 1) * es;
+    };
+    uintptr_t olo, ohi, lo, hi;
+    span(out, p->M, p->scm, p->N, p->scn, p->batch, p->scb, &olo, &ohi);
+    span(a, p->M, p->sam, p->K, p->sak, p->batch, p->sab, &lo, &hi);
+    if (p->K > 0 && lo < ohi && olo < hi) return srtErrorInvalidValue;
+    span(b, p->K, p->sbk, p->N, p->sbn, p->batch, p->sbb, &lo, &hi);
+    if (p->K > 0 && lo < ohi && olo < hi) return srtErrorInvalidValue;
+    if (bias) {
+      span(bias, p->N, p->sbias, 1, 0, 1, 0, &lo, &hi);
+      if (lo < ohi && olo < hi) return srtErrorInvalidValue;
+    }
+  }
 
   // Column-major (or otherwise M-contiguous) result: compute C^T = op(B)^T . op(A)^T so the
   // kernels always write rows with the smaller stride innermost.
@@ -360,7 +384,7 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
   GemmProblem p;
   bool empty = false;
   srtStatus s = build_problem(a, aDesc, transposeA, b, bDesc, transposeB, nullptr, nullptr,
-                              srtActivationIdentity, 0.0, const_cast<void*>(out), oDesc, &p, &empty);
+                              srtActivationIdentity, 0.0, const_cast<void*>(out), oDesc, &p, &empty, false);
   if (s != srtSuccess) return s;
   const char* n = "empty";
   if (!empty) {
@@ -415,6 +439,12 @@ srtStatus srtMatmulTune(const void* a, const srtTensorDescriptor* aDesc, int32_t
     if (plan == kPlanGeneric && fallback != kPlanGeneric && 2.0 * p.M * p.N * p.K * p.batch > 1e9) continue;
     const int warm = 2, reps = 8;
     for (int i = 0; i < warm && err == hipSuccess; ++i) err = launch_plan(p, plan, hs);
+    if (plan == kPlanSplitK && err == hipErrorOutOfMemory) {
+      // no room for this plan's workspace (nothing was launched): it is not a candidate, as in run()
+      (void)hipGetLastError();
+      err = hipSuccess;
+      continue;
+    }
     if (err == hipSuccess) err = hipEventRecord(e0, hs);
     for (int i = 0; i < reps && err == hipSuccess; ++i) err = launch_plan(p, plan, hs);
     if (err == hipSuccess) err = hipEventRecord(e1, hs);

@@ -403,7 +403,7 @@ srtStatus srtMemsetAsync(void* dst, int32_t value, size_t byteCount, srtStream s
     hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, hs(stream),
                        reinterpret_cast<unsigned char*>(dst), v, byteCount);
   }
-  return from_hip(hipGetLastError());
+  return from_hip(srt::launch_status(hs(stream)));
 }
 
 srtStatus srtDelayStream(double seconds, srtStream stream) {

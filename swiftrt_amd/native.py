@@ -97,7 +97,6 @@ SIGNATURES = {
     "srtPlanCacheCount": (_i32, [ctypes.POINTER(ctypes.c_size_t)]),
     "srtPlanCacheSave": (_i32, [ctypes.c_char_p]),
     "srtPlanCacheLoad": (_i32, [ctypes.c_char_p]),
-    "srtAddFlat": (_i32, [_i32, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "srtCopyFlat": (_i32, [_i32, _vp, _i32, _vp, ctypes.c_size_t, _vp]),
     "srtFillFlat": (_i32, [_i32, _vp, _vp, ctypes.c_size_t, _vp]),
 }
@@ -105,6 +104,10 @@ SIGNATURES = {
 for _name in ("Add", "Sub", "Mul", "Div", "Max", "Min"):
     SIGNATURES["srt" + _name] = (_i32, [_vp, _descp, _vp, _descp, _vp, _descp, _vp])
     SIGNATURES["srt" + _name + "TE"] = (_i32, [_vp, _descp, _vp, _vp, _descp, _vp])
+    SIGNATURES["srt" + _name + "Flat"] = (_i32, [_i32, _vp, _vp, _vp, ctypes.c_size_t, _vp])
+    SIGNATURES["srt" + _name + "TEFlat"] = (_i32, [_vp, _i32, _vp, _vp, ctypes.c_size_t, _vp])
+for _name in ("Min", "Max"):
+    SIGNATURES["srt" + _name + "FlatTE"] = (_i32, [_i32, _vp, _vp, _vp, ctypes.c_size_t, _vp])
 for _name in ("Neg", "Exp", "Sigmoid", "Tanh", "Copy"):
     SIGNATURES["srt" + _name] = (_i32, [_vp, _descp, _vp, _descp, _vp])
 

@@ -87,6 +87,7 @@ class HipQueue:
         self.uses_cpu = False
         self.memory_type = "discrete"
         self.mode = "async"
+        self.use_flat_forms = True   # dense element-wise operands go through the Flat entry points
         L = native.lib()
         check(L.srtSetDevice(gpu_id), "srtSetDevice")
         s = ctypes.c_void_p()
@@ -194,10 +195,26 @@ class HipQueue:
         tensor-tensor form when `rhs` is a tensor, tensor-element form when it is a scalar, unary
         form when it is None.  Inputs must already have the shape of `out` (a broadcast operand is
         a stride-0 view, Tensor.repeating)."""
-        import numpy as np
         self.select()
         L = native.lib()
         a_ptr = lhs.device_read(self)
+        # dense operands of one shape take the Flat forms, as CudaQueue does when canFlatten holds
+        # (CudaMath.swift:103-113)
+        binary = name in ("Add", "Sub", "Mul", "Div", "Max", "Min")
+        if binary and self.use_flat_forms and rhs is not None and lhs.is_contiguous and out.is_contiguous \
+                and lhs.shape == out.shape and lhs.type_id == out.type_id and lhs.order == out.order:
+            if not hasattr(rhs, "device_read"):
+                element = lhs.element_storage(rhs)
+                o_ptr = out.device_read_write(self)
+                check(getattr(L, "srt" + name + "TEFlat")(a_ptr, lhs.type_id, ctypes.c_void_p(element.ctypes.data),
+                                                          o_ptr, out.count, self.stream), "srt" + name + "TEFlat")
+                return
+            if rhs.is_contiguous and rhs.shape == out.shape and rhs.type_id == out.type_id and rhs.order == out.order:
+                b_ptr = rhs.device_read(self)
+                o_ptr = out.device_read_write(self)
+                check(getattr(L, "srt" + name + "Flat")(out.type_id, a_ptr, b_ptr, o_ptr, out.count, self.stream),
+                      "srt" + name + "Flat")
+                return
         ad, ka = lhs.descriptor()
         if rhs is None:
             o_ptr = out.device_read_write(self)

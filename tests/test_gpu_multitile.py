@@ -1,0 +1,191 @@
+"""GPU parity tests of the path the headline benchmark times: the persistent 256 x 256 kernels with
+several tiles per workgroup, whole k stages and the k loop running across tile boundaries (the next
+tile's first stages are requested while the current tile's last ones are multiplied).
+
+Integer-valued operands in [-3, 3] make every partial sum exact in fp32 for K up to 1.8 M, so the
+result is bit-exact whatever the summation order: each pinned plan must reproduce, bit for bit,
+(a) the exact product on sampled rows and columns that cross every tile (float64 matmul of small
+integers is exact), and (b) over the WHOLE result, what the 128 x 128 kernel computes -- a kernel
+with no persistent grid, no ring and no cross-tile state, itself checked against the oracle at
+smaller sizes.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import swiftrt_amd as srt
+from swiftrt_amd import native
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+LAYOUTS = [(False, False), (False, True), (True, False), (True, True)]
+
+
+@pytest.fixture(autouse=True)
+def clean_plan_cache():
+    srt.PlanCache.clear()
+    yield
+    srt.PlanCache.clear()
+
+
+def query_kernel(a, ta, b, tb, out):
+    ad, k1 = a.descriptor()
+    bd, k2 = b.descriptor()
+    od, k3 = out.descriptor()
+    q = srt.current_queue()
+    buf = ctypes.create_string_buffer(64)
+    native.check(native.lib().srtMatmulQueryKernel(ctypes.byref(ad), int(ta), ctypes.byref(bd), int(tb),
+                                                   ctypes.byref(od), a.device_read(q), b.device_read(q),
+                                                   out.device_read(q), buf, 64))
+    return buf.value.decode()
+
+
+def pin(tmp_path, plan, dt, M, N, K, ta, tb, bias=False, act=srt.ActivationType.identity, batch=1):
+    layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
+    f = tmp_path / "plan.txt"
+    f.write_text(f"{dt} {M} {N} {K} {batch} {layout} {(1 if bias else 0) | (int(act) << 1)} {plan}\n")
+    srt.PlanCache.clear()
+    srt.PlanCache.load(f)
+
+
+_operands = {}
+
+
+def integer_operands(dt, shape, seed):
+    """One storage array of integers in [-3, 3] per (type, shape, seed), kept on the device."""
+    key = (dt, tuple(shape), seed)
+    if key not in _operands:
+        vals = H.rng(seed).integers(-3, 4, tuple(shape)).astype(np.float32)
+        t = srt.Tensor(H.encode(vals, dt))
+        t.device_read(srt.current_queue())
+        _operands[key] = (vals, t)
+    return _operands[key]
+
+
+def sample(extent, count, salt):
+    """`count` indices spread over [0, extent): every 256-wide tile is crossed, at varying offsets inside it."""
+    step = max(1, extent // count)
+    idx = (np.arange(count) * step + (np.arange(count) * salt) % step) % extent
+    return np.unique(idx)
+
+
+def run_pinned(tmp_path, plan, dt, a_t, ta, b_t, tb, M, N, K, bias=None, act=srt.ActivationType.identity):
+    pin(tmp_path, plan, dt, M, N, K, ta, tb, bias=bias is not None, act=act)
+    out = srt.Tensor(shape=[M, N], dtype=H.NP_STORAGE[dt])
+    assert query_kernel(a_t, ta, b_t, tb, out) == plan
+    srt.current_queue().matmul(a_t, ta, b_t, tb, out, bias=bias, activation=act)
+    return out.array()
+
+
+def check_plan(tmp_path, plan, dt, M, N, K, ta, tb, with_bias_relu=False):
+    a_vals, a_t = integer_operands(dt, (K, M) if ta else (M, K), seed=41)
+    b_vals, b_t = integer_operands(dt, (N, K) if tb else (K, N), seed=42)
+    bias_vals = bias_t = None
+    act = srt.ActivationType.identity
+    if with_bias_relu:
+        bias_vals, bias_t = integer_operands(dt, (N,), seed=43)
+        act = srt.ActivationType.relu
+    got = run_pinned(tmp_path, plan, dt, a_t, ta, b_t, tb, M, N, K, bias=bias_t, act=act)
+    # (a) sampled rows and columns against the exact product
+    a64 = (a_vals.T if ta else a_vals).astype(np.float64)
+    b64 = (b_vals.T if tb else b_vals).astype(np.float64)
+    rows, cols = sample(M, 64, 37), sample(N, 64, 53)
+
+    def finish(x, bias_part):
+        if with_bias_relu:
+            x = np.maximum(x + bias_part, 0.0)
+        return H.encode(x.astype(np.float32), dt)
+
+    want_rows = finish(a64[rows] @ b64, None if bias_vals is None else bias_vals[None, :].astype(np.float64))
+    want_cols = finish(a64 @ b64[:, cols], None if bias_vals is None else bias_vals[None, cols].astype(np.float64))
+    assert np.array_equal(got[rows].view(np.uint16), want_rows.view(np.uint16)), (plan, "rows")
+    assert np.array_equal(got[:, cols].view(np.uint16), want_cols.view(np.uint16)), (plan, "columns")
+    # (b) every element against the 128 x 128 kernel
+    ref = run_pinned(tmp_path, "mfma_128x128", dt, a_t, ta, b_t, tb, M, N, K, bias=bias_t, act=act)
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), (plan, "whole result")
+    return got
+
+
+def plans_for(ta, tb):
+    plans = ["mfma_256x256_m16", "mfma_256x256"]
+    if not ta and tb:
+        plans.append("mfma_256x256_k64")    # two k-contiguous operands
+    if not ta:
+        plans.append("mfma_128x256_m16")    # k-contiguous A
+    return plans
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+@pytest.mark.parametrize("ta,tb", LAYOUTS)
+def test_headline_shape_integer_bit_exact(dt, ta, tb, tmp_path):
+    """8192^3: 1024 tiles = 4 per workgroup, 256 whole stages, per-XCD k rotation with a transposed lhs."""
+    for plan in plans_for(ta, tb):
+        check_plan(tmp_path, plan, dt, 8192, 8192, 8192, ta, tb)
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+@pytest.mark.parametrize("ta,tb", LAYOUTS)
+def test_ragged_round_integer_bit_exact(dt, ta, tb, tmp_path):
+    """4608 x 4608 x 2048: 324 tiles on 256 workgroups (a second, ragged round; the grid is evened to 168),
+    64 whole stages; and 4400 x 4360 x 320: edge tiles in M and N, ten whole stages."""
+    for plan in plans_for(ta, tb):
+        check_plan(tmp_path, plan, dt, 4608, 4608, 2048, ta, tb)
+        check_plan(tmp_path, plan, dt, 4400, 4360, 320, ta, tb)
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+def test_dense_shape_bias_relu_integer_bit_exact(dt, tmp_path):
+    """The Dense configuration's shape, 4096 x 11008 x 4096 with an integer bias and relu: 688 tiles run as
+    three even rounds of 232 workgroups."""
+    for plan in ("mfma_256x256_m16", "mfma_256x256"):
+        got = check_plan(tmp_path, plan, dt, 4096, 11008, 4096, False, False, with_bias_relu=True)
+        assert np.all(H.decode(got) >= 0.0)
+
+
+def test_heuristic_takes_the_checked_kernels():
+    """The shapes above are run by the kernels checked above when nothing is pinned."""
+    a = srt.Tensor(shape=[8192, 8192], dtype=np.uint16)
+    out = srt.Tensor(shape=[8192, 8192], dtype=np.uint16)
+    assert query_kernel(a, False, a, False, out) == "mfma_256x256_m16"
+    assert query_kernel(a, True, a, False, out) == "mfma_256x256_m16"
+    x = srt.Tensor(shape=[4096, 4096], dtype=np.uint16)
+    w = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+    y = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+    assert query_kernel(x, False, w, False, y) == "mfma_256x256_m16"
+
+
+# ---- the reference's batched known answers on the device, bf16 included -----------------------------------
+@pytest.mark.parametrize("dt", [H.F32, H.F16, H.BF16])
+def test_reference_kat_batched_and_right_batched(kats, dt):
+    """test_AlgebraicField.swift:572-597 (batched) through the codec -- values up to 275 are not all bf16
+    numbers -- and the right-batched form: one lhs matrix against a batch (batch stride 0)."""
+    k = kats["matmul_batched"]
+    a = H.encode(np.arange(12, dtype=np.float32).reshape(k["a_arange_shape"]), dt)
+    b = H.encode(np.arange(16, dtype=np.float32).reshape(k["b_arange_shape"]), dt)
+    got = srt.matmul(srt.Tensor(a), srt.Tensor(b)).array()
+    assert np.array_equal(got.view(np.uint8), H.encode(np.array(k["c"], np.float32), dt).view(np.uint8))
+    kr = kats["matmul_right_batched"]
+    a2 = srt.Tensor(H.encode(np.arange(6, dtype=np.float32).reshape(3, 2), dt))
+    a3 = srt.Tensor.repeating(a2, (2, 3, 2))
+    assert a3.strides[0] == 0
+    got = srt.matmul(a3, srt.Tensor(b)).array()
+    assert np.array_equal(got.view(np.uint8), H.encode(np.array(kr["c"], np.float32), dt).view(np.uint8))
+
+
+# ---- operands that alias the result -------------------------------------------------------------------
+def test_result_overlapping_an_operand_is_refused():
+    q = srt.current_queue()
+    buf = srt.Tensor(np.zeros((64, 64), np.float32))
+    other = srt.Tensor(np.zeros((32, 32), np.float32))
+    a, out = buf[0:32, 0:32], buf[16:48, 0:32]      # spans overlap
+    with pytest.raises(native.SrtError) as e:
+        q.matmul(a, False, other, False, out)
+    assert e.value.status == native.ERROR_INVALID_VALUE
+    with pytest.raises(native.SrtError):
+        q.matmul(other, False, a, False, out)
+    # disjoint row blocks of one buffer are fine
+    lo, hi = buf[0:32, :], buf[32:64, :]
+    w = srt.Tensor(np.eye(64, dtype=np.float32))
+    q.matmul(lo, False, w, False, hi)
