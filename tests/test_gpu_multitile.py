@@ -45,7 +45,9 @@ def query_kernel(a, ta, b, tb, out):
 def pin(tmp_path, plan, dt, M, N, K, ta, tb, bias=False, act=srt.ActivationType.identity, batch=1):
     layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
     f = tmp_path / "plan.txt"
-    f.write_text(f"{dt} {M} {N} {K} {batch} {layout} {(1 if bias else 0) | (int(act) << 1)} {plan}\n")
+    # the call's own epilogue key, and the plain one the kernel query looks up
+    keys = {(1 if bias else 0) | (int(act) << 1), int(srt.ActivationType.identity) << 1}
+    f.write_text("".join(f"{dt} {M} {N} {K} {batch} {layout} {e} {plan}\n" for e in sorted(keys)))
     srt.PlanCache.clear()
     srt.PlanCache.load(f)
 
