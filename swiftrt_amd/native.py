@@ -7,7 +7,9 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libSwiftRTHip.so")
+# SWIFTRT_HIP_LIBRARY selects another build of the same library (e.g. lib/debug/libSwiftRTHip.so from
+# `make DEBUG=1`, which checks every launch synchronously)
+LIB_PATH = os.environ.get("SWIFTRT_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libSwiftRTHip.so")
 
 # srtStatus
 SUCCESS = 0
@@ -91,6 +93,8 @@ SIGNATURES = {
     "srtDelayStream": (_i32, [ctypes.c_double, _vp]),
     "srtActivationBackwardBias": (_i32, [_vp, _descp, _vp, _descp, _i32, ctypes.c_double, _vp, _descp,
                                           _vp, _descp, _vp]),
+    "srtActivationBackwardBiasNoAlloc": (_i32, [_vp, _descp, _vp, _descp, _i32, ctypes.c_double, _vp, _descp,
+                                                 _vp, _descp, _vp]),
     "srtMatmulTune": (_i32, [_vp, _descp, _i32, _vp, _descp, _i32, _vp, _descp, _i32, ctypes.c_double, _vp, _descp,
                               _vp, ctypes.c_char_p, ctypes.c_size_t]),
     "srtPlanCacheClear": (_i32, []),
