@@ -281,6 +281,21 @@ srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yD
                                     void* dx, const srtTensorDescriptor* dxDesc,
                                     void* dbias, const srtTensorDescriptor* dbiasDesc, srtStream stream);
 
+/* The same computation for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Identical arguments and
+ * results (bit for bit) to srtActivationBackwardBias, but the fp32 partial rows of the bias gradient
+ * live in a fixed 8 MiB device array inside the library (one per GPU, held until the process ends)
+ * instead of a block from the allocator: the call performs no device or host allocation and frees
+ * nothing.  Limit: with a bias gradient, N <= 2 097 152 columns (one fp32 partial row must fit the 8 MiB);
+ * srtErrorInvalidValue beyond that.  Every call on a GPU shares that GPU's array:
+ * calls that overlap in time on one GPU (different streams, or different threads) race; serialise them.
+ * The array needs no clearing between calls (every entry read is written first by the same call). */
+srtStatus srtActivationBackwardBiasNoAlloc(const void* y, const srtTensorDescriptor* yDesc,
+                                           const void* dy, const srtTensorDescriptor* dyDesc,
+                                           srtActivation activation, double coef,
+                                           void* dx, const srtTensorDescriptor* dxDesc,
+                                           void* dbias, const srtTensorDescriptor* dbiasDesc, srtStream stream);
+
 /* ---- element-wise neighbours of the path ---------------------------------------------------------
  * Same names, argument order and conventions as the reference's native module
  * (Modules/SwiftRTCuda/math_api.h: srtAdd :75-100, srtDiv :138-148, srtExp :166-170, srtMul

@@ -162,8 +162,40 @@ __global__ __launch_bounds__(256) void bias_gradient_finish_kernel(const float* 
     dbias[(long long)n * stride] = T::from_float((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]));
 }
 
+// Scratch of the entry point that allocates nothing (srtActivationBackwardBiasNoAlloc): the chunks'
+// partial bias-gradient rows, [chunks][N] fp32.  One copy per device, held until the process ends;
+// kScratchBytes is the entry point's size limit.  Host code never passes the array's name to a
+// kernel: it asks the runtime for the device's address of it once per device and uses that pointer.
+constexpr size_t kScratchBytes = 8u << 20;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
+
+// The current device's address of `scratch` (cached per device), or null with *status set.
+float* scratch_of_current_device(srtStatus* status) {
+  static std::atomic<void*> cached[64];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) {
+    *status = srtErrorNoDevice;
+    return nullptr;
+  }
+  void* ptr = cached[device].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      *status = e == hipSuccess ? srtErrorUnknown : from_hip(e);
+      return nullptr;
+    }
+    cached[device].store(ptr, std::memory_order_release);
+  }
+  *status = srtSuccess;
+  return static_cast<float*>(ptr);
+}
+
+// fixed_workspace: false -- the partial rows come from the library's stream-ordered allocator;
+// true -- from the device's static scratch array (nothing is allocated or freed), and a problem
+// whose partial rows exceed it is refused.
 template <typename T>
-srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_t stream) {
+srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_t stream, bool fixed_workspace) {
   constexpr int VEC = 16 / sizeof(typename T::storage);
   const size_t es = sizeof(typename T::storage);
   auto vec_ok = [&](const void* ptr, long long sm, long long sn) {
@@ -177,12 +209,23 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
   const int max_chunks = (p.M + 15) / 16;
   if (chunks > max_chunks) chunks = max_chunks;
   if (chunks > 65535) chunks = 65535;
+  // the chunks' partial rows fit the fixed workspace of the entry point that does not allocate whenever
+  // a single row does (both entry points cut the rows the same way, so their sums agree bit for bit)
+  const long long fit = (long long)(kScratchBytes / sizeof(float)) / p.N;
+  if (chunks > fit) chunks = (int)fit;
   if (chunks < 1) chunks = 1;
   p.rows_per_chunk = (p.M + chunks - 1) / chunks;
   chunks = (p.M + p.rows_per_chunk - 1) / p.rows_per_chunk;
 
   void* workspace = nullptr;
-  if (dbias) {
+  if (dbias && fixed_workspace) {
+    if ((size_t)chunks * p.N * sizeof(float) > kScratchBytes) return srtErrorInvalidValue;
+    srtStatus s;
+    workspace = scratch_of_current_device(&s);
+    if (!workspace) return s;
+    // every entry the second kernel reads is written by the first (all chunks, all N columns), so the
+    // previous call's contents need no clearing
+  } else if (dbias) {
     srtStatus s = srtDeviceAllocate(&workspace, (size_t)chunks * p.N * sizeof(float), reinterpret_cast<srtStream>(stream));
     if (s != srtSuccess) return s;
   }
@@ -198,18 +241,18 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
   }
   // stream-ordered: the block becomes reusable for other streams only after the work queued so
   // far on `stream` has finished
-  if (workspace) (void)srtDeviceFree(workspace);
+  if (workspace && !fixed_workspace) (void)srtDeviceFree(workspace);
   return from_hip(e);
 }
 
 }  // namespace
 }  // namespace srt
 
-extern "C" srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yDesc, const void* dy,
-                                               const srtTensorDescriptor* dyDesc, srtActivation activation,
-                                               double coef, void* dx, const srtTensorDescriptor* dxDesc,
-                                               void* dbias, const srtTensorDescriptor* dbiasDesc,
-                                               srtStream stream) {
+static srtStatus activation_backward_bias(const void* y, const srtTensorDescriptor* yDesc, const void* dy,
+                                          const srtTensorDescriptor* dyDesc, srtActivation activation,
+                                          double coef, void* dx, const srtTensorDescriptor* dxDesc,
+                                          void* dbias, const srtTensorDescriptor* dbiasDesc,
+                                          srtStream stream, bool fixed_workspace) {
   auto ok = [](const srtTensorDescriptor* d) { return d && d->shape && d->strides; };
   if (!ok(yDesc) || !ok(dyDesc) || !ok(dxDesc)) return srtErrorInvalidValue;
   if (dxDesc->rank != 2) return srtErrorNotSupported;
@@ -250,8 +293,24 @@ extern "C" srtStatus srtActivationBackwardBias(const void* y, const srtTensorDes
   p.coef = (float)coef;
   hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
   switch (t) {
-    case srtReal32F: return srt::run<srt::F32>(p, dbias, dbias_stride, hs);
-    case srtReal16F: return srt::run<srt::F16>(p, dbias, dbias_stride, hs);
-    default: return srt::run<srt::BF16>(p, dbias, dbias_stride, hs);
+    case srtReal32F: return srt::run<srt::F32>(p, dbias, dbias_stride, hs, fixed_workspace);
+    case srtReal16F: return srt::run<srt::F16>(p, dbias, dbias_stride, hs, fixed_workspace);
+    default: return srt::run<srt::BF16>(p, dbias, dbias_stride, hs, fixed_workspace);
   }
+}
+
+extern "C" srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yDesc, const void* dy,
+                                               const srtTensorDescriptor* dyDesc, srtActivation activation,
+                                               double coef, void* dx, const srtTensorDescriptor* dxDesc,
+                                               void* dbias, const srtTensorDescriptor* dbiasDesc,
+                                               srtStream stream) {
+  return activation_backward_bias(y, yDesc, dy, dyDesc, activation, coef, dx, dxDesc, dbias, dbiasDesc, stream, false);
+}
+
+extern "C" srtStatus srtActivationBackwardBiasNoAlloc(const void* y, const srtTensorDescriptor* yDesc, const void* dy,
+                                                      const srtTensorDescriptor* dyDesc, srtActivation activation,
+                                                      double coef, void* dx, const srtTensorDescriptor* dxDesc,
+                                                      void* dbias, const srtTensorDescriptor* dbiasDesc,
+                                                      srtStream stream) {
+  return activation_backward_bias(y, yDesc, dy, dyDesc, activation, coef, dx, dxDesc, dbias, dbiasDesc, stream, true);
 }

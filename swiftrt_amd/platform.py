@@ -262,9 +262,11 @@ class HipQueue:
         check(native.lib().srtFillFlat(out.type_id, o_ptr, ctypes.c_void_p(element.ctypes.data), out.count,
                                        self.stream), "srtFillFlat")
 
-    def activation_backward(self, y, dy, activation, coef, dx, dbias=None):
+    def activation_backward(self, y, dy, activation, coef, dx, dbias=None, no_alloc=False):
         """Role of CudaActivation.backward (platform/cuda/layers/CudaActivation.swift:101-127) fused
-        with the bias gradient: dx = dy * act'(y), dbias = column sums of dx."""
+        with the bias gradient: dx = dy * act'(y), dbias = column sums of dx.  no_alloc: the entry
+        point that takes its workspace from a fixed array inside the library (the tensors must then
+        already be resident on the device, or the mirror's own staging would allocate)."""
         self.select()
         y_ptr, dy_ptr = y.device_read(self), dy.device_read(self)
         dx_ptr = dx.device_read_write(self)
@@ -277,11 +279,12 @@ class HipQueue:
             dbd_ref = ctypes.byref(dbd)
         else:
             db_ptr, dbd_ref, k4 = None, None, None
-        st = native.lib().srtActivationBackwardBias(y_ptr, ctypes.byref(yd), dy_ptr, ctypes.byref(dyd),
-                                                    int(activation), float(coef), dx_ptr, ctypes.byref(dxd),
-                                                    db_ptr, dbd_ref, self.stream)
+        name = "srtActivationBackwardBiasNoAlloc" if no_alloc else "srtActivationBackwardBias"
+        st = getattr(native.lib(), name)(y_ptr, ctypes.byref(yd), dy_ptr, ctypes.byref(dyd),
+                                         int(activation), float(coef), dx_ptr, ctypes.byref(dxd),
+                                         db_ptr, dbd_ref, self.stream)
         del k1, k2, k3, k4
-        check(st, "srtActivationBackwardBias")
+        check(st, name)
 
     def __del__(self):
         try:
