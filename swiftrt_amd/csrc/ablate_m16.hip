@@ -1,0 +1,146 @@
+// Measuring instrument, not part of the library: times the headline kernel (gemm_m16_kernel, bf16,
+// 8192 x 8192 x 8192 by default) with parts of its main loop taken out, to attribute time and -- under
+// the power limit, through the clock the device sustains -- energy to them.  Compiled once per variant:
+//   -DSRT_ABLATE=<bits>   see gemm_mfma_m16.h (1 no barrier, 2 no operand traffic, 4 fragments stay in
+//                         registers, 8 every workgroup requests tile 0)
+//   -DABL_NS=<3|4|5>      ring depth (prefetch distance NS - 1 stages)
+//   -DABL_DEEP=1          the 64-deep form of the kernel (gemm_mfma_m16d.h; no ablation switches)
+//   -DABL_AKC / -DABL_BKC operand layouts (defaults 1 / 0: the headline's row-major A and B)
+// Run: ablate_m16 [normal|zero] [M N K]; operands ~ N(0,1)/sqrt(K) (generated on the device) or zeros.
+// Prints one line: variant, data, median and minimum time per launch, TFLOP/s, and (unablated builds) the
+// largest error of 64 sampled results against a double-precision dot product.
+#define SRT_M16_ANY_RING_DEPTH 1
+#include "gemm_mfma_m16d.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#ifndef ABL_NS
+#define ABL_NS 5
+#endif
+#ifndef ABL_DEEP
+#define ABL_DEEP 0
+#endif
+#ifndef ABL_AKC
+#define ABL_AKC 1
+#endif
+#ifndef ABL_BKC
+#define ABL_BKC 0
+#endif
+
+#define CHECK(x)                                                              \
+  do {                                                                        \
+    hipError_t e_ = (x);                                                      \
+    if (e_ != hipSuccess) {                                                   \
+      fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_));                 \
+      exit(1);                                                                \
+    }                                                                         \
+  } while (0)
+
+namespace {
+
+__device__ inline uint32_t mix(uint32_t x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+__global__ void fill_normal(uint16_t* dst, size_t n, float scale, uint32_t seed, int zero) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float v = 0.0f;
+    if (!zero) {
+      const uint32_t s = seed + (uint32_t)i * 2u;
+      const float u1 = (mix(s) >> 8) * (1.0f / 16777216.0f) + 1e-7f;
+      const float u2 = (mix(s + 1u) >> 8) * (1.0f / 16777216.0f);
+      v = sqrtf(-2.0f * logf(u1)) * cosf(6.2831853f * u2) * scale;
+    }
+    dst[i] = srt::BF16::from_float(v);
+  }
+}
+
+float bf16_to_float(uint16_t h) {
+  uint32_t u = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  const bool zero = argc > 1 && strcmp(argv[1], "zero") == 0;
+  int M = 8192, N = 8192, K = 8192;
+  if (argc > 4) { M = atoi(argv[2]); N = atoi(argv[3]); K = atoi(argv[4]); }
+  if (M % 256 || N % 256 || K % 32 || K < 160) { fprintf(stderr, "M, N multiples of 256; K a multiple of 32, at least 160\n"); return 1; }
+  uint16_t *a, *b, *c;
+  CHECK(hipMalloc(&a, (size_t)M * K * 2));
+  CHECK(hipMalloc(&b, (size_t)K * N * 2));
+  CHECK(hipMalloc(&c, (size_t)M * N * 2));
+  const float scale = 1.0f / sqrtf((float)K);
+  hipLaunchKernelGGL(fill_normal, dim3(4096), dim3(256), 0, 0, a, (size_t)M * K, scale, 0x1234567u, zero ? 1 : 0);
+  hipLaunchKernelGGL(fill_normal, dim3(4096), dim3(256), 0, 0, b, (size_t)K * N, scale, 0x89abcdeu, zero ? 1 : 0);
+  CHECK(hipDeviceSynchronize());
+
+  srt::GemmProblem p{};
+  p.dtype = srtReal16BF;
+  p.M = M; p.N = N; p.K = K; p.batch = 1;
+  p.A = a; p.B = b; p.C = c;
+  // A stored [M, K] (k-contiguous) or [K, M]; B stored [N, K] (k-contiguous) or [K, N]
+  if (ABL_AKC) { p.sam = K; p.sak = 1; } else { p.sam = 1; p.sak = M; }
+  if (ABL_BKC) { p.sbn = K; p.sbk = 1; } else { p.sbn = 1; p.sbk = N; }
+  p.scm = N; p.scn = 1;
+  p.activation = srtActivationIdentity;
+
+  auto launch = [&]() {
+    if (ABL_DEEP) CHECK((srt::m16d::launch_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN>(p, 0)));
+    else CHECK((srt::m16::launch_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN, ABL_NS, 8>(p, 0)));
+  };
+  hipEvent_t e0, e1;
+  CHECK(hipEventCreate(&e0));
+  CHECK(hipEventCreate(&e1));
+  auto group_ms = [&](int launches) {
+    CHECK(hipEventRecord(e0));
+    for (int i = 0; i < launches; ++i) launch();
+    CHECK(hipEventRecord(e1));
+    CHECK(hipEventSynchronize(e1));
+    float ms;
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+    return ms / launches;
+  };
+  const double flop = 2.0 * M * N * K;
+  const int per_group = std::max(4, (int)(20.0 * 1.1e12 / flop));
+  // settle: at least 0.6 s of load
+  double spent = 0.0;
+  while (spent < 600.0) spent += group_ms(per_group) * per_group;
+  std::vector<float> t;
+  for (int g = 0; g < 7; ++g) t.push_back(group_ms(per_group));
+  std::sort(t.begin(), t.end());
+  const float med = t[t.size() / 2];
+
+  double worst = -1.0;
+  if (SRT_ABLATE == 0 && !zero) {
+    // 64 sampled results against double-precision dot products of the stored operands
+    std::vector<uint16_t> ha((size_t)M * K), hb((size_t)K * N), hc((size_t)M * N);
+    CHECK(hipMemcpy(ha.data(), a, ha.size() * 2, hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hb.data(), b, hb.size() * 2, hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hc.data(), c, hc.size() * 2, hipMemcpyDeviceToHost));
+    worst = 0.0;
+    for (int s = 0; s < 64; ++s) {
+      const int m = (int)(((long long)s * 2654435761LL) % M), n = (int)(((long long)s * 40503LL * 977) % N);
+      double ref = 0.0;
+      for (int k = 0; k < K; ++k)
+        ref += (double)bf16_to_float(ha[(size_t)m * p.sam + (size_t)k * p.sak]) *
+               (double)bf16_to_float(hb[(size_t)k * p.sbk + (size_t)n * p.sbn]);
+      worst = std::max(worst, fabs(ref - (double)bf16_to_float(hc[(size_t)m * N + n])));
+    }
+  }
+  printf("ablate=%d deep=%d ns=%d akc=%d bkc=%d %-6s M=%d N=%d K=%d: median %.4f ms %.1f TFLOP/s (min %.4f ms %.1f)", SRT_ABLATE,
+         ABL_DEEP, ABL_NS, ABL_AKC, ABL_BKC, zero ? "zero" : "normal", M, N, K, med, flop / (med * 1e-3) * 1e-12, t[0],
+         flop / (t[0] * 1e-3) * 1e-12);
+  if (worst >= 0.0) printf("  max |error| of 64 samples %.3g (|c| ~ %.2g)", worst, 1.0 / sqrt((double)K) * sqrt((double)K) / sqrt((double)K));
+  printf("\n");
+  return 0;
+}

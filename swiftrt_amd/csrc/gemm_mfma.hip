@@ -59,6 +59,14 @@ SRT_M16_DECL(F16)
 SRT_M16P_DECL(BF16)
 SRT_M16P_DECL(F16)
 #undef SRT_M16P_DECL
+#define SRT_M16D_DECL(T)                                                  \
+  hipError_t launch_m16d_##T##_00(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_##T##_01(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_##T##_10(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_##T##_11(const GemmProblem&, hipStream_t);
+SRT_M16D_DECL(BF16)
+SRT_M16D_DECL(F16)
+#undef SRT_M16D_DECL
 hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_F16_10(const GemmProblem&, hipStream_t);
@@ -479,6 +487,21 @@ hipError_t launch_m16<F16>(const GemmProblem& p, bool a_kc, bool b_kc, hipStream
   return launch_m16_F16_00(p, stream);
 }
 
+// the 64-deep form of the 16x16x32 kernel
+template <typename T>
+hipError_t launch_m16d(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) {
+    if (a_kc && b_kc) return launch_m16d_BF16_11(p, stream);
+    if (a_kc) return launch_m16d_BF16_10(p, stream);
+    if (b_kc) return launch_m16d_BF16_01(p, stream);
+    return launch_m16d_BF16_00(p, stream);
+  }
+  if (a_kc && b_kc) return launch_m16d_F16_11(p, stream);
+  if (a_kc) return launch_m16d_F16_10(p, stream);
+  if (b_kc) return launch_m16d_F16_01(p, stream);
+  return launch_m16d_F16_00(p, stream);
+}
+
 // the 128 x 256 form of the 16x16x32 ring kernel (k-contiguous A)
 template <typename T>
 hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
@@ -495,6 +518,7 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 4: return T::dtype == srtReal16BF ? launch_kc64_BF16(p, stream) : launch_kc64_F16(p, stream);
     case 5: return launch_m16<T>(p, a_kc, b_kc, stream);
     case 6: return launch_m16h<T>(p, b_kc, stream);
+    case 9: return launch_m16d<T>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     case 7: return launch_any_layout<T, 128, 128>(p, stream);
     case 8: return launch_any_layout<T, 64, 64>(p, stream);
@@ -532,7 +556,8 @@ static int mfma_layout(const GemmProblem& p) {
 
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
-// 128 x 256 form for a k-contiguous A), or 0 when the problem does not qualify for it.
+// 128 x 256 form for a k-contiguous A, 9: the 16x16x32 kernel with 64-deep staging units), or 0 when the
+// problem does not qualify for it.
 int mfma_config(const GemmProblem& p, int tile) {
   if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
     if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
@@ -540,8 +565,9 @@ int mfma_config(const GemmProblem& p, int tile) {
     return tile << 2;
   }
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || tile > 6) return 0;
+  if (layout < 0 || tile < 1 || (tile > 6 && tile != 9)) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
+  if (tile == 9 && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
   if (tile == 6 && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
@@ -625,8 +651,14 @@ int mfma_select(const GemmProblem& p) {
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
                                    (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
   const long long ring_from = layout == 3 ? 96 : (p.K >= 1024 ? 24 : 32);
+  //  * the 64-deep form of the 16x16x32 kernel (whole-line loads of k-contiguous operands, one barrier per 128
+  //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
+  //    NN 1440 -> 1505 TFLOP/s, NT 1420 -> 1531, TN 1443 -> 1501, TT 1477 -> 1538), and of the 32x32x16
+  //    64-deep kernel that two k-contiguous operands used to take for short k loops; it needs whole units
+  const bool deep_ok = p.K % 64 == 0 && p.K >= 512;
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
+  else if (whole_ok && deep_ok && t256 >= 128) tile = 9;
   else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
   else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
   else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout & 2) == 0))) tile = 1;
@@ -780,6 +812,7 @@ const char* mfma_name(int config) {
     case 4: return "mfma_256x256_k64";
     case 5: return "mfma_256x256_m16";
     case 6: return "mfma_128x256_m16";
+    case 9: return "mfma_256x256_m16_k64";
     case 2: return "mfma_128x128";
     case 7: return "mfma_128x128_any";
     case 8: return "mfma_64x64_any";

@@ -192,14 +192,14 @@ def test_kernel_selection_is_queryable_without_gpu():
         assert st == 0
         return buf.value.decode()
 
-    # a full device and a long k loop: the 256 x 256 ring on 16x16x32 MFMAs, in every layout
-    assert query(native.REAL16BF, 8192, 8192, 8192) == "mfma_256x256_m16"
-    assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256_m16"
-    assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256_m16"
-    assert query(native.REAL16BF, 8192, 8192, 8192, tb=True) == "mfma_256x256_m16"
-    # short k loops: the same, except that two k-contiguous operands take the kernel with 64-deep stages
-    assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256_m16"
-    assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_k64"
+    # a full device: the 16x16x32 kernel with 64-deep staging units, in every layout
+    assert query(native.REAL16BF, 8192, 8192, 8192) == "mfma_256x256_m16_k64"
+    assert query(native.REAL16BF, 8192, 8192, 8192, ta=True) == "mfma_256x256_m16_k64"
+    assert query(native.REAL16BF, 4096, 11008, 4096) == "mfma_256x256_m16_k64"
+    assert query(native.REAL16BF, 8192, 8192, 8192, tb=True) == "mfma_256x256_m16_k64"
+    # short k loops: the same (two k-contiguous operands used to take the 32x32x16 kernel with 64-deep stages)
+    assert query(native.REAL16BF, 4096, 4096, 1024) == "mfma_256x256_m16_k64"
+    assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_m16_k64"
     # few tiles and a long k loop: K split over the idle compute units -- when that buys more than the
     # half-height tiles a k-contiguous A allows
     assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_256x256_splitk"           # eight parts
@@ -210,11 +210,11 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: from K = 2048
     assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x256"        # 32 tiles: the ring from 24 up
     assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_64x64"          # 16 tiles
-    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x256_m16"    # two parts at K = 2048 do not pay
+    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x256_m16_k64"    # two parts at K = 2048 do not pay
     # mid-size problems: the 256 x 256 kernels from 24 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
-    assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16"             # 144 tiles, long k loop
-    assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256_m16"             # and a short one
+    assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16_k64"             # 144 tiles, long k loop
+    assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256_m16_k64"             # and a short one
     # a k-contiguous A and at most one round of 128 x 256 tiles: the half-height form of the 16x16x32 kernel
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16"             # 128 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16"
@@ -222,7 +222,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: whole tiles, K split
     assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x256"
     assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_128x256_m16"            # 258 whole tiles: two rounds for two tiles
-    assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16"   # both k-contiguous: one round of halves or none
+    assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16_k64"   # both k-contiguous: one round of halves or none
     assert query(native.REAL16BF, 1536, 4096, 11008, tb=True) == "mfma_256x256_splitk"
     assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16"              # 8 half tiles
     assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
@@ -252,11 +252,11 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL32F, 512, 512, 512) in ("generic", "f32_mfma")
     # operands of 1 Gi elements or more: halves of M (N for a k-contiguous B, the batch first) that the
     # 256 x 256 kernels' 32-bit offsets reach; a k walk out of reach keeps the small tiles
-    assert query(native.REAL16BF, 32768, 32768, 8192) == "mfma_256x256_m16/pieces"           # C alone is 1 Gi
-    assert query(native.REAL16BF, 262144, 8192, 8192) == "mfma_256x256_m16/pieces"           # A and C
-    assert query(native.REAL16BF, 8192, 262144, 8192, tb=True) == "mfma_256x256_m16/pieces"  # B [N, K] and C
+    assert query(native.REAL16BF, 32768, 32768, 8192) == "mfma_256x256_m16_k64/pieces"           # C alone is 1 Gi
+    assert query(native.REAL16BF, 262144, 8192, 8192) == "mfma_256x256_m16_k64/pieces"           # A and C
+    assert query(native.REAL16BF, 8192, 262144, 8192, tb=True) == "mfma_256x256_m16_k64/pieces"  # B [N, K] and C
     assert query(native.REAL16BF, 8192, 8192, 262144, ta=True) == "mfma_128x128"             # k walk of A and B
-    assert query(native.REAL16BF, 32768, 32512, 8192) == "mfma_256x256_m16"                  # just within reach
+    assert query(native.REAL16BF, 32768, 32512, 8192) == "mfma_256x256_m16_k64"                  # just within reach
     assert query(native.REAL16BF, 8, 65664, 32768, tb=True) == "skinny/pieces"
 
 

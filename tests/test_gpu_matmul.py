@@ -296,7 +296,7 @@ def test_cfg3_bf16_8192_sampled_rows_and_invariants(ta):
     a = H.encode((r.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n))), H.BF16)
     b = H.encode((r.standard_normal((n, n), dtype=np.float32) / np.float32(np.sqrt(n))), H.BF16)
     a_stored = np.ascontiguousarray(a.T) if ta else a
-    got = gpu_matmul(a_stored, b, ta=ta, want_kernel="mfma_256x256_m16")
+    got = gpu_matmul(a_stored, b, ta=ta, want_kernel="mfma_256x256_m16_k64")
     rows = np.unique(np.concatenate([np.arange(0, n, 131), [n - 1, 255, 256, 4095, 4096]]))
     c64 = H.to64(a[rows]) @ H.to64(b)
     absprod = np.abs(H.to64(a[rows])) @ np.abs(H.to64(b))
@@ -790,13 +790,18 @@ def test_m16_half_tile_epilogues_vs_oracle_and_nan(act, tmp_path):
     srt.PlanCache.clear()
 
 
-def test_m16_kernel_is_the_choice_for_a_full_device_and_long_k():
+def test_m16_kernels_are_the_choice_for_a_full_device():
+    """From half a device up: the 64-deep form when K is a whole number of 64-deep units (at least eight), else
+    the 32-deep one."""
     a = srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16))
     b = srt.Tensor(H.encode(np.zeros((2048, 4096), np.float32), H.BF16))
     out = srt.Tensor(shape=[4096, 4096], dtype=a.dtype)
-    assert query_kernel(a, False, b, False, out) == "mfma_256x256_m16"
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_m16_k64"
     assert query_kernel(a, False, srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16)), True, out) == \
-        "mfma_256x256_m16"
+        "mfma_256x256_m16_k64"
+    a2 = srt.Tensor(H.encode(np.zeros((4096, 2080), np.float32), H.BF16))      # K = 2080 = 32.5 units
+    b2 = srt.Tensor(H.encode(np.zeros((2080, 4096), np.float32), H.BF16))
+    assert query_kernel(a2, False, b2, False, out) == "mfma_256x256_m16"
 
 
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
@@ -958,14 +963,14 @@ def test_bf16_operands_beyond_4_gib_bit_exact(case):
     block = big0.astype(np.float64) @ small.astype(np.float64).T          # [P, small_rows], exact integers
     if case == "nn_big_a":      # A [65664, K] . B [K, 512]
         a, b, ta, tb = _periodic(H.encode(big0, H.BF16), reps, 0), H.encode(np.ascontiguousarray(small.T), H.BF16), False, False
-        want, kernel = np.concatenate([block] * reps, 0), "mfma_256x256_m16/pieces"
+        want, kernel = np.concatenate([block] * reps, 0), "mfma_256x256_m16_k64/pieces"
     elif case == "tn_big_a":    # A stored [K, 65664], transposed
         a, b, ta, tb = _periodic(H.encode(np.ascontiguousarray(big0.T), H.BF16), reps, 1), H.encode(np.ascontiguousarray(small.T), H.BF16), True, False
         want, kernel = np.concatenate([block] * reps, 0), "mfma_128x128"
     else:                       # x [512 or 8, K] . W [65664, K]^T
         a, b, ta, tb = H.encode(small, H.BF16), _periodic(H.encode(big0, H.BF16), reps, 0), False, True
         want = np.concatenate([block.T] * reps, 1)
-        kernel = "skinny/pieces" if case == "skinny_big_w" else "mfma_256x256_m16/pieces"
+        kernel = "skinny/pieces" if case == "skinny_big_w" else "mfma_256x256_m16_k64/pieces"
     assert max(a.size, b.size) > 2 ** 31
     got = gpu_matmul(a, b, ta, tb, want_kernel=kernel)
     assert np.array_equal(got, H.encode(want.astype(np.float32), H.BF16))
@@ -983,7 +988,7 @@ def test_bf16_batches_beyond_reach_run_in_pieces_bit_exact():
     b = np.ascontiguousarray(np.concatenate([H.encode(b0, H.BF16)] * (nb // 3), 0))
     at, bt = srt.Tensor(a), srt.Tensor(b)
     out = srt.Tensor(shape=[nb, M, N], dtype=a.dtype)
-    assert query_kernel(at, False, bt, False, out) == "mfma_256x256_m16/pieces"
+    assert query_kernel(at, False, bt, False, out) == "mfma_256x256_m16_k64/pieces"
     srt.current_queue().matmul(at, False, bt, False, out, bias=srt.Tensor(H.encode(bias, H.BF16)),
                                activation=srt.ActivationType.relu)
     block = np.maximum(a0.astype(np.float64) @ b0.astype(np.float64) + bias, 0.0)
