@@ -125,7 +125,7 @@ def main():
                     help="only run three 256 MiB device-to-device copies (known traffic, for scaling the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     ap.add_argument("--only", default=None,
-                    help="run one configuration alone, a few launches, and exit (for profilers): headline, cfg3_tn, "
+                    help="run one configuration alone, a few launches, and exit (for profilers): headline, cfg3_tn, cfg3_nt, "
                          "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, dense_backward, add, add_bias, tanh, cast")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -223,7 +223,7 @@ def main():
 class Bench:
     """The configurations, each as one prepared foreign call per step."""
 
-    SECONDARY = ("cfg3_tn", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1")
+    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1")
 
     def __init__(self, srt, native, q):
         self.srt, self.native, self.q = srt, native, q
@@ -278,6 +278,15 @@ class Bench:
             call, kernel = self.prepared(at, True, h["b"], False, c)
             return {"name": "cfg3 bf16 8192^3 transposeLhs", "call": call, "kernel": kernel, "flops": 2.0 * n ** 3,
                     "bytes": 3 * n * n * 2, "bound": "mfma", "dtype": "bf16", "steps": 40}
+        if name == "cfg3_nt":
+            h = self.headline()
+            n = 8192
+            bt = srt.Tensor(np.ascontiguousarray(h["b_st"].T))
+            c = srt.Tensor(shape=[n, n], dtype=np.uint16)
+            call, kernel = self.prepared(h["a"], False, bt, True, c)
+            return {"name": "cfg3 bf16 8192^3 transposeRhs (the dX product of the backward pass)", "call": call,
+                    "kernel": kernel, "flops": 2.0 * n ** 3, "bytes": 3 * n * n * 2, "bound": "mfma", "dtype": "bf16",
+                    "steps": 40}
         if name == "cfg4_dense":
             g = rng(3)
             x = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))

@@ -168,7 +168,12 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
   const int S = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least four)
 
   // per-XCD start of the k walk for an A stored k x m (see gemm_ring_kernel)
-  const int rot = A_KC ? 0 : (int)(((unsigned)(blockIdx.x & 7) * (unsigned)S) / 8u);
+#ifndef SRT_M16D_ROTATE   // measurement builds: 0 never, 1 always
+  constexpr bool rotate = !A_KC;
+#else
+  constexpr bool rotate = SRT_M16D_ROTATE != 0;
+#endif
+  const int rot = rotate ? (int)(((unsigned)(blockIdx.x & 7) * (unsigned)S) / 8u) : 0;
   auto stage_of = [&](int r) {
     int e = r + rot;
     e = e >= S ? e - S : e;
@@ -293,8 +298,13 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
             }
             SRT_FENCE();
           }
+#ifdef SRT_M16D_SWAP_OPERANDS   // measurement builds: A fragment first (accumulator tiles come out untransposed)
+          if constexpr (FIRST) mfma16_first<T>(acc[4 * AH + i][j], af[4 * AH + i], bf[j]);
+          else mfma16<T>(acc[4 * AH + i][j], af[4 * AH + i], bf[j]);
+#else
           if constexpr (FIRST) mfma16_first<T>(acc[4 * AH + i][j], bf[j], af[4 * AH + i]);
           else mfma16<T>(acc[4 * AH + i][j], bf[j], af[4 * AH + i]);
+#endif
           if (ld >= 0) {
             SRT_FENCE();
             const int si = LOADS == 3 ? Loader<B_KC>::sindex(ld) : Loader<A_KC>::sindex(ld);
@@ -302,12 +312,14 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
             if (LOADS == 3) ring::load_to_lds_at_m0(rb, lb.voff[Loader<B_KC>::vindex(ld)], so);
             else ring::load_to_lds_at_m0(ra, la.voff[Loader<A_KC>::vindex(ld)], so);
           }
-          if (OWN) {
-            if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
-            if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.template read<H>(ua, 4 + ((u - 8) >> 1));
-          } else {
-            if (u < 16 && (u & 3) == 1) af[u >> 2] = fa.template read<H>(ua, u >> 2);
-            if (u < 16 && (u & 3) == 3) bf[u >> 2] = fb.template read<H>(ub, u >> 2);
+          if (!(SRT_ABLATE & 4) || FIRST) {   // (measurement builds can keep the first super-stage's fragments)
+            if (OWN) {
+              if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
+              if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.template read<H>(ua, 4 + ((u - 8) >> 1));
+            } else {
+              if (u < 16 && (u & 3) == 1) af[u >> 2] = fa.template read<H>(ua, u >> 2);
+              if (u < 16 && (u & 3) == 3) bf[u >> 2] = fb.template read<H>(ub, u >> 2);
+            }
           }
           ev(u);
           SRT_FENCE();
@@ -353,7 +365,8 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
         if (u == 25) tb = x + Loader<B_KC>::wave_share(wave);
       });
       // ---- sync: all of super-stage s is in registers, A_{s+1} and B_{s+1} have landed ----
-      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (SRT_ABLATE & 1) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       SRT_FENCE();
       // ---- phase 3: k half 1, A tiles 4-7; the loads of B_{s+2}; reads of super-stage s + 1 ----
       phase(C1{}, std::false_type{}, std::false_type{}, C0{}, C3{}, xa1, xb1, tb, so_b0, so_b1, so_b2, so_b3, [&](int u) __attribute__((always_inline)) {
