@@ -28,6 +28,7 @@ struct GemmProblem {
   int bias_per_row;  // 0: bias indexed by column n (the Dense case); 1: by row m (after a C^T flip)
   int activation;    // srtActivation
   float coef;
+  int tile_n;        // kernel-specific: columns per workgroup when a launcher narrows its tile (0: the kernel's own)
 };
 
 // ---- element codecs ---------------------------------------------------------------------
@@ -183,6 +184,19 @@ inline hipError_t ensure_lds_limit(const void* kernel, int bytes, std::atomic<ui
   e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
   if (e == hipSuccess) done.fetch_or(bit, std::memory_order_relaxed);
   return e;
+}
+
+// Compute units of the current device (cached per device).
+inline int compute_units() {
+  static std::atomic<int> cached[32];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return 256;
+  int n = cached[device & 31].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+    cached[device & 31].store(n, std::memory_order_relaxed);
+  }
+  return n;
 }
 
 // ---- launchers (one per kernel family), defined in the .hip files ------------------------

@@ -813,19 +813,6 @@ inline bool ring_fits(const GemmProblem& p, bool a_kc, bool b_kc) {
   return true;
 }
 
-// Compute units of the current device (cached per device).
-inline int compute_units() {
-  static std::atomic<int> cached[32];
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess) return 256;
-  int n = cached[device & 31].load(std::memory_order_relaxed);
-  if (n == 0) {
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
-    cached[device & 31].store(n, std::memory_order_relaxed);
-  }
-  return n;
-}
-
 // Workgroups of the persistent grid: one per compute unit (a workgroup takes a whole unit's LDS),
 // a multiple of 8 because the XCD-aware tile order wants the stride between a workgroup's tiles
 // to be one -- and, when the tiles do not fill the last round, only as many as spread them evenly

@@ -111,7 +111,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, h = lane >> 5;
-  const int n0 = blockIdx.x * (32 * NW);
+  // columns of this workgroup: 32 NW, or fewer (a multiple of 8) when the launcher narrowed the tile so that
+  // the workgroups come out even over the compute units; what lies beyond is neither loaded nor stored
+  const int cols = (!W_MN && p.tile_n > 0) ? p.tile_n : 32 * NW;
+  const int n0 = blockIdx.x * cols;
   const int bz = blockIdx.y;
 
   const uint16_t* X = (const uint16_t*)p.A + (long long)bz * p.sab;
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     } else {
       wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
       const int n = n0 + row;
-      wvoff[i] = n < p.N ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * 8) * 2) : SK_OOB;
+      wvoff[i] = (n < p.N && row < cols) ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * 8) * 2) : SK_OOB;
     }
   }
 #pragma unroll
@@ -289,7 +292,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 #pragma unroll
   for (int t = 0; t < NW; ++t) {
     const int n = n0 + 32 * t + r;
-    if (n >= p.N) continue;
+    if (n >= p.N || 32 * t + r >= cols) continue;
     const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -314,7 +317,8 @@ hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
   constexpr int lds_bytes = SkinnyShape<XR, NW>::LDS;
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kernel, dim3((p.N + 32 * NW - 1) / (32 * NW), p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
+  const int cols = (!W_MN && p.tile_n > 0) ? p.tile_n : 32 * NW;
+  hipLaunchKernelGGL(kernel, dim3((p.N + cols - 1) / cols, p.batch), dim3(SK_WAVES * 64), lds_bytes, stream, p);
   return launch_status(stream);
 }
 
@@ -333,11 +337,21 @@ hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
   if (p.M <= 16) return launch_skinny_shape<T, 16, 1>(p, stream);
   // two W tiles per workgroup once that still gives most CUs a workgroup (192 of them)
   const long long wide_groups = (long long)((p.N + 63) / 64) * p.batch;
+  // One such workgroup fits a compute unit, so with fewer workgroups than units the rest idle and the weight
+  // streams that much slower (14336 columns: 224 workgroups of 64, 23.5 us; the kernel of 32 columns, two
+  // workgroups per unit, is no better because x then crosses L2 -> LDS twice as often).  When the columns
+  // allow, the tile is narrowed to a multiple of 8 columns that gives every unit one workgroup: 14336 = 256 x 56.
+  GemmProblem q = p;
+  if (wide_groups >= 192 && p.batch == 1) {
+    const int cus = compute_units();
+    const int even = 8 * (int)((p.N + 8LL * cus - 1) / (8LL * cus));
+    if (even > 32 && even < 64) q.tile_n = even;
+  }
   if (p.M <= 32) {
-    if (wide_groups >= 192) return launch_skinny_shape<T, 32, 2>(p, stream);
+    if (wide_groups >= 192) return launch_skinny_shape<T, 32, 2>(q, stream);
     return launch_skinny_shape<T, 32, 1>(p, stream);
   }
-  if (wide_groups >= 192) return launch_skinny_shape<T, 64, 2>(p, stream);
+  if (wide_groups >= 192) return launch_skinny_shape<T, 64, 2>(q, stream);
   return launch_skinny_shape<T, 64, 1>(p, stream);
 }
 

@@ -58,7 +58,7 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
   p->scm = (long long)od->strides[r]; p->scn = (long long)od->strides[r + 1];
   p->scb = rank == 3 ? (long long)od->strides[0] : 0;
   p->bias = nullptr; p->sbias = 0; p->bias_per_row = 0;
-  p->activation = activation; p->coef = (float)coef;
+  p->activation = activation; p->coef = (float)coef; p->tile_n = 0;
   if (bias) {
     if (!biasd || !biasd->shape || !biasd->strides) return srtErrorInvalidValue;
     if (biasd->type != od->type) return srtErrorNotSupported;
