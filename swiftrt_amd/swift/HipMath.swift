@@ -27,7 +27,7 @@ extension HipQueue {
         }
       }
     }
-    HipPlatform.cpuFallback(status) { $0.add(lhs, rhs, &out) }
+    cpuFallback(status) { $0.add(lhs, rhs, &out) }
   }
 
   // tensor Element (CudaMath.swift:128-146)
@@ -36,12 +36,20 @@ extension HipQueue {
   ) where E.Value: AdditiveArithmetic {
     guard useGpu else { cpu_add(lhs, rhs, &out); return }
     let element = E.stored(value: rhs)
-    let status = out.withMutableTensor(using: self) { o, oDesc in
-      lhs.withTensor(using: self) { l, lDesc in
-        withUnsafePointer(to: element) { srtAddTE(l, lDesc, $0, o, oDesc, stream) }
+    var status: srtStatus
+    if canFlatten(lhs, out) {
+      // dense operand and result: the flat tensor-element form (srtAddTEFlat, math_api.h:95-100)
+      status = withUnsafePointer(to: element) {
+        srtAddTEFlat(lhs.deviceRead(using: self), E.type, $0, out.deviceReadWrite(using: self), out.count, stream)
+      }
+    } else {
+      status = out.withMutableTensor(using: self) { o, oDesc in
+        lhs.withTensor(using: self) { l, lDesc in
+          withUnsafePointer(to: element) { srtAddTE(l, lDesc, $0, o, oDesc, stream) }
+        }
       }
     }
-    HipPlatform.cpuFallback(status) { $0.add(lhs, rhs, &out) }
+    cpuFallback(status) { $0.add(lhs, rhs, &out) }
   }
 
   //--------------------------------------------------------------------------
@@ -58,7 +66,7 @@ extension HipQueue {
         rhs.withTensor(using: self) { r, rDesc in native(l, lDesc, r, rDesc, o, oDesc, stream) }
       }
     }
-    HipPlatform.cpuFallback(status, fallback)
+    cpuFallback(status, fallback)
   }
 
   @inlinable public func subtract<S, E>(_ lhs: Tensor<S, E>, _ rhs: Tensor<S, E>, _ out: inout Tensor<S, E>)
@@ -87,7 +95,7 @@ extension HipQueue {
     let status = out.withMutableTensor(using: self) { o, oDesc in
       x.withTensor(using: self) { a, aDesc in native(a, aDesc, o, oDesc, stream) }
     }
-    HipPlatform.cpuFallback(status, fallback)
+    cpuFallback(status, fallback)
   }
 
   @inlinable public func neg<S, E>(_ x: Tensor<S, E>, _ out: inout Tensor<S, E>)
@@ -107,7 +115,7 @@ extension HipQueue {
     let status = out.withMutableTensor(using: self) { o, oDesc in
       x.withTensor(using: self) { a, aDesc in srtCopy(a, aDesc, o, oDesc, stream) }
     }
-    HipPlatform.cpuFallback(status) { $0.copy(from: x, to: &out) }
+    cpuFallback(status) { $0.copy(from: x, to: &out) }
   }
 
   /// fill(_:with:) of a dense tensor (role of CudaFill.swift's srtFillFlat call)
@@ -117,7 +125,7 @@ extension HipQueue {
     let status = withUnsafePointer(to: stored) {
       srtFillFlat(E.type, out.deviceReadWrite(using: self), $0, out.count, stream)
     }
-    HipPlatform.cpuFallback(status) { $0.fill(&out, with: element) }
+    cpuFallback(status) { $0.fill(&out, with: element) }
   }
 
   //--------------------------------------------------------------------------

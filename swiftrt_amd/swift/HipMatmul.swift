@@ -80,7 +80,7 @@ extension HipQueue {
         }
       }
     }
-    HipPlatform.cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
+    cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
   }
 
   //--------------------------------------------------------------------------
@@ -98,7 +98,7 @@ extension HipQueue {
         }
       }
     }
-    HipPlatform.cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
+    cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
   }
 
   //--------------------------------------------------------------------------
@@ -166,7 +166,7 @@ where E: StorageElement, E.Value: StorageElement & Numeric {
         }
       }
     }
-    HipPlatform.cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
+    cpuFallback(status) { $0.matmul(lhs, transposeLhs, rhs, transposeRhs, &result) }
     queue.diagnostic(.queueGpu, "matmul plan: \(String(cString: name))", categories: .queueGpu)
   }
 }

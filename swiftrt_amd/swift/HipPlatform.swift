@@ -9,62 +9,135 @@
 //     #elseif canImport(SwiftRTCuda) ...
 //
 // Types here fill the roles of platform/cuda/device/{CudaPlatform,CudaDevice,CudaQueue,
-// CudaEvent}.swift.  They were written against include/srt_hip.h; this environment has no
-// Swift toolchain, so they have not been compiled.
+// CudaEvent}.swift and are written requirement by requirement against the protocols in
+// platform/common/Platform.swift:37-71, :280-330 and platform/common/DeviceQueue.swift:22-82
+// (`Logging` and `deviceName` have default implementations there: common/Log.swift:200-207,
+// DeviceQueue.swift:129-133).  They import the C module of include/srt_hip.h.
+//
+// UNCOMPILED: this environment has no Swift toolchain.  The sources have been checked against
+// the protocol declarations by reading, not by a compiler.
 //******************************************************************************
 import Foundation
 import SwiftRTHip
 
 //==============================================================================
-/// hipCheck: role of cudaCheck (CudaPlatform.swift:180-193).  Any status other than success
-/// is a hard error: report and trap.
+/// hipCheck: role of cudaCheck(cudaError_t) (CudaPlatform.swift:180-193).  Any status other
+/// than success is a hard error: log on the current queue and trap.
 @inlinable public func hipCheck(
-  _ status: srtStatus, file: String = #file, function: String = #function, line: Int = #line
+  _ status: srtStatus,
+  file: String = #file,
+  function: String = #function,
+  line: Int = #line
 ) {
   if status != srtSuccess {
-    let name = String(cString: srtGetStatusString(status))
+    let location = "HIP error in \(file) at \(function):\(line)"
+    let message = String(cString: srtGetStatusString(status))
     _ = srtDeviceSynchronize()
-    fatalError("hip error \(name) in \(function) at \(file):\(line)")
+    currentQueue.writeLog("\(message) at \(location)")
+    fatalError("unrecoverable error")
   }
+}
+
+/// hipCheck(stream): role of cudaCheck(cudaStream_t) (CudaPlatform.swift:160-177).  In DEBUG builds
+/// every launch is followed by a stream synchronization so that asynchronous errors surface at the
+/// call that caused them (the native module built with `make DEBUG=1` does the same on its side).
+@inlinable public func hipCheck(
+  _ stream: srtStream?,
+  file: String = #file,
+  function: String = #function,
+  line: Int = #line
+) {
+  #if DEBUG
+    hipCheck(srtStreamSynchronize(stream), file: file, function: function, line: line)
+  #endif
 }
 
 //==============================================================================
 /// HipPlatform: role of CudaPlatform (CudaPlatform.swift:22-115)
-public final class HipPlatform: ComputePlatform {
+public class HipPlatform: ComputePlatform {
+  // types
   public typealias Storage = DiscreteStorage
-  public static var local = HipPlatform()
-  public static var acceleratorQueueCount: Int = 2
-  public static let startTime = Date()
 
-  public var discreteMemoryDeviceId: Int { 1 }
-  public var devices: [HipDevice]
-  public let name: String
-  @inlinable public static var queueStack: [HipQueue] {
-    get { local.queueStack } set { local.queueStack = newValue }
+  // shared (the static requirements of ComputePlatform, Platform.swift:44-70)
+  public static var cpuQueueCount = 0
+  public static let discreteMemoryDeviceId = 1
+  public static let eventId = AtomicCounter()
+  public static let local = HipPlatform()
+  public static let mainThread = pthread_self()
+  public static let objectId = AtomicCounter()
+  public static let queueId = AtomicCounter()
+  public static let startTime = Date()
+  public static var lastRandomSeed: RandomSeed = generateRandomSeed()
+
+  public static var acceleratorQueueCount: Int = 2 {
+    didSet {
+      precondition(acceleratorQueueCount > 0, "there must be at least 1 accelerator queue")
+    }
   }
+
+  /// for synchronous execution and syncing with the app thread (cpu, no stream)
+  public static let syncQueue =
+    HipQueue(deviceIndex: 0, name: "appThread", queueMode: .sync, useGpu: false)
+
+  // instance state
+  public var devices: [HipDevice]
+  public let logInfo: LogInfo
+  public let name: String
   public var queueStack: [HipQueue]
 
-  @inlinable public init(name: String? = nil) {
-    self.name = name ?? "\(Self.self)"
-    // device 0 is the cpu, as in the reference's numbering
+  /// the shared single-zero storage AD uses for Element.zero (CudaPlatform.swift:60-66)
+  public static let zeroStorage: Storage = {
+    Storage(storedElement: Int64(0), name: "Zero")
+  }()
+
+  @inlinable public init() {
+    // device 0 is the cpu, as in the reference's numbering; HipDevice covers both kinds so that no
+    // existential is needed
     let cpuDevice = HipDevice(index: 0)
     devices = [cpuDevice]
-    var gpuCount: Int32 = 0
-    hipCheck(srtGetDeviceCount(&gpuCount))
-    for i in 1..<Int(gpuCount + 1) { devices.append(HipDevice(index: i)) }
-    // the first gpu queue (or the cpu queue when no gpu is visible) is the default
-    let defaultDevice = gpuCount > 0 ? 1 : 0
-    queueStack = [devices[defaultDevice].queues[0]]
-  }
-
-  /// cpuFallback: role of CudaPlatform.swift:122-144.  srtErrorNotSupported means the native
-  /// module declined the layout or element type; run the same op on the cpu queue instead.
-  @inlinable public static func cpuFallback(_ status: srtStatus, _ body: (HipQueue) -> Void) {
-    if status == srtErrorNotSupported {
-      using(device: 0) { body(currentQueue) }
-    } else {
-      hipCheck(status)
+    if devices[0].queues.count == 0 {
+      devices[0].queues.append(Self.syncQueue)
     }
+
+    queueStack = []
+    var gpuDeviceCount: Int32 = 0
+    hipCheck(srtGetDeviceCount(&gpuDeviceCount))
+    for i in 1..<Int(gpuDeviceCount + 1) {
+      devices.append(HipDevice(index: i))
+    }
+
+    name = "\(Self.self)"
+    logInfo = LogInfo(logWriter: log, logLevel: .error, namePath: name, nestingLevel: 0)
+
+    // the first gpu's queue 0 is the default
+    if gpuDeviceCount > 0 {
+      queueStack = [devices[1].queues[0]]
+    } else {
+      queueStack = [Self.syncQueue]
+      writeLog("There are no '\(self.name)' devices installed", level: .warning)
+    }
+    diagnostic(.device, "default: \(queueStack[0].name)", categories: .device)
+  }
+}
+
+//==============================================================================
+/// cpuFallback: role of CudaPlatform.swift:117-144.  srtErrorNotSupported means the native module
+/// declined the layout or element type: run the same op on the cpu device's queue instead.
+@usableFromInline func _cpuFallback(_ body: (Platform.Device.Queue) -> Void) {
+  let name = currentQueue.deviceName
+  using(device: 0) {
+    currentQueue.diagnostic(
+      .fallback, "unsupported function on \(name) delegated to \(currentQueue.name)",
+      categories: .fallback)
+    body(currentQueue)
+  }
+}
+
+@inlinable public func cpuFallback(_ status: srtStatus, _ body: (Platform.Device.Queue) -> Void) {
+  if status == srtErrorNotSupported {
+    _cpuFallback(body)
+  } else {
+    hipCheck(status)
   }
 }
 
@@ -75,37 +148,56 @@ public final class HipDevice: ComputeDevice {
   public let memoryType: MemoryType
   public let name: String
   public var queues: [HipQueue]
-  public var properties: [String]
 
   @inlinable public init(index: Int) {
     let isCpu = index == 0
     self.index = index
-    self.name = isCpu ? "cpu:0" : "gpu:\(index - 1)"
+    self.name = "dev:\(index)"
     self.memoryType = isCpu ? .unified : .discrete
-    properties = []
     queues = []
+
+    let description = isCpu ? getCpuProperties() : getHipDeviceProperties()
+    diagnostic(.device, "\(name) \(description)", categories: .device)
+
     if isCpu {
-      queues.append(HipQueue(deviceIndex: index, name: "\(name)_q0", queueMode: .sync, useGpu: false))
-    } else {
-      var p = srtDeviceProperties()
-      hipCheck(srtGetDeviceProperties(&p, Int32(index - 1)))
-      let gpu = withUnsafePointer(to: &p.name) {
-        $0.withMemoryRebound(to: CChar.self, capacity: 256) { String(cString: $0) }
+      for i in 0..<Platform.cpuQueueCount {
+        queues.append(
+          HipQueue(deviceIndex: index, name: "\(name)_q\(i)", queueMode: .async, useGpu: false))
       }
-      properties = ["[type: \(gpu), multiprocessors: \(p.multiProcessorCount), "
-        + "memory: \(p.totalGlobalMem >> 30) GB, addressing: \(memoryType)]"]
-      for i in 0..<HipPlatform.acceleratorQueueCount {
-        queues.append(HipQueue(deviceIndex: index, name: "\(name)_q\(i)", queueMode: .async, useGpu: true))
+    } else {
+      for i in 0..<Platform.acceleratorQueueCount {
+        queues.append(
+          HipQueue(deviceIndex: index, name: "\(name)_q\(i)", queueMode: .async, useGpu: true))
       }
     }
   }
 
+  /// device 0 is the cpu, so the gpu hardware index is one less
   @inlinable public func select() { hipCheck(srtSetDevice(Int32(index - 1))) }
+
+  @inlinable func getCpuProperties() -> String {
+    let info = ProcessInfo.processInfo
+    let oneGB = UInt64(1) << 30
+    return "[type: cpu, cores: \(info.activeProcessorCount), memory: "
+      + "\(info.physicalMemory / oneGB + 1) GB, addressing: \(memoryType)]"
+  }
+
+  @inlinable func getHipDeviceProperties() -> String {
+    var props = srtDeviceProperties()
+    hipCheck(srtGetDeviceProperties(&props, Int32(index - 1)))
+    let deviceName = withUnsafePointer(to: &props.name) {
+      $0.withMemoryRebound(to: UInt8.self, capacity: MemoryLayout.size(ofValue: props.name)) {
+        String(cString: $0)
+      }
+    }
+    return "[type: \(deviceName), multiprocessors: \(props.multiProcessorCount), "
+      + "memory: \(props.totalGlobalMem >> 30) GB, addressing: \(memoryType)]"
+  }
 }
 
 //==============================================================================
-/// HipDeviceMemory: role of CudaDeviceMemory (CudaDevice.swift:96-162).  The Swift object
-/// owns the pointer; the native module keeps no reference to tensor memory.
+/// HipDeviceMemory: role of CudaDeviceMemory (CudaDevice.swift:96-162).  The Swift object owns
+/// the pointer; the native module keeps no reference to tensor memory.
 public final class HipDeviceMemory: DeviceMemory {
   public let buffer: UnsafeMutableRawBufferPointer
   public let deviceIndex: Int
@@ -114,43 +206,85 @@ public final class HipDeviceMemory: DeviceMemory {
   public let type: MemoryType
   public var version: Int
   public let isReference: Bool
+  /// the stream the block was allocated on: the allocator reuses it there at once
+  public let stream: srtStream?
 
-  @inlinable public var mutablePointer: UnsafeMutableRawPointer { UnsafeMutableRawPointer(buffer.baseAddress!) }
-  @inlinable public var pointer: UnsafeRawPointer { UnsafeRawPointer(buffer.baseAddress!) }
+  @inlinable public var mutablePointer: UnsafeMutableRawPointer {
+    UnsafeMutableRawPointer(buffer.baseAddress!)
+  }
+  @inlinable public var pointer: UnsafeRawPointer {
+    UnsafeRawPointer(buffer.baseAddress!)
+  }
 
   @inlinable public init(_ deviceIndex: Int, _ byteCount: Int, _ stream: srtStream?) {
     self.deviceIndex = deviceIndex
-    // pad to the widest vector access, as CudaDevice.swift:141-142 does
-    let padded = roundUp(byteCount, multiple: 32)
-    var p: UnsafeMutableRawPointer?
-    hipCheck(srtDeviceAllocate(&p, padded, stream))
-    buffer = UnsafeMutableRawBufferPointer(start: p, count: byteCount)
-    type = .discrete
-    version = -1
-    isReference = false
+    self.stream = stream
+    // pad to the widest vector access (32 bytes, as CudaDevice.swift:141-142 does with double4)
+    let paddedByteCount = roundUp(byteCount, multiple: 32)
+    var devicePointer: UnsafeMutableRawPointer?
+    hipCheck(srtDeviceAllocate(&devicePointer, paddedByteCount, stream))
+    self.buffer = UnsafeMutableRawBufferPointer(start: devicePointer!, count: byteCount)
+    self.type = .discrete
+    self.isReference = false
+    self.version = -1
+    self.releaseMessage = nil
   }
 
-  @inlinable deinit { if !isReference { hipCheck(srtDeviceFree(buffer.baseAddress!)) } }
+  /// The free is ordered on the allocating stream.  Storage that was last written or read on another
+  /// queue has already made this queue wait for that work (DiscreteStorage.swift:271-296 synchronizes
+  /// replicas across queues with events before a buffer changes hands).
+  @inlinable deinit {
+    hipCheck(srtDeviceFree(buffer.baseAddress!))
+    #if DEBUG
+      if let name = name, let msg = releaseMessage {
+        diagnostic(.release, "\(name)\(msg)", categories: .dataAlloc)
+      }
+    #endif
+  }
 }
 
 //==============================================================================
 /// HipEvent: role of CudaEvent (CudaEvent.swift:23-75)
-public final class HipEvent: QueueEvent {
-  public let handle: srtEvent
-  public var recordedTime: Date?
+public class HipEvent: QueueEvent, Logging {
+  public let id = Platform.eventId.next
+  // used to synchronize with a cpu async queue
+  @usableFromInline let cpuEvent: DispatchSemaphore
+  // used to synchronize with a stream
+  @usableFromInline let handle: srtEvent
 
-  @inlinable public init(options: QueueEventOptions) {
-    var e: srtEvent?
-    hipCheck(srtEventCreate(&e, options.contains(.timing) ? 1 : 0))
-    handle = e!
+  @inlinable public init(recordedOn queue: HipQueue, options: QueueEventOptions = []) {
+    // blocking only for the async cpu case; signaled for sync cpu and streams so wait() falls through
+    let value = queue.deviceIndex == 0 && queue.mode == .async ? 0 : 1
+    cpuEvent = DispatchSemaphore(value: value)
+    var temp: srtEvent?
+    hipCheck(srtEventCreate(&temp, options.contains(.timing) ? 1 : 0))
+    handle = temp!
   }
-  @inlinable deinit { _ = srtEventDestroy(handle) }
+
+  @inlinable deinit {
+    _ = srtEventDestroy(handle)
+  }
+
+  /// only called by the cpu async queue implementation
+  @inlinable public func signal() {
+    cpuEvent.signal()
+    _ = srtEventRecord(handle, nil)
+  }
+
+  @inlinable public func wait() {
+    // wait for the first occurrence, then let all other waiters through
+    cpuEvent.wait()
+    cpuEvent.signal()
+    _ = srtEventSynchronize(handle)
+  }
+
   @inlinable public var occurred: Bool { srtEventQuery(handle) == srtSuccess }
-  @inlinable public func wait() { hipCheck(srtEventSynchronize(handle)) }
 }
 
 //==============================================================================
 /// HipQueue: role of CudaQueue (CudaQueue.swift:22-196): one non-blocking stream on one device.
+/// The functions it overrides live in HipMatmul.swift and HipMath.swift; everything else comes
+/// from CpuFunctions' defaults.
 public final class HipQueue: DeviceQueue, CpuFunctions {
   public let creatorThread: Thread
   public var defaultQueueEventOptions: QueueEventOptions
@@ -162,11 +296,19 @@ public final class HipQueue: DeviceQueue, CpuFunctions {
   public let queue: DispatchQueue
   public let group: DispatchGroup
   public let useGpu: Bool
+
   public let gpuId: Int
   public let stream: srtStream?
   @inlinable public var usesCpu: Bool { !useGpu }
+  /// DeviceQueue.deviceName (a default exists, DeviceQueue.swift:129-133; spelled out for the record)
+  @inlinable public var deviceName: String { platform.devices[deviceIndex].name }
 
-  @inlinable public init(deviceIndex: Int, name: String, queueMode: DeviceQueueMode, useGpu: Bool) {
+  @inlinable public init(
+    deviceIndex: Int,
+    name: String,
+    queueMode: DeviceQueueMode,
+    useGpu: Bool
+  ) {
     self.id = Platform.queueId.next
     self.name = name
     self.deviceIndex = deviceIndex
@@ -178,46 +320,84 @@ public final class HipQueue: DeviceQueue, CpuFunctions {
     self.queue = DispatchQueue(label: name)
     self.group = DispatchGroup()
     self.useGpu = useGpu
+
     if useGpu {
       hipCheck(srtSetDevice(Int32(gpuId)))
-      var s: srtStream?
-      hipCheck(srtStreamCreate(&s))     // non-blocking, default priority
-      stream = s
+      var hipStream: srtStream?
+      hipCheck(srtStreamCreate(&hipStream))   // non-blocking, default priority
+      stream = hipStream
     } else {
-      stream = nil
+      stream = nil   // a cpu queue never reaches the native module (the reference creates a stream here too)
+    }
+    diagnostic(.create, "queue: \(name)", categories: .queueAlloc)
+  }
+
+  @inlinable public func selectDevice() {
+    hipCheck(srtSetDevice(Int32(gpuId)))
+  }
+
+  /// allocate a device memory buffer suitably aligned for any type
+  @inlinable public func allocate(byteCount: Int, heapIndex: Int = 0) -> DeviceMemory {
+    if usesCpu {
+      let buffer = UnsafeMutableRawBufferPointer.allocate(
+        byteCount: byteCount, alignment: MemoryLayout<Int>.alignment)
+      return CpuDeviceMemory(deviceIndex, buffer, memoryType)
+    } else {
+      selectDevice()
+      return HipDeviceMemory(deviceIndex, byteCount, stream)
     }
   }
 
-  @inlinable public func allocate(byteCount: Int, heapIndex: Int = 0) -> DeviceMemory {
-    if usesCpu { return CpuDeviceMemory(deviceIndex, byteCount) }
-    hipCheck(srtSetDevice(Int32(gpuId)))
-    return HipDeviceMemory(deviceIndex, byteCount, stream)
+  @inlinable public func delay(_ interval: TimeInterval) {
+    guard useGpu else {
+      cpu_delay(interval)
+      return
+    }
+    hipCheck(srtDelayStream(interval, stream))
   }
 
   /// role of CudaQueue.copyAsync (CudaQueue.swift:112-153)
   @inlinable public func copyAsync(from src: DeviceMemory, to dst: DeviceMemory) {
     assert(src.buffer.count == dst.buffer.count)
-    let kind: srtMemcpyKind
     switch (src.type, dst.type) {
-    case (.unified, .discrete): kind = srtMemcpyHostToDevice
-    case (.discrete, .unified): kind = srtMemcpyDeviceToHost
-    case (.discrete, .discrete): kind = srtMemcpyDeviceToDevice
-    default:
-      dst.buffer.copyMemory(from: UnsafeRawBufferPointer(src.buffer))
-      return
+    case (.unified, .unified):
+      cpu_copyAsync(from: src, to: dst)
+    case (.unified, .discrete):
+      hipCheck(srtMemcpyAsync(dst.mutablePointer, src.pointer, src.buffer.count, srtMemcpyHostToDevice, stream))
+    case (.discrete, .unified):
+      hipCheck(srtMemcpyAsync(dst.mutablePointer, src.pointer, src.buffer.count, srtMemcpyDeviceToHost, stream))
+    case (.discrete, .discrete):
+      hipCheck(srtMemcpyAsync(dst.mutablePointer, src.pointer, src.buffer.count, srtMemcpyDeviceToDevice, stream))
     }
-    hipCheck(srtMemcpyAsync(dst.mutablePointer, src.pointer, src.buffer.count, kind, stream))
   }
 
   @inlinable public func recordEvent() -> HipEvent {
-    let event = HipEvent(options: defaultQueueEventOptions)
-    if useGpu { hipCheck(srtEventRecord(event.handle, stream)) }
+    let event = HipEvent(recordedOn: self, options: defaultQueueEventOptions)
+    if useGpu {
+      hipCheck(srtEventRecord(event.handle, stream))
+    } else if mode == .async {
+      queue.async(group: group) { event.signal() }
+    }
     return event
   }
+
+  /// causes this queue to wait until the event has occurred
   @inlinable public func wait(for event: HipEvent) {
-    if useGpu { hipCheck(srtStreamWaitEvent(stream, event.handle)) } else { event.wait() }
+    if useGpu {
+      hipCheck(srtStreamWaitEvent(stream, event.handle))
+    } else if mode == .sync {
+      event.wait()
+    } else {
+      queue.async(group: group) { event.wait() }
+    }
   }
+
+  /// the synchronous queue completes work as it is queued, so it is always complete
   @inlinable public func waitForCompletion() {
-    if useGpu { hipCheck(srtStreamSynchronize(stream)) }
+    if useGpu {
+      hipCheck(srtStreamSynchronize(stream))
+    } else if mode == .async {
+      group.wait()
+    }
   }
 }
