@@ -33,6 +33,16 @@ extern "C" {
  * default visibility) */
 #pragma GCC visibility push(default)
 
+/* Enumerations cross the boundary as 32-bit integers.  A caller may hand in a value that is none of the
+ * enumerators (another cudaDataType id, a tiled order): the library answers srtErrorNotSupported or
+ * srtErrorInvalidValue.  In C++ the types get a fixed underlying type so that holding such a value is
+ * well defined; in C an enumeration is an integer anyway. */
+#ifdef __cplusplus
+#define SRT_ENUM(tag) enum tag : int32_t
+#else
+#define SRT_ENUM(tag) enum tag
+#endif
+
 /* ---- status ---------------------------------------------------------------------------- */
 typedef int32_t srtStatus;
 enum {
@@ -53,7 +63,7 @@ const char* srtGetStatusString(srtStatus status);
  * Replaces srtDataType, Modules/SwiftRTCuda/tensor_api.h:28-65.  The values the path uses keep
  * the reference's numeric ids (they are the cudaDataType values) so `E.type` in
  * StorageElement.swift:123-129 ports unchanged. */
-typedef enum {
+typedef SRT_ENUM(srtDataType_e) {
   srtUnknownType = -1,
   srtReal32F = 0,
   srtReal64F = 1,   /* declared for completeness; matmul returns srtErrorNotSupported */
@@ -65,7 +75,7 @@ typedef enum {
  * (tensor_api.h:76); same numeric values as CUBLASLT_ORDER_COL / CUBLASLT_ORDER_ROW, which is
  * what `order.cublas` yields (CudaPlatform.swift:297-311).  Strides are authoritative; order
  * is checked only to reject tiled layouts (anything else -> srtErrorNotSupported). */
-typedef enum { srtOrderCol = 0, srtOrderRow = 1 } srtOrder;
+typedef SRT_ENUM(srtOrder_e) { srtOrderCol = 0, srtOrderRow = 1 } srtOrder;
 
 /* Tensor descriptor.  Replaces srtTensorDescriptor, tensor_api.h:70-87, field for field, so
  * Tensor.withTensor (CudaExtensions.swift:24-84) builds it the same way.  shape / strides /
@@ -84,7 +94,7 @@ typedef struct {
 
 /* Epilogue activation.  Case order and values follow ActivationType,
  * Sources/SwiftRTCore/platform/common/FunctionProperties.swift:44-51 (rawValue ports 1:1). */
-typedef enum {
+typedef SRT_ENUM(srtActivation_e) {
   srtActivationSigmoid = 0,     /* 1 / (1 + exp(-x))                                         */
   srtActivationRelu = 1,        /* max(x, 0)                                                 */
   srtActivationTanh = 2,
@@ -162,7 +172,7 @@ srtStatus srtDeviceEmptyCache(void);
 srtStatus srtHostAllocate(void** hostPtr, size_t size);
 srtStatus srtHostFree(void* hostPtr);
 
-typedef enum {
+typedef SRT_ENUM(srtMemcpyKind_e) {
   srtMemcpyHostToDevice = 1,
   srtMemcpyDeviceToHost = 2,
   srtMemcpyDeviceToDevice = 3

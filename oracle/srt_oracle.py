@@ -19,7 +19,7 @@ ACC_VALUE, ACC_F32 = 0, 1
 SIGMOID, RELU, TANH, CLIPPED_RELU, ELU, IDENTITY = range(6)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libsrt_oracle.so")
+_LIB_PATH = os.environ.get("SRT_ORACLE_LIBRARY") or os.path.join(_HERE, "libsrt_oracle.so")
 _lib = None
 
 
