@@ -37,11 +37,23 @@ class HipQueue;
 
 class HipDeviceMemory {
  public:
-  HipDeviceMemory(size_t bytes, srtStream stream) : bytes_(bytes) {
+  HipDeviceMemory(size_t bytes, srtStream stream) : bytes_(bytes), stream_(stream), last_stream_(stream) {
     size_t padded = (bytes + 31) / 32 * 32;   // CudaDevice.swift:141-142
     check(srtDeviceAllocate(&ptr_, padded ? padded : 32, stream), "srtDeviceAllocate");
   }
-  ~HipDeviceMemory() { srtDeviceFree(ptr_); }
+  // The free hands the block back to the allocating stream at once: work another stream still has in
+  // flight on it is ordered first (event on that stream, wait on the allocating one).
+  ~HipDeviceMemory() {
+    if (last_stream_ != stream_) {
+      srtEvent e = nullptr;
+      if (srtEventCreate(&e, 0) == srtSuccess) {
+        if (srtEventRecord(e, last_stream_) == srtSuccess) (void)srtStreamWaitEvent(stream_, e);
+        (void)srtEventDestroy(e);
+      }
+    }
+    srtDeviceFree(ptr_);
+  }
+  void used_on(srtStream stream) { last_stream_ = stream; }
   HipDeviceMemory(const HipDeviceMemory&) = delete;
   HipDeviceMemory& operator=(const HipDeviceMemory&) = delete;
   void* pointer() const { return ptr_; }
@@ -50,6 +62,7 @@ class HipDeviceMemory {
  private:
   void* ptr_ = nullptr;
   size_t bytes_;
+  srtStream stream_, last_stream_;
 };
 
 class HipEvent {
@@ -198,6 +211,7 @@ class Tensor {
       q.wait(e);
     }
     s.last_queue = &q;
+    s.device->used_on(q.stream());
     if (s.device_version < s.host_version) {
       q.copy_to_device(s.device->pointer(), s.host.data(), s.host.size() * sizeof(E));
       q.wait_for_completion();

@@ -65,10 +65,17 @@ class HipDeviceMemory:
         self.pointer = p.value
         self.version = -1
         self.name = None
+        self.queue = queue          # the allocator hands the block back to this queue's stream at once
+        self.last_queue = queue     # the queue that used the block last (kept up to date by the tensor)
 
     def __del__(self):
+        """srtDeviceFree makes the block reusable at once on the stream it was allocated on.  Work that
+        another queue still has in flight on it must come first: the allocating stream is made to wait for
+        an event recorded on that queue (the contract stated with srtDeviceAllocate in the header)."""
         try:
             if self.pointer:
+                if self.last_queue is not None and self.last_queue is not self.queue:
+                    self.queue.wait(self.last_queue.record_event())
                 native.lib().srtDeviceFree(ctypes.c_void_p(self.pointer))
                 self.pointer = None
         except Exception:

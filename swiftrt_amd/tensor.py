@@ -194,6 +194,7 @@ class Tensor:
         if s.last_queue is not None and s.last_queue is not queue:
             queue.wait(s.last_queue.record_event())   # cross-queue sync, DiscreteStorage.swift:271-296
         s.last_queue = queue
+        s.device.last_queue = queue
 
     def device_read(self, queue):
         """Pointer to this view's first element on the queue's device, copying host->device when

@@ -103,6 +103,32 @@ def test_events_delay_and_cross_queue_wait():
     assert time.time() - t0 < 5.0
 
 
+def test_block_used_on_another_queue_is_not_handed_back_early():
+    """A block is reusable at once on the stream it was allocated on.  When its last use was on ANOTHER
+    queue, the host object orders that queue's work before the free: the allocating queue, which gets the
+    same block straight back, is held until the other queue is through with it."""
+    import gc
+    p = srt.HipPlatform.local()
+    q0, q1 = p.devices[1].queues[0], p.devices[1].queues[1]
+    n = 1 << 18
+    t = srt.Tensor(np.zeros(n, np.float32))
+    t.device_read(q0)                                  # allocated on queue 0
+    ptr = t.storage.device.pointer
+    q0.wait_for_completion()
+    start = q0.record_event(timing=True)
+    q1.delay(0.05)                                     # queue 1 is busy ...
+    t.device_read_write(q1)                            # ... and is the last user of the block
+    del t
+    gc.collect()                                       # freed while queue 1 still spins
+    u = srt.Tensor(np.ones(n, np.float32))
+    u.device_read(q0)                                  # same size class, same stream: the same block
+    assert u.storage.device.pointer == ptr
+    done = q0.record_event(timing=True)
+    done.wait()
+    assert done.elapsed_ms_since(start) >= 45.0        # queue 0 waited for queue 1's delay before reusing it
+    assert np.array_equal(u.array(), np.ones(n, np.float32))
+
+
 def test_storage_migration_flags():
     # DiscreteStorage's lazy replica movement: first device read copies host->device, a second does not;
     # reading on the host after a device write copies back once
