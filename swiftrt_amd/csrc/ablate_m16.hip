@@ -5,6 +5,8 @@
 //                         registers, 8 every workgroup requests tile 0)
 //   -DABL_NS=<3|4|5>      ring depth (prefetch distance NS - 1 stages)
 //   -DABL_DEEP=1          the 64-deep form of the kernel (gemm_mfma_m16d.h; no ablation switches)
+//   -DABL_TAIL=1          (with ABL_DEEP) the tail-sharing form; every element of its result is then compared
+//                         with the plain 64-deep kernel's
 //   -DABL_AKC / -DABL_BKC operand layouts (defaults 1 / 0: the headline's row-major A and B)
 // Run: ablate_m16 [normal|zero] [M N K]; operands ~ N(0,1)/sqrt(K) (generated on the device) or zeros.
 // Prints one line: variant, data, median and minimum time per launch, TFLOP/s, and (unablated builds) the
@@ -24,6 +26,9 @@
 #endif
 #ifndef ABL_DEEP
 #define ABL_DEEP 0
+#endif
+#ifndef ABL_TAIL
+#define ABL_TAIL 0
 #endif
 #ifndef ABL_AKC
 #define ABL_AKC 1
@@ -70,6 +75,20 @@ float bf16_to_float(uint16_t h) {
 
 }  // namespace
 
+// The tail-sharing launcher takes its workspace from the library's allocator; this probe stands alone.
+extern "C" srtStatus srtDeviceAllocate(void** ptr, size_t size, srtStream) {
+  static void* block = nullptr;
+  static size_t held = 0;
+  if (size > held) {
+    if (block) (void)hipFree(block);
+    if (hipMalloc(&block, size) != hipSuccess) return srtErrorOutOfMemory;
+    held = size;
+  }
+  *ptr = block;
+  return srtSuccess;
+}
+extern "C" srtStatus srtDeviceFree(void*) { return srtSuccess; }
+
 int main(int argc, char** argv) {
   const bool zero = argc > 1 && strcmp(argv[1], "zero") == 0;
   int M = 8192, N = 8192, K = 8192;
@@ -95,7 +114,8 @@ int main(int argc, char** argv) {
   p.activation = srtActivationIdentity;
 
   auto launch = [&]() {
-    if (ABL_DEEP) CHECK((srt::m16d::launch_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN>(p, 0)));
+    if (ABL_DEEP && ABL_TAIL) CHECK((srt::m16d::launch_tail_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN>(p, 0)));
+    else if (ABL_DEEP) CHECK((srt::m16d::launch_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN>(p, 0)));
     else CHECK((srt::m16::launch_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN, ABL_NS, 8>(p, 0)));
   };
   hipEvent_t e0, e1;
@@ -137,10 +157,42 @@ int main(int argc, char** argv) {
       worst = std::max(worst, fabs(ref - (double)bf16_to_float(hc[(size_t)m * N + n])));
     }
   }
+  long long differing = -1;
+  double worst_pair = 0.0;
+  if (ABL_DEEP && ABL_TAIL && !zero) {
+    std::vector<uint16_t> tail((size_t)M * N), plain((size_t)M * N);
+    CHECK(hipMemcpy(tail.data(), c, tail.size() * 2, hipMemcpyDeviceToHost));
+    CHECK((srt::m16d::launch_kernel<srt::BF16, ABL_AKC != 0, ABL_BKC != 0, srt::m16::EPI_PLAIN>(p, 0)));
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipMemcpy(plain.data(), c, plain.size() * 2, hipMemcpyDeviceToHost));
+    differing = 0;
+    for (size_t i = 0; i < tail.size(); ++i) {
+      if (tail[i] != plain[i]) ++differing;
+      worst_pair = std::max(worst_pair, (double)fabsf(bf16_to_float(tail[i]) - bf16_to_float(plain[i])));
+    }
+  }
+#ifdef SRT_TAIL_TRACE
+  if (ABL_DEEP) {
+    // one more launch, then the piece boundaries of some workgroups relative to the earliest start, in us
+    std::vector<unsigned long long> tr(256 * 16, 0);
+    CHECK(hipMemcpyToSymbol(HIP_SYMBOL(srt::m16d::tail_trace), tr.data(), tr.size() * 8));
+    launch();
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipMemcpyFromSymbol(tr.data(), HIP_SYMBOL(srt::m16d::tail_trace), tr.size() * 8));
+    unsigned long long t0 = ~0ull;
+    for (int w = 0; w < 256; ++w) if (tr[w * 16]) t0 = std::min(t0, tr[w * 16]);
+    for (int w = 0; w < 256; w += (w < 4 ? 1 : 21)) {
+      printf("wg %3d:", w);
+      for (int e = 0; e < 16 && tr[w * 16 + e]; ++e) printf(" %.1f", (double)(tr[w * 16 + e] - t0) / 100.0);
+      printf("\n");
+    }
+  }
+#endif
   printf("ablate=%d deep=%d ns=%d akc=%d bkc=%d %-6s M=%d N=%d K=%d: median %.4f ms %.1f TFLOP/s (min %.4f ms %.1f)", SRT_ABLATE,
-         ABL_DEEP, ABL_NS, ABL_AKC, ABL_BKC, zero ? "zero" : "normal", M, N, K, med, flop / (med * 1e-3) * 1e-12, t[0],
+         ABL_DEEP + 10 * ABL_TAIL, ABL_NS, ABL_AKC, ABL_BKC, zero ? "zero" : "normal", M, N, K, med, flop / (med * 1e-3) * 1e-12, t[0],
          flop / (t[0] * 1e-3) * 1e-12);
   if (worst >= 0.0) printf("  max |error| of 64 samples %.3g (|c| ~ %.2g)", worst, 1.0 / sqrt((double)K) * sqrt((double)K) / sqrt((double)K));
+  if (differing >= 0) printf("  vs plain kernel: %lld of %lld elements differ, largest difference %.3g", differing, (long long)M * N, worst_pair);
   printf("\n");
   return 0;
 }

@@ -214,6 +214,7 @@ hipError_t launch_mfma(const GemmProblem& p, int config, hipStream_t stream);
 // Split-K over the 256 x 256 kernel: number of k parts (0: the problem does not qualify) and launch.
 int mfma_splitk_parts(const GemmProblem& p);
 bool mfma_prefers_splitk(const GemmProblem& p);
+bool mfma_prefers_tail(const GemmProblem& p);
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream);
 
 bool skinny_supported(const GemmProblem& p);

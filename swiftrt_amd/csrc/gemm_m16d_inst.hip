@@ -12,4 +12,14 @@ hipError_t SRT_CAT(launch_m16d, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const Ge
   return m16d::launch<SRT_M16_TYPE, SRT_M16_AKC != 0, SRT_M16_BKC != 0>(p, stream);
 }
 
+// launch_m16d_tail_<type>_<akc><bkc>: the tail-sharing form
+hipError_t SRT_CAT(launch_m16d_tail, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const GemmProblem& p, hipStream_t stream) {
+  return m16d::launch_tail<SRT_M16_TYPE, SRT_M16_AKC != 0, SRT_M16_BKC != 0>(p, stream);
+}
+
+// whether the tail-sharing form applies to `p` (defined once)
+#if SRT_M16_AKC == 0 && SRT_M16_BKC == 0
+bool SRT_CAT(m16d_tail_fits, SRT_M16_TYPE, x, x)(const GemmProblem& p) { return m16d::tail_fits(p); }
+#endif
+
 }  // namespace srt

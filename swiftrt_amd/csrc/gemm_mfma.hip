@@ -67,6 +67,15 @@ SRT_M16P_DECL(F16)
 SRT_M16D_DECL(BF16)
 SRT_M16D_DECL(F16)
 #undef SRT_M16D_DECL
+#define SRT_M16DT_DECL(T)                                                      \
+  hipError_t launch_m16d_tail_##T##_00(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_tail_##T##_01(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_tail_##T##_10(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_tail_##T##_11(const GemmProblem&, hipStream_t);
+SRT_M16DT_DECL(BF16)
+SRT_M16DT_DECL(F16)
+#undef SRT_M16DT_DECL
+bool m16d_tail_fits_BF16_xx(const GemmProblem&);   // (the answer does not depend on the element type)
 hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_F16_10(const GemmProblem&, hipStream_t);
@@ -504,6 +513,19 @@ hipError_t launch_m16d(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t s
 
 // the 128 x 256 form of the 16x16x32 ring kernel (k-contiguous A)
 template <typename T>
+hipError_t launch_m16d_tail(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) {
+    if (a_kc && b_kc) return launch_m16d_tail_BF16_11(p, stream);
+    if (a_kc) return launch_m16d_tail_BF16_10(p, stream);
+    if (b_kc) return launch_m16d_tail_BF16_01(p, stream);
+    return launch_m16d_tail_BF16_00(p, stream);
+  }
+  if (a_kc && b_kc) return launch_m16d_tail_F16_11(p, stream);
+  if (a_kc) return launch_m16d_tail_F16_10(p, stream);
+  if (b_kc) return launch_m16d_tail_F16_01(p, stream);
+  return launch_m16d_tail_F16_00(p, stream);
+}
+template <typename T>
 hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16h_BF16_11(p, stream) : launch_m16h_BF16_10(p, stream);
   return b_kc ? launch_m16h_F16_11(p, stream) : launch_m16h_F16_10(p, stream);
@@ -519,6 +541,7 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 5: return launch_m16<T>(p, a_kc, b_kc, stream);
     case 6: return launch_m16h<T>(p, b_kc, stream);
     case 9: return launch_m16d<T>(p, a_kc, b_kc, stream);
+    case 10: return launch_m16d_tail<T>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     case 7: return launch_any_layout<T, 128, 128>(p, stream);
     case 8: return launch_any_layout<T, 64, 64>(p, stream);
@@ -557,7 +580,7 @@ static int mfma_layout(const GemmProblem& p) {
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
 // 128 x 256 form for a k-contiguous A, 9: the 16x16x32 kernel with 64-deep staging units), or 0 when the
-// problem does not qualify for it.
+// problem does not qualify for it.  10: tile 9's tail-sharing form.
 int mfma_config(const GemmProblem& p, int tile) {
   if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
     if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
@@ -565,9 +588,13 @@ int mfma_config(const GemmProblem& p, int tile) {
     return tile << 2;
   }
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || (tile > 6 && tile != 9)) return 0;
+  if (layout < 0 || tile < 1 || (tile > 6 && tile != 9 && tile != 10)) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
   if (tile == 9 && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
+  if (tile == 10) {   // left-over tiles to share, k in whole quads, no transcendental activation
+    const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
+    if (trans || !m16d_tail_fits_BF16_xx(p)) return 0;
+  }
   if (tile == 6 && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
@@ -637,8 +664,11 @@ int mfma_select(const GemmProblem& p) {
   // against 51 us for whole tiles).
   const int m_rest = p.M % 256;
   const bool half_nt = p.batch == 1 ? (th >= 96 && rounds_h == 1) : ((m_rest > 0 && m_rest <= 128) || p.K <= 512);
+  // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
+  // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
+  const bool deep = p.K % 64 == 0 && p.K >= 512;
   const bool half_ok = p.K >= 64 && (p.N > 64 || (layout == 2 && p.K >= 512)) &&
-                       (layout == 3 ? half_nt : 6 * rounds_h <= 10 * rounds256);
+                       (layout == 3 ? half_nt : (deep ? 7 : 6) * rounds_h <= 10 * rounds256);
   // Whole tiles: padding up to 256 rows and columns is affordable when the alternative is the 64 x 64
   // kernel on two n- / m-contiguous operands, which it transposes in registers, and the device is at
   // least half full (64 x 8 x 1024 x 256: 13.6 us against 19.6 us), or when the k loop is long, where the
@@ -766,6 +796,35 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 192));
 }
 
+// Whether the heuristic takes the tail-sharing form of the 64-deep kernel (tile 10): the tiles left over
+// after the whole rounds are cut along k so that every compute unit works on them.  Adding up a tile's
+// parts costs about what three quads (768 k) of multiplying do, so it pays for long k loops only.  After
+// whole rounds it buys nothing that stands out of the run-to-run spread: a partly filled round runs at
+// higher clocks than a full one, and the workgroups leave the shared pieces out of step, which costs the
+// whole tiles that follow some of their L2 hits (384 tiles: 151 us against 156; 640 tiles: 241-250 against
+// 242-252; 4096 x 11008 x 4096, 176 tiles left over: 270 against 254) -- unless only a handful of tiles
+// is left over, which would otherwise cost a round of their own (1536 x 11008 x 4096, 258 tiles: 130 against
+// 139 whole and 135 in half tiles).  Otherwise it is taken only where there is no whole round.  Measured against what the other rules pick (us, K = 4096 unless given):
+//   64 tiles (three parts)    1024 x 4096 x 4096: 43 against 47-50 (split-K), K = 8192: 64 against 70
+//   128 tiles (two parts)     x . W^T: 56-59 against 62-66 (half tiles), K = 8192: 97-100 against 117-122;
+//                             x . W: 57-59 against 55-57 (half tiles in one round: those stay), K = 8192: 98-103
+//                             against 103-110
+//   144 tiles                 3072 x 3072 x 4096: 67-69 against 71-73 (whole tiles)
+//   below 64 tiles split-K cuts deeper (32 tiles, K = 16384: 73 against 104); from 160 tiles up whole tiles
+//   are as good (160 tiles: 74-76 against 72-75)
+bool mfma_prefers_tail(const GemmProblem& p) {
+  if (p.K < 4096 || mfma_config(p, 10) == 0) return false;
+  const int layout = mfma_layout(p);
+  const long long cus = compute_units();
+  const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
+  const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
+  const long long left = t256 % cus;
+  if (t256 >= cus) return left > 0 && 8 * left <= cus;   // a handful left over: see above
+  if (left < 64 || left > 160) return false;
+  if (left <= 96) return true;
+  return layout == 3 || (layout & 2) == 0 || p.K >= 8192 || th > cus;
+}
+
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream) {
   const int parts = mfma_splitk_parts(p);
   if (parts < 2) return hipErrorInvalidValue;
@@ -813,6 +872,7 @@ const char* mfma_name(int config) {
     case 5: return "mfma_256x256_m16";
     case 6: return "mfma_128x256_m16";
     case 9: return "mfma_256x256_m16_k64";
+    case 10: return "mfma_256x256_m16_k64_tail";
     case 2: return "mfma_128x128";
     case 7: return "mfma_128x128_any";
     case 8: return "mfma_64x64_any";

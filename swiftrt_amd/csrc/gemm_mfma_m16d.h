@@ -136,8 +136,193 @@ struct FragReader<false> {
   }
 };
 
-template <typename T, bool A_KC, bool B_KC, int EPI>
-__global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
+// The epilogue of the tail-sharing form: m16::store_tile (TM = 8) with switches that are uniform at run time,
+// so that the kernel holds one copy of it and one place where the accumulators are read.  (With a copy per
+// case the compiler moves all 256 accumulators out of their registers once, ahead of the branches, spilling
+// what does not fit: every epilogue then took 23 us instead of 5.)
+//   foreign   1 or 2: the tile's sum is spread over two or three workgroups; the accumulators of the other
+//             one or two (f0, f1: what they published, see publish_accumulators) are added on the way out,
+//             in the order of the parts along k whoever does the adding, streamed from memory two rows of
+//             accumulator tiles ahead
+// Partials are written and read with the agent-scope policy (cache policy operand 16: sc1): another
+// workgroup, maybe on another XCD, reads or wrote them during this launch.
+struct TailStore {
+  __amdgpu_buffer_rsrc_t f0, f1;
+  int foreign;
+  bool own_last;   // foreign = 2: the sum is (f0 + f1) + own instead of (own + f0) + f1
+};
+
+// The accumulators to `mine` as they lie in the registers: [64 accumulator tiles][64 lanes][4] floats per
+// wave.  Written out as instructions because they can take their data from the accumulator registers
+// directly; through the compiler every value would first be copied to a vector register.
+__device__ __forceinline__ void publish_accumulators(const f32x4_t (&acc)[8][8], u32x4_t mine, int lane) {
+  const int lane16 = lane * 16;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen sc1"
+                   :: "a"(acc[i][j]), "v"(lane16), "s"(mine), "s"((i * 8 + j) * 1024) : "memory");
+}
+
+template <typename T, bool HAS_BIAS, int CLAMP>
+__device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0, int wave_n0,
+                                                int bz, int lane, uint32_t stage, const u32x2_t (&b)[8], const TailStore& t) {
+  constexpr int AGENT = 16;
+  constexpr int DEPTH = 2;
+  using S = typename T::storage;
+  const bool per_row = p.bias_per_row != 0;
+  const float ceiling = p.coef;
+  constexpr bool FIXUP = T::dtype == srtReal16BF;
+  S* C = (S*)p.C + (long long)bz * p.scb;
+  const long long c_last = (long long)(p.M - 1) * p.scm + p.N;
+  const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(C, 0, (int)(c_last * 2), 0x00020000);
+  const int ldc2 = (int)(p.scm * 2);
+  const int jn = lane & 15, g = lane >> 4;
+  const int rd_chunk = lane & 15, rd_row = lane >> 4;
+  const int n_rd = wave_n0 + 8 * rd_chunk;
+  const bool n_rd_ok = n_rd < p.N;
+  const int lane16 = lane * 16;
+  const bool one = t.foreign >= 1, two = t.foreign == 2, last = t.own_last;
+
+  f32x4_t others[DEPTH][2][8];   // [row mod DEPTH][f0 / f1][j]; written and read under the same conditions
+  auto fetch = [&](int i) {
+    if (one) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        others[i % DEPTH][0][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(t.f0, lane16, (i * 8 + j) * 1024, AGENT));
+    }
+    if (two) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        others[i % DEPTH][1][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(t.f1, lane16, (i * 8 + j) * 1024, AGENT));
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < DEPTH; ++i) fetch(i);
+
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    bool nan = false;
+#pragma unroll
+    for (int ii = 0; ii < 4; ++ii) {
+      const int i = 4 * half + ii;
+      const int row = 16 * ii + jn;
+      const uint32_t row_addr = stage + (uint32_t)row * 256u + (uint32_t)(g & 1) * 8u;
+      SRT_FENCE();
+      // the row's accumulators: one copy out of the accumulator registers, here, for every use
+      float a[8][4];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        a[j][0] = acc[i][j][0]; a[j][1] = acc[i][j][1]; a[j][2] = acc[i][j][2]; a[j][3] = acc[i][j][3];
+        asm volatile("" : "+v"(a[j][0]), "+v"(a[j][1]), "+v"(a[j][2]), "+v"(a[j][3]));
+      }
+      if (two) {
+        // (f0 + u) + w with (u, w) = (own, f1) or (f1, own)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const f32x4_t f0 = others[i % DEPTH][0][j], f1 = others[i % DEPTH][1][j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[j][e] = (f0[e] + (last ? f1[e] : a[j][e])) + (last ? a[j][e] : f1[e]);
+        }
+      } else if (one) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const f32x4_t f0 = others[i % DEPTH][0][j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[j][e] += f0[e];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float a0 = a[j][0], a1 = a[j][1], a2 = a[j][2], a3 = a[j][3];
+        if (HAS_BIAS) {
+          const float br = T::to_float((S)(b[i].x & 0xffffu));
+          a0 += per_row ? br : T::to_float((S)(b[j].x & 0xffffu));
+          a1 += per_row ? br : T::to_float((S)(b[j].x >> 16));
+          a2 += per_row ? br : T::to_float((S)(b[j].y & 0xffffu));
+          a3 += per_row ? br : T::to_float((S)(b[j].y >> 16));
+        }
+        if (CLAMP >= 1) {
+          a0 = __builtin_fmaxf(a0, 0.0f); a1 = __builtin_fmaxf(a1, 0.0f);
+          a2 = __builtin_fmaxf(a2, 0.0f); a3 = __builtin_fmaxf(a3, 0.0f);
+        }
+        if (CLAMP == 2) {
+          a0 = __builtin_fminf(a0, ceiling); a1 = __builtin_fminf(a1, ceiling);
+          a2 = __builtin_fminf(a2, ceiling); a3 = __builtin_fminf(a3, ceiling);
+        }
+        if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
+        const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};
+        const int c = 2 * j + (g >> 1);
+        *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
+      }
+      if (i + DEPTH < 8) {   // the row's registers are free again
+        SRT_FENCE();
+        fetch(i + DEPTH);
+      }
+    }
+    SRT_FENCE();
+    const bool fix = FIXUP && __builtin_amdgcn_ballot_w64(nan) != 0;
+    // ---- staging -> global: 16 instructions of 4 rows x 256 bytes, read four at a time ----
+#pragma unroll
+    for (int it4 = 0; it4 < 4; ++it4) {
+      u32x4_t v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 4 * (4 * it4 + q);
+        v[q] = *reinterpret_cast<const SRT_LDS u32x4_t*>(stage + (uint32_t)row * 256u +
+                                                         (uint32_t)((rd_chunk ^ (row & 15)) << 4));
+      }
+      if (fix) {   // rare: some accumulator of this half was a NaN
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[q][e] = ring::canonical_nans_bf16x2(v[q][e]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = rd_row + 4 * (4 * it4 + q);
+        const int m = wave_m0 + 64 * half + row;
+        const uint32_t off = (n_rd_ok && m < p.M) ? (uint32_t)(m * ldc2 + n_rd * 2) : OOB;
+        __builtin_amdgcn_raw_buffer_store_b128(v[q], rc, (int)off, 0, SRT_STORE_AUX);
+      }
+      SRT_FENCE();
+    }
+  }
+}
+
+#ifdef SRT_TAIL_TRACE   // measurement builds: times (100 MHz) of piece boundaries, 16 per workgroup
+static __device__ unsigned long long tail_trace[256 * 16];
+#endif
+
+// What the tail-sharing form of the kernel needs beyond the problem (see gemm_m16d_body, SK).
+struct TailShare {
+  float* partial;                // [left-over tile][part][wave][64 accumulator tiles][64 lanes][4] floats
+  unsigned long long* flags;     // [left-over tile][part]: `epoch` once that piece's partial is complete
+  unsigned long long epoch;      // a value no earlier use of the memory has left there
+  int parts;                     // pieces per left-over tile, 2 or 3
+  int cut1, cut2;                // part k covers quads [cut(k), cut(k+1)): 0, cut1, cut2, quads per tile (cut2 = that for 2 parts)
+  int groups;                    // workgroups that take the parts 1.. (a multiple of 8)
+  int per_group;                 // pieces each of them takes at most
+};
+constexpr int TAIL_MAX_PARTS = 3;
+
+// SK = false: workgroup w computes tiles w, w + G, ... whole.
+// SK = true, the tail-sharing form, for a tile count that is not a multiple of G.  The tiles left over after
+// the whole rounds (the last total mod G tile numbers) are cut along k, all at the same places (in quads: four
+// super-stages), into 2 or 3 parts.  Workgroup i takes part 0 of left-over tile i; the other parts go to
+// `groups` further workgroups, `per_group` pieces each, one after the other.  So every piece starts at the
+// same k as its neighbours' and the workgroups of an XCD walk k together through a patch of tiles, as they do
+// on whole tiles -- cut into runs of equal length instead, pieces start anywhere along k, no operand byte is
+// shared in L2 and the walk is memory-bound (measured: a third slower than doing without).  All pieces of a
+// tile are on one XCD.  Each piece is a tile walk like any other -- its operand offsets start further along k
+// and it has fewer super-stages -- so the k loop runs on across pieces as it does across tiles.  The piece
+// of a tile that finishes last adds the others' accumulators to its own, in the order of the parts whoever
+// it is (the bits do not depend on timing), and stores the tile; see the epilogue.  No workgroup ever waits
+// for another, so the form makes no assumption about which workgroups are resident.  Every workgroup takes
+// its pieces first and its whole tiles afterwards.
+template <typename T, bool A_KC, bool B_KC, int EPI, bool SK>
+__device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailShare& ts) {
   constexpr int TM = 8;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
@@ -165,7 +350,7 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
   const uint32_t kstep_a = A_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * lda * 2);   // bytes per super-stage
   const uint32_t kstep_b = B_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * ldb * 2);
   const uint32_t lstep_a = Loader<A_KC>::step(lda), lstep_b = Loader<B_KC>::step(ldb);
-  const int S = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least four)
+  const int S_full = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least four)
 
   // per-XCD start of the k walk for an A stored k x m (see gemm_ring_kernel)
 #ifndef SRT_M16D_ROTATE   // measurement builds: 0 never, 1 always
@@ -173,16 +358,92 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
 #else
   constexpr bool rotate = SRT_M16D_ROTATE != 0;
 #endif
-  const int rot = rotate ? (int)(((unsigned)(blockIdx.x & 7) * (unsigned)S) / 8u) : 0;
-  auto stage_of = [&](int r) {
+  const int rot = rotate && !SK ? (int)(((unsigned)(blockIdx.x & 7) * (unsigned)S_full) / 8u) : 0;
+  auto stage_of = [&](int r) {   // r = 0, 1, 2 only; a piece has at least four super-stages
+    if constexpr (SK) return r;
     int e = r + rot;
-    e = e >= S ? e - S : e;
-    e = e >= S ? e - S : e;
+    e = e >= S_full ? e - S_full : e;
+    e = e >= S_full ? e - S_full : e;
     return e;
   };
   auto wrap = [&](uint32_t a) { return a >= lds_end ? a - UNITS * UNIT : a; };
 
-  TileRef cur_tile = m16::locate_tile<A_KC, B_KC, 256>(p, v, tiles_m, tiles_n);
+  // ---- the walk: pieces of work, each a tile or (SK) some quads of one ----
+  struct Piece {
+    TileRef t;   // offa / offb already advanced to the piece's first super-stage
+    int n;       // super-stages
+    int tile;    // SK: index among the left-over tiles when the piece is a part of one, else -1
+    int part;
+  };
+  // an explicit move to the scalar unit (what feeds a scalar operand of an instruction written out below
+  // must be in a scalar register, and the compiler keeps some uniform values in vector ones)
+  // The compiler does not see inside the statement, so the wait states this instruction needs on gfx950 are
+  // written out: one after a vector write of the register it reads (the copy into it may be the
+  // instruction just before -- without the s_nop the read returned the register's previous content), and
+  // those between a vector write of a scalar register and its use by a vector (2) or memory (5) instruction.
+  auto scalar = [](int x) {
+    int r;
+    asm volatile("s_nop 0\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(r) : "v"(x));
+    return r;
+  };
+  const int rounds = total / grid;
+  const int left = total - rounds * grid;       // SK: the last `left` tile numbers are the shared ones
+  const int left8 = (left + 7) & ~7;
+  const int Q = S_full >> 2;                    // quads per tile
+  auto cut = [&](int k) { return k == 0 ? 0 : k == 1 ? ts.cut1 : k == 2 ? ts.cut2 : Q; };
+  int taken = 0;   // SK: pieces taken so far (or tried)
+  int round = 0;   // SK: whole tiles taken so far
+  const int me = (int)blockIdx.x;
+  auto take = [&](Piece& w) {   // SK only; false when the workgroup has nothing left
+    int tile = -1, part = 0;
+    if (me < left) {
+      if (taken == 0) tile = me;
+      taken = 1;
+    } else if (me >= left8 && me - left8 < ts.groups) {
+      while (tile < 0 && taken < ts.per_group) {
+        const int e = me - left8 + taken * ts.groups;
+        ++taken;
+        if (e < (ts.parts - 1) * left8 && e % left8 < left) {
+          tile = e % left8;
+          part = 1 + e / left8;
+        }
+      }
+    }
+    if (tile >= 0) {
+      const int s0 = cut(part) * 4;
+      w.t = m16::locate_tile<A_KC, B_KC, 256>(p, rounds * grid + tile, tiles_m, tiles_n);
+      w.t.offa += (uint32_t)s0 * kstep_a;
+      w.t.offb += (uint32_t)s0 * kstep_b;
+      w.n = (cut(part + 1) - cut(part)) * 4;
+      w.tile = tile;
+      w.part = part;
+      return true;
+    }
+    if (round < rounds) {
+      w.t = m16::locate_tile<A_KC, B_KC, 256>(p, me + round * grid, tiles_m, tiles_n);
+      w.n = S_full;
+      w.tile = -1;
+      w.part = 0;
+      ++round;
+      return true;
+    }
+    return false;
+  };
+  auto uniform = [&](Piece& w) {
+    w.t.offa = (uint32_t)scalar((int)w.t.offa);
+    w.t.offb = (uint32_t)scalar((int)w.t.offb);
+    w.n = scalar(w.n);
+  };
+
+  TileRef cur_tile;
+  Piece cur_piece, next_piece;
+  if constexpr (SK) {
+    if (!take(cur_piece)) return;
+    uniform(cur_piece);
+    cur_tile = cur_piece.t;
+  } else {
+    cur_tile = m16::locate_tile<A_KC, B_KC, 256>(p, v, tiles_m, tiles_n);
+  }
 
   // the eight loads of one unit, outside the main loop (first fill, and B_1 after an epilogue)
   auto issue_a = [&](const Loader<A_KC>& l, uint32_t slot, uint32_t base) {
@@ -200,6 +461,17 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
 
   uint32_t x = lds;   // slot of A_s; B_s follows it, then A_{s+1}, B_{s+1}, A_{s+2} (B_{s+2} goes where A_s is)
 
+#ifdef SRT_TAIL_TRACE   // measurement builds: times (100 MHz) of piece boundaries, 16 per workgroup
+  int trace_at = 0;
+  auto stamp = [&]() {
+    if (threadIdx.x == 0 && trace_at < 16) tail_trace[blockIdx.x * 16 + trace_at] = (unsigned long long)wall_clock64();
+    ++trace_at;
+  };
+#define SRT_STAMP() stamp()
+#else
+#define SRT_STAMP()
+#endif
+  SRT_STAMP();
   bool first_tile = true;
   for (;;) {
     // per-lane addressing state, derived per tile and scoped to it (see gemm_ring_kernel)
@@ -225,14 +497,27 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
     first_tile = false;
     SRT_FENCE();
 
-    const int vn = v + grid;
-    const bool has_next = vn < total;
-    const TileRef next_tile =
-        m16::locate_tile<A_KC, B_KC, 256>(p, (int)select_lt(vn, total, (uint32_t)vn, (uint32_t)v), tiles_m, tiles_n);
+    int vn = 0, S = S_full;
+    bool has_next;
+    TileRef next_tile;
+    if constexpr (SK) {
+      S = cur_piece.n;
+      has_next = take(next_piece);
+      if (!has_next) next_piece = cur_piece;
+      uniform(next_piece);
+      next_tile = next_piece.t;
+      vn = scalar(has_next ? 0 : 1);   // vn < 1 below: there is a next piece
+    } else {
+      vn = v + grid;
+      has_next = vn < total;
+      next_tile =
+          m16::locate_tile<A_KC, B_KC, 256>(p, (int)select_lt(vn, total, (uint32_t)vn, (uint32_t)v), tiles_m, tiles_n);
+    }
+    const int vn_bound = SK ? 1 : total;
     // A requests below limit_a are real (A'_0 and A'_1 of the next tile); of B only B'_0: B'_1 would land in
     // the staging area
-    const int limit_a = (int)select_lt(vn, total, (uint32_t)(S + 2), (uint32_t)S);
-    const int limit_b = (int)select_lt(vn, total, (uint32_t)(S + 1), (uint32_t)S);
+    const int limit_a = (int)select_lt(vn, vn_bound, (uint32_t)(S + 2), (uint32_t)S);
+    const int limit_b = (int)select_lt(vn, vn_bound, (uint32_t)(S + 1), (uint32_t)S);
 
     f32x4_t acc[TM][8];   // defined by the MFMAs of the tile's first super-stage
     u32x4_t af[TM], bf[8];
@@ -391,19 +676,87 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
     // Every load in flight must have landed, in every wave, before the slots vacated last become the
     // staging area.  The s_nops are the wait states between the last MFMAs and the first reads of their
     // accumulators by other instructions.
+    SRT_STAMP();   // the piece's main loop is done
     const int em0 = cur_tile.m0 + wm0, en0 = cur_tile.n0 + wn0, bz = cur_tile.bz;
     const int le = lane_id();
     constexpr bool LINEAR_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED;
     u32x2_t bias_regs[8];
     if (LINEAR_BIAS) m16::load_bias<T, TM>(p, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
-    if (LINEAR_BIAS) m16::pin_all<TM>(acc);
+    if (LINEAR_BIAS || SK) m16::pin_all<TM>(acc);
     // staging: the slots of A_{S-1} (waves 0, 1) and B_{S-1} (waves 2, 3), half a slot each; x is A_S's by now
     uint32_t sa = x < lds + 2 * UNIT ? x + 3 * UNIT : x - 2 * UNIT;
     uint32_t sb = x < lds + UNIT ? x + 4 * UNIT : x - UNIT;
     const uint32_t stage = ((wave & 2) ? sb : sa) + (uint32_t)(wave & 1) * (uint32_t)(UNIT / 2);
 
-    if (EPI == EPI_PARTIAL) {
+    if constexpr (SK) {
+      // One copy of the epilogue (store_tile_tail), run once or twice.
+      // A whole tile: once, plain.  A part of a tile: whichever piece of the tile finds the flags of all
+      // the others raised adds up the partials in the order of the parts -- its own straight from the
+      // registers -- and stores the tile; a piece that does not leaves its accumulators in `partial`
+      // (first run), raises its flag and looks again: of two pieces that finish together at least one
+      // then sees the other, and if both do, both store the same bits (second run).  Nobody waits.
+      // Coherence between workgroups is per access, not per cache: partials and flags are written and read
+      // with the agent-scope policy (sc1: stores write through, loads do not trust a cached copy), and
+      // s_waitcnt vmcnt(0) -- the stores have been acknowledged -- orders partials before the flag and the
+      // flag before the second look.  (Agent-scope fences would write back and invalidate whole L2s, once
+      // per workgroup: measured at 100 us per launch.)
+      const bool part_of_tile = cur_piece.tile >= 0;
+      const int place0 = cur_piece.tile * TAIL_MAX_PARTS, mine = cur_piece.part;
+      auto others_done = [&]() {
+        bool ok = true;
+        for (int k = 0; k < ts.parts; ++k)
+          if (k != mine)
+            ok &= __hip_atomic_load(ts.flags + place0 + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ts.epoch;
+        return ok;
+      };
+      // one thread decides for the workgroup; the verdict travels through the first word of the staging area
+      SRT_LDS int* verdict = reinterpret_cast<SRT_LDS int*>(sa);
+      auto agree = [&](auto&& decide) {
+        if (threadIdx.x == 0) *verdict = decide() ? 1 : 0;
+        __syncthreads();
+        const int v = __builtin_amdgcn_readfirstlane(*verdict);
+        __syncthreads();
+        return v != 0;
+      };
+      auto partial_of = [&](int part) {
+        float* base = ts.partial + ((size_t)((place0 + part) * 4 + wave) * 64) * 256;
+        return __builtin_amdgcn_make_buffer_rsrc(base, 0, part_of_tile ? 65536 : 0, 0x00020000);
+      };
+      TailStore how;
+      how.foreign = 0;
+      how.own_last = false;
+      // the other parts in order: f0, then f1 if there are three
+      const int o0 = mine == 0 ? 1 : 0;
+      const int o1 = ts.parts == 3 ? (mine == 2 ? 1 : 2) : o0;
+      how.f0 = partial_of(o0);
+      how.f1 = partial_of(o1);
+      // part 0 is expected to end last (see tail_plan) and looks first; the others publish first
+      constexpr bool HAS_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED;
+      constexpr int CLAMP = EPI == EPI_CLIPPED ? 2 : (EPI == EPI_RELU || EPI == EPI_BIAS_RELU) ? 1 : 0;
+      bool finish = true;
+      if (part_of_tile) finish = mine == 0 && agree(others_done);
+      for (;;) {
+        if (finish) {
+          if (part_of_tile) {
+            how.foreign = ts.parts - 1;
+            how.own_last = mine == 2;
+          }
+          m16::pin_all<TM>(acc);   // (nothing read from the accumulators moves out of the loop)
+          store_tile_tail<T, HAS_BIAS, CLAMP>(p, acc, em0, en0, bz, lane_id(), stage, bias_regs, how);
+          break;
+        }
+        publish_accumulators(acc, ring::make_rsrc(ts.partial + ((size_t)((place0 + mine) * 4 + wave) * 64) * 256, 65536), lane_id());
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        finish = agree([&]() {
+          __hip_atomic_store(ts.flags + place0 + mine, ts.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          return others_done();
+        });
+        if (!finish) break;
+      }
+    } else if (EPI == EPI_PARTIAL) {
       m16::store_tile_partial<TM>(p, acc, em0, en0, bz, le, stage);
     } else if (EPI == EPI_TRANS) {
       m16::load_bias<T, TM>(p, em0, en0, le, bias_regs);
@@ -415,13 +768,25 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
       else if (EPI == EPI_CLIPPED) m16::store_tile<T, TM, true, 2>(p, acc, em0, en0, bz, le, stage, bias_regs);
       else m16::store_tile<T, TM, false, 0>(p, acc, em0, en0, bz, le, stage, bias_regs);
     }
+    SRT_STAMP();   // and its epilogue
     if (!has_next) break;
 
     // every wave has finished reading its staging area before any wave's loads overwrite it
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    v = vn;
+    if constexpr (SK) cur_piece = next_piece;
+    else v = vn;
     cur_tile = next_tile;
   }
+}
+
+template <typename T, bool A_KC, bool B_KC, int EPI>
+__global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
+  gemm_m16d_body<T, A_KC, B_KC, EPI, false>(p, TailShare{});
+}
+
+template <typename T, bool A_KC, bool B_KC, int EPI>
+__global__ __launch_bounds__(NT) void gemm_m16d_tail_kernel(GemmProblem p, TailShare ts) {
+  gemm_m16d_body<T, A_KC, B_KC, EPI, true>(p, ts);
 }
 
 #undef SRT_FENCE
@@ -439,6 +804,113 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   const int grid = ring::persistent_grid(tiles);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return launch_status(stream);
+}
+
+// ---- the tail-sharing form ----------------------------------------------------------------------------
+constexpr size_t TAIL_PARTIAL_BYTES = 256 * 256 * sizeof(float);   // per piece
+constexpr size_t TAIL_FLAG_BYTES = 8192;                           // 255 x 3 flags, ahead of the partials
+
+// How the tail-sharing form would cut the left-over tiles of `p`; parts = 0: it does not apply.
+struct TailPlan {
+  int parts, cut1, cut2, groups, per_group;
+  int left;          // tiles shared
+  int tail_quads;    // length of the longest workgroup's share of them, in quads (a whole tile: K / 256)
+};
+inline TailPlan tail_plan(const GemmProblem& p) {
+  TailPlan t{};
+  if (!deep_fits(p) || p.K % (4 * DK) != 0) return t;
+  const int grid = compute_units();
+  if (grid % 8 != 0 || grid > 256) return t;
+  const long long tiles = (long long)((p.M + 255) / 256) * ((p.N + BN - 1) / BN) * p.batch;
+  const int left = (int)(tiles % grid), left8 = (left + 7) & ~7;
+  const int Q = p.K / (4 * DK);
+  if (left == 0 || tiles >= (1ll << 30)) return t;
+  // Part 0 is made long enough to end after the others have published theirs (publishing costs about
+  // what two quads of multiplying do), so that it finds their flags raised, publishes nothing and is the
+  // only one to add up: pieces that end together would both publish and both add up.
+  constexpr int PUB = 2;
+  const int even = std::min(TAIL_MAX_PARTS, grid / left8);   // parts of one workgroup each
+  if (even == 3 && Q >= 7) {
+    t.parts = 3;
+    t.cut1 = (Q + 2 * PUB + 2) / 3;
+    t.cut2 = t.cut1 + (Q - t.cut1 + 1) / 2;
+    t.groups = 2 * left8;
+    t.per_group = 1;
+  } else if (even >= 2 && Q >= 4) {
+    t.parts = 2;
+    t.cut1 = (Q + PUB + 1) / 2;
+    t.cut2 = Q;
+    t.groups = left8;
+    t.per_group = 1;
+  } else if (even < 2) {
+    // two parts, the second short enough for a workgroup to take m of them in the time of a first part
+    for (int m = 2; m <= 4 && t.parts == 0; ++m) {
+      const int groups = ((left + m - 1) / m + 7) & ~7;
+      const int cut = (m * (Q + PUB) + m) / (m + 1);   // ceil(m (Q + PUB) / (m + 1))
+      if (left8 + groups <= grid && cut < Q) {
+        t.parts = 2;
+        t.cut1 = cut;
+        t.cut2 = Q;
+        t.groups = groups;
+        t.per_group = m;
+      }
+    }
+  }
+  t.tail_quads = t.cut1 + 3;   // part 0 and its adding up (against quads per tile + 1 for a whole tile)
+  t.left = left;
+  return t;
+}
+inline bool tail_fits(const GemmProblem& p) { return tail_plan(p).parts != 0; }
+
+// Flag values: a process-wide launch counter under a fixed 32-bit tag.  The flags live in memory that
+// other kernels have written before (the allocator recycles blocks), so what they hold at launch is
+// arbitrary; a launch waits for its own value, which no earlier launch has written and which arbitrary
+// data matches with probability 2^-64 per flag.
+inline unsigned long long next_tail_epoch() {
+  static std::atomic<unsigned long long> counter{0};
+  return 0x5ca1ab1e00000000ull | (++counter & 0xffffffffull);
+}
+
+template <typename T, bool A_KC, bool B_KC, int EPI>
+hipError_t launch_tail_kernel(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_m16d_tail_kernel<T, A_KC, B_KC, EPI>;
+  constexpr int lds_bytes = UNITS * UNIT;
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
+  const TailPlan plan = tail_plan(p);
+  if (plan.parts == 0) return hipErrorInvalidValue;
+  const int grid = compute_units();
+  void* workspace = nullptr;
+  const size_t bytes = TAIL_FLAG_BYTES + (size_t)plan.left * TAIL_MAX_PARTS * TAIL_PARTIAL_BYTES;
+  if (srtDeviceAllocate(&workspace, bytes, reinterpret_cast<srtStream>(stream)) != srtSuccess) return hipErrorOutOfMemory;
+  TailShare ts;
+  ts.parts = plan.parts;
+  ts.cut1 = plan.cut1;
+  ts.cut2 = plan.cut2;
+  ts.groups = plan.groups;
+  ts.per_group = plan.per_group;
+  ts.flags = reinterpret_cast<unsigned long long*>(workspace);
+  ts.partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + TAIL_FLAG_BYTES);
+  ts.epoch = next_tail_epoch();
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p, ts);
+  const hipError_t e = launch_status(stream);
+  (void)srtDeviceFree(workspace);   // stream-ordered: reused only by work queued after the kernel
+  return e;
+}
+
+// (the transcendental activations have no tail-sharing form)
+template <typename T, bool A_KC, bool B_KC>
+hipError_t launch_tail(const GemmProblem& p, hipStream_t stream) {
+  const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
+                     p.activation == srtActivationElu;
+  if (trans) return hipErrorInvalidValue;
+  if (p.activation == srtActivationClippedRelu) return launch_tail_kernel<T, A_KC, B_KC, EPI_CLIPPED>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_tail_kernel<T, A_KC, B_KC, EPI_BIAS_RELU>(p, stream);
+    return launch_tail_kernel<T, A_KC, B_KC, EPI_RELU>(p, stream);
+  }
+  if (p.bias) return launch_tail_kernel<T, A_KC, B_KC, EPI_BIAS>(p, stream);
+  return launch_tail_kernel<T, A_KC, B_KC, EPI_PLAIN>(p, stream);
 }
 
 template <typename T, bool A_KC, bool B_KC>

@@ -112,12 +112,13 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
 // (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
 // and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
 enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK,
-            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanCount };
+            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanCount };
 
 const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
                                             "f32_mfma_64x64", "f32_mfma_splitk", "mfma_256x256_k64",
                                             "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16",
-                                            "mfma_128x128_any", "mfma_64x64_any", "mfma_256x256_m16_k64"};
+                                            "mfma_128x128_any", "mfma_64x64_any", "mfma_256x256_m16_k64",
+                                            "mfma_256x256_m16_k64_tail"};
 
 bool plan_supported(const GemmProblem& p, Plan plan) {
   switch (plan) {
@@ -132,6 +133,7 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
     case kPlanAny128: return srt::mfma_config(p, 7) != 0;
     case kPlanAny64: return srt::mfma_config(p, 8) != 0;
     case kPlanM16D: return srt::mfma_config(p, 9) != 0;
+    case kPlanM16DTail: return srt::mfma_config(p, 10) != 0;
     case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
     case kPlanF32SplitK: return srt::f32_mfma_supported(p);
     default: return srt::generic_supported(p);
@@ -140,6 +142,8 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 
 Plan heuristic_plan(const GemmProblem& p) {
   if (srt::skinny_supported(p) && srt::skinny_preferred(p)) return kPlanSkinny;
+  // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units
+  if (srt::mfma_prefers_tail(p)) return kPlanM16DTail;
   // few 256 x 256 tiles and a long k loop: K split over the idle compute units
   if (srt::mfma_prefers_splitk(p)) return kPlanSplitK;
   const int c = srt::mfma_select(p);
@@ -153,6 +157,7 @@ Plan heuristic_plan(const GemmProblem& p) {
       case 7: return kPlanAny128;
       case 8: return kPlanAny64;
       case 9: return kPlanM16D;
+      case 10: return kPlanM16DTail;
       default: return kPlanMfma64;
     }
   }
@@ -173,6 +178,7 @@ hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
     case kPlanAny128: return srt::launch_mfma(p, srt::mfma_config(p, 7), stream);
     case kPlanAny64: return srt::launch_mfma(p, srt::mfma_config(p, 8), stream);
     case kPlanM16D: return srt::launch_mfma(p, srt::mfma_config(p, 9), stream);
+    case kPlanM16DTail: return srt::launch_mfma(p, srt::mfma_config(p, 10), stream);
     case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
     case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
     default: return srt::launch_generic(p, stream);
@@ -345,10 +351,10 @@ srtStatus run(const GemmProblem& p, hipStream_t stream) {
   const Plan plan = select(p);
   if (plan == kPlanGeneric && !srt::generic_supported(p)) return srtErrorNotSupported;
   hipError_t e = launch_plan(p, plan, stream);
-  if (plan == kPlanSplitK && e == hipErrorOutOfMemory) {
+  if ((plan == kPlanSplitK || plan == kPlanM16DTail) && e == hipErrorOutOfMemory) {
     // no room for the workspace (nothing was launched): the plan that needs none
     (void)hipGetLastError();
-    const int c = srt::mfma_select(p);
+    const int c = plan == kPlanM16DTail ? srt::mfma_config(p, 9) : srt::mfma_select(p);
     e = c ? srt::launch_mfma(p, c, stream) : srt::launch_generic(p, stream);
   }
   return srt::from_hip(e);
@@ -442,7 +448,7 @@ srtStatus srtMatmulTune(const void* a, const srtTensorDescriptor* aDesc, int32_t
     if (plan == kPlanGeneric && fallback != kPlanGeneric && 2.0 * p.M * p.N * p.K * p.batch > 1e9) continue;
     const int warm = 2, reps = 8;
     for (int i = 0; i < warm && err == hipSuccess; ++i) err = launch_plan(p, plan, hs);
-    if (plan == kPlanSplitK && err == hipErrorOutOfMemory) {
+    if ((plan == kPlanSplitK || plan == kPlanM16DTail) && err == hipErrorOutOfMemory) {
       // no room for this plan's workspace (nothing was launched): it is not a candidate, as in run()
       (void)hipGetLastError();
       err = hipSuccess;

@@ -204,8 +204,15 @@ def test_kernel_selection_is_queryable_without_gpu():
     # half-height tiles a k-contiguous A allows
     assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_256x256_splitk"           # eight parts
     assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_256x256_splitk"
-    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_128x256_m16"             # four parts: half tiles tie, no workspace
-    assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_256x256_splitk"          # four parts, K = 8192
+    # 64 to 160 tiles: the tail-sharing form of the 64-deep kernel (every tile cut along k into two or three parts),
+    # unless half-height tiles fill one round as well
+    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_256x256_m16_k64_tail"
+    assert query(native.REAL16BF, 2048, 4096, 4096, tb=True) == "mfma_256x256_m16_k64_tail"
+    assert query(native.REAL16BF, 2048, 4096, 4096) == "mfma_128x256_m16"
+    assert query(native.REAL16BF, 2048, 4096, 8192) == "mfma_256x256_m16_k64_tail"
+    assert query(native.REAL16BF, 4096, 10240, 4096) == "mfma_256x256_m16_k64"        # after whole rounds it buys nothing
+    assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_256x256_m16_k64_tail"    # 64 tiles again
+    assert query(native.REAL16BF, 1024, 2048, 8192) == "mfma_256x256_splitk"          # 32 tiles: eight parts
     assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_256x256_splitk"
     assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: from K = 2048
     assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x256"        # 32 tiles: the ring from 24 up
@@ -221,9 +228,11 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16"             # 256 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: whole tiles, K split
     assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x256"
-    assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_128x256_m16"            # 258 whole tiles: two rounds for two tiles
-    assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16_k64"   # both k-contiguous: one round of halves or none
-    assert query(native.REAL16BF, 1536, 4096, 11008, tb=True) == "mfma_256x256_splitk"
+    # 258 whole tiles: a whole round, and the two left over cut along k in three parts each
+    assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_256x256_m16_k64_tail"
+    assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16_k64_tail"
+    assert query(native.REAL16BF, 1536, 11008, 2048) == "mfma_256x256_m16_k64"        # (not for a k loop this short)
+    assert query(native.REAL16BF, 1536, 4096, 11008, tb=True) == "mfma_256x256_m16_k64_tail"   # 96 tiles, two parts each
     assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16"              # 8 half tiles
     assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
     assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16"              # K too short to split

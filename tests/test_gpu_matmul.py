@@ -963,14 +963,16 @@ def test_bf16_operands_beyond_4_gib_bit_exact(case):
     block = big0.astype(np.float64) @ small.astype(np.float64).T          # [P, small_rows], exact integers
     if case == "nn_big_a":      # A [65664, K] . B [K, 512]
         a, b, ta, tb = _periodic(H.encode(big0, H.BF16), reps, 0), H.encode(np.ascontiguousarray(small.T), H.BF16), False, False
-        want, kernel = np.concatenate([block] * reps, 0), "mfma_256x256_m16_k64/pieces"
+        # (each half: 130 tiles and K = 32768 -- the tail-sharing form, two parts per tile)
+        want, kernel = np.concatenate([block] * reps, 0), "mfma_256x256_m16_k64_tail/pieces"
     elif case == "tn_big_a":    # A stored [K, 65664], transposed
         a, b, ta, tb = _periodic(H.encode(np.ascontiguousarray(big0.T), H.BF16), reps, 1), H.encode(np.ascontiguousarray(small.T), H.BF16), True, False
         want, kernel = np.concatenate([block] * reps, 0), "mfma_128x128"
     else:                       # x [512 or 8, K] . W [65664, K]^T
         a, b, ta, tb = H.encode(small, H.BF16), _periodic(H.encode(big0, H.BF16), reps, 0), False, True
         want = np.concatenate([block.T] * reps, 1)
-        kernel = "skinny/pieces" if case == "skinny_big_w" else "mfma_256x256_m16_k64/pieces"
+        # (each half of N: 258 tiles -- a whole round, and the two left over cut along k)
+        kernel = "skinny/pieces" if case == "skinny_big_w" else "mfma_256x256_m16_k64_tail/pieces"
     assert max(a.size, b.size) > 2 ** 31
     got = gpu_matmul(a, b, ta, tb, want_kernel=kernel)
     assert np.array_equal(got, H.encode(want.astype(np.float32), H.BF16))

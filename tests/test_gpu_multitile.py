@@ -246,6 +246,78 @@ def test_heuristic_takes_the_checked_kernels():
     assert query_kernel(x, False, w, False, y) == "mfma_256x256_m16_k64"
 
 
+# ---- the tail-sharing form of the 64-deep kernel ------------------------------------------------------------
+TAIL = "mfma_256x256_m16_k64_tail"
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+@pytest.mark.parametrize("ta,tb", LAYOUTS)
+def test_tail_sharing_integer_bit_exact(dt, ta, tb, tmp_path):
+    """Tiles left over after the whole rounds, cut along k and added up by whichever piece ends last:
+    2048 x 4096 x 2048 -- 128 tiles and no whole round, two parts per tile (5 + 3 quads);
+    4096 x 5120 x 2048 -- one whole round, then 64 tiles in three parts (4 + 2 + 2);
+    4400 x 4360 x 2048 -- ragged edges in M and N, 68 tiles left over (not a multiple of 8), three parts."""
+    for (M, N, K) in [(2048, 4096, 2048), (4096, 5120, 2048), (4400, 4360, 2048)]:
+        check_plan(tmp_path, TAIL, dt, M, N, K, ta, tb)
+
+
+def test_tail_sharing_dense_shape_bias_relu(tmp_path):
+    """4096 x 11008 x 4096 with bias and relu: two whole rounds, then 176 tiles cut 14 + 2 quads, the short
+    parts taken three at a time by 64 further workgroups."""
+    got = check_plan(tmp_path, TAIL, H.BF16, 4096, 11008, 4096, False, False, with_bias_relu=True)
+    assert np.all(H.decode(got) >= 0.0)
+
+
+def test_tail_sharing_batched_clipped_and_repeatable(tmp_path):
+    """A strided batch (96 tiles over three batches, two parts each), the clipped-relu epilogue on random
+    operands against the plain kernel (the parts' sums are added in another order: one rounding step of the
+    result type apart at most), and the same bits on every run, whichever piece happened to add up."""
+    r = H.rng(77)
+    B_, M, N, K = 3, 1024, 2048, 1024
+    a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+    w = r.integers(-3, 4, (B_, K, N)).astype(np.float32)
+    pin(tmp_path, TAIL, H.BF16, M, N, K, False, False, batch=B_)
+    at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+    out = srt.matmul(at, wt)
+    assert query_kernel(at, False, wt, False, out) == TAIL
+    assert np.array_equal(out.array(), H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), H.BF16))
+
+    M, N, K = 2048, 4096, 4096
+    x = srt.Tensor(H.encode((r.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32), H.BF16))
+    wt = srt.Tensor(H.encode(r.standard_normal((K, N)).astype(np.float32), H.BF16))
+    bt = srt.Tensor(H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), H.BF16))
+    act = srt.ActivationType.clippedRelu
+    runs = {}
+    for plan in (TAIL, DEEP):
+        pin(tmp_path, plan, H.BF16, M, N, K, False, False, bias=True, act=act)
+        out = srt.Tensor(shape=[M, N], dtype=np.uint16)
+        assert query_kernel(x, False, wt, False, out) == plan
+        runs[plan] = []
+        for _ in range(3 if plan == TAIL else 1):
+            srt.current_queue().matmul(x, False, wt, False, out, bias=bt, activation=act, coef=0.75)
+            runs[plan].append(out.array().copy())
+    assert np.array_equal(runs[TAIL][0], runs[TAIL][1]) and np.array_equal(runs[TAIL][0], runs[TAIL][2])
+    tail, plain = H.decode(runs[TAIL][0]), H.decode(runs[DEEP][0])
+    assert np.all(np.abs(tail - plain) <= 2.0 ** -7 * np.maximum(np.abs(plain), 2.0 ** -7))
+    assert np.count_nonzero(runs[TAIL][0] != runs[DEEP][0]) < 0.01 * M * N
+    assert tail.max() == 0.75 and tail.min() == 0.0
+
+
+def test_tail_sharing_is_refused_where_it_does_not_apply(tmp_path):
+    """No tiles left over, k not in whole quads, or too few quads to cut: a pinned tail-sharing plan is ignored
+    and the heuristic's kernel runs."""
+    def kernel_for(M, N, K):
+        pin(tmp_path, TAIL, H.BF16, M, N, K, False, False)
+        a = srt.Tensor(shape=[M, K], dtype=np.uint16)
+        b = srt.Tensor(shape=[K, N], dtype=np.uint16)
+        out = srt.Tensor(shape=[M, N], dtype=np.uint16)
+        return query_kernel(a, False, b, False, out)
+    assert kernel_for(2048, 4096, 2048) == TAIL
+    assert kernel_for(4096, 4096, 2048) != TAIL      # 256 tiles: nothing left over
+    assert kernel_for(2048, 4096, 2048 + 64) != TAIL  # k not a multiple of 256
+    assert kernel_for(2048, 4096, 512) != TAIL        # two quads: too short to cut
+
+
 # ---- the reference's batched known answers on the device, bf16 included -----------------------------------
 @pytest.mark.parametrize("dt", [H.F32, H.F16, H.BF16])
 def test_reference_kat_batched_and_right_batched(kats, dt):
