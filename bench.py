@@ -126,7 +126,7 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     ap.add_argument("--only", default=None,
                     help="run one configuration alone, a few launches, and exit (for profilers): headline, cfg3_tn, cfg3_nt, "
-                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, dense_backward, add, add_bias, tanh, cast")
+                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, few_tiles, dense_backward, add, add_bias, tanh, cast")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the single-GPU matmul path; run it with --gpus 1 "
@@ -223,7 +223,7 @@ def main():
 class Bench:
     """The configurations, each as one prepared foreign call per step."""
 
-    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1")
+    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1", "few_tiles")
 
     def __init__(self, srt, native, q):
         self.srt, self.native, self.q = srt, native, q
@@ -320,6 +320,17 @@ class Bench:
             return {"name": "cfg2 fp16 batch 32 x 256^3 transposeRhs", "call": call, "kernel": kernel,
                     "flops": 2.0 * 32 * 256 ** 3, "bytes": 32 * 3 * 256 * 256 * 2, "bound": "mfma", "dtype": "f16",
                     "steps": 200}
+        if name == "few_tiles":
+            # not a BASELINE configuration: a quarter-full device with a long k loop, the case of the
+            # tail-sharing form of the headline kernel (every tile cut along k into three parts)
+            g = rng(5)
+            a = srt.Tensor(bf16_encode(g.standard_normal((1024, 4096), dtype=np.float32) / np.float32(64)))
+            b = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))
+            c = srt.Tensor(shape=[1024, 4096], dtype=np.uint16)
+            call, kernel = self.prepared(a, False, b, False, c)
+            return {"name": "bf16 1024x4096x4096 (64 tiles of 256 x 256)", "call": call, "kernel": kernel,
+                    "flops": 2.0 * 1024 * 4096 * 4096, "bytes": (1024 * 4096 * 2 + 4096 * 4096) * 2, "bound": "mfma",
+                    "dtype": "bf16", "steps": 200}
         if name == "cfg1":
             g = rng(0)
             a1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))

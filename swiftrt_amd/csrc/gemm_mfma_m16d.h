@@ -32,6 +32,10 @@
 // workgroup's next tile are requested while this tile's last super-stages are multiplied; the two slots
 // vacated last are the epilogue's staging area and B'_1 is requested after it.
 // Preconditions beyond the 32-deep kernel's: K a multiple of 64 and at least 256.
+//
+// A second form of the kernel (gemm_m16d_tail_kernel, "tail sharing") is for tile counts that leave some
+// compute units without work in the last round: the tiles left over after the whole rounds are cut along k
+// and all workgroups share them; see gemm_m16d_body.
 #pragma once
 #include "gemm_mfma_m16.h"
 
@@ -314,8 +318,8 @@ constexpr int TAIL_MAX_PARTS = 3;
 // `groups` further workgroups, `per_group` pieces each, one after the other.  So every piece starts at the
 // same k as its neighbours' and the workgroups of an XCD walk k together through a patch of tiles, as they do
 // on whole tiles -- cut into runs of equal length instead, pieces start anywhere along k, no operand byte is
-// shared in L2 and the walk is memory-bound (measured: a third slower than doing without).  All pieces of a
-// tile are on one XCD.  Each piece is a tile walk like any other -- its operand offsets start further along k
+// shared in L2 and the walk is memory-bound (measured: a third slower than doing without).  (With workgroups
+// dealt to the XCDs in turn all pieces of a tile are on one XCD; nothing relies on that.)  Each piece is a tile walk like any other -- its operand offsets start further along k
 // and it has fewer super-stages -- so the k loop runs on across pieces as it does across tiles.  The piece
 // of a tile that finishes last adds the others' accumulators to its own, in the order of the parts whoever
 // it is (the bits do not depend on timing), and stores the tile; see the epilogue.  No workgroup ever waits
