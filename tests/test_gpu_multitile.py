@@ -303,6 +303,49 @@ def test_tail_sharing_batched_clipped_and_repeatable(tmp_path):
     assert tail.max() == 0.75 and tail.min() == 0.0
 
 
+def test_tail_sharing_every_way_of_cutting(tmp_path):
+    """Left-over counts that reach every branch of the cutting rule -- three parts, two parts, one short part
+    taken two, three and four at a time, counts that are not multiples of 8, a single left-over tile, with and
+    without whole rounds before them -- on ragged M and N, in rotating layouts and both types: bit-exact against
+    the 128 x 128 kernel over the whole result."""
+    r = H.rng(911)
+    # (tiles along M, tiles along N, batch, K): left over = tiles mod 256
+    cases = [(1, 1, 1, 1792),      # 1 tile: three parts (7 quads: 4 + 2 + 1)
+             (1, 7, 1, 1024),      # 7: a 4-quad tile is too short for three parts -> two (3 + 1)
+             (3, 3, 1, 2304),      # 9: three parts (5 + 2 + 2)
+             (5, 16, 1, 1792),     # 80: three parts, every compute unit but 16 at work
+             (2, 43, 1, 1024),     # 86: two parts
+             (3, 43, 1, 1792),     # 129: two parts (6 + 1), the short one taken two at a time
+             (9, 19, 1, 2560),     # 171: (9 + 1) three at a time
+             (4, 11, 4, 2560),     # 176 over four batches: three at a time
+             (8, 25, 1, 3328),     # 200: (12 + 1) four at a time
+             (16, 17, 1, 1024),    # 272 = a whole round + 16
+             (11, 31, 1, 1280)]    # 341 = a whole round + 85
+    for i, (tm, tn, batch, K) in enumerate(cases):
+        dt = (H.BF16, H.F16)[i % 2]
+        ta, tb = LAYOUTS[i % 4]
+        M = tm * 256 - int(r.integers(0, 31)) * 8
+        N = tn * 256 - int(r.integers(0, 31)) * 8
+        a = r.integers(-3, 4, (batch, K, M) if ta else (batch, M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (batch, N, K) if tb else (batch, K, N)).astype(np.float32)
+        at, bt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(b, dt))
+        got = {}
+        for plan in (TAIL, "mfma_128x128"):
+            pin(tmp_path, plan, dt, M, N, K, ta, tb, batch=batch)
+            out = srt.Tensor(shape=[batch, M, N], dtype=H.NP_STORAGE[dt])
+            assert query_kernel(at, ta, bt, tb, out) == plan, (plan, tm, tn, batch, K)
+            srt.current_queue().matmul(at, ta, bt, tb, out)
+            got[plan] = out.array().copy()
+        assert np.array_equal(got[TAIL].view(np.uint16), got["mfma_128x128"].view(np.uint16)), (tm, tn, batch, K, ta, tb)
+        # and a sampled row of each batch against the exact product
+        for z in range(batch):
+            row = int(r.integers(0, M))
+            a_row = (a[z][:, row] if ta else a[z][row]).astype(np.int64)
+            b_mat = (b[z].T if tb else b[z]).astype(np.int64)
+            want = H.encode((a_row @ b_mat).astype(np.float32), dt)
+            assert np.array_equal(got[TAIL][z, row].view(np.uint16), want.view(np.uint16)), (tm, tn, z, row)
+
+
 def test_tail_sharing_is_refused_where_it_does_not_apply(tmp_path):
     """No tiles left over, k not in whole quads, or too few quads to cut: a pinned tail-sharing plan is ignored
     and the heuristic's kernel runs."""
