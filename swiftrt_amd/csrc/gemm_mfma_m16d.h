@@ -146,8 +146,8 @@ struct FragReader<false> {
 // what does not fit: every epilogue then took 23 us instead of 5.)
 //   foreign   1 or 2: the tile's sum is spread over two or three workgroups; the accumulators of the other
 //             one or two (f0, f1: what they published, see publish_accumulators) are added on the way out,
-//             in the order of the parts along k whoever does the adding, streamed from memory two rows of
-//             accumulator tiles ahead
+//             in the order of the parts along k whoever does the adding, streamed from memory four (one
+//             foreign part) or two (two) rows of accumulator tiles ahead
 // Partials are written and read with the agent-scope policy (cache policy operand 16: sc1): another
 // workgroup, maybe on another XCD, reads or wrote them during this launch.
 struct TailStore {
@@ -173,7 +173,6 @@ template <typename T, bool HAS_BIAS, int CLAMP>
 __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0, int wave_n0,
                                                 int bz, int lane, uint32_t stage, const u32x2_t (&b)[8], const TailStore& t) {
   constexpr int AGENT = 16;
-  constexpr int DEPTH = 2;
   using S = typename T::storage;
   const bool per_row = p.bias_per_row != 0;
   const float ceiling = p.coef;
@@ -189,21 +188,35 @@ __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x
   const int lane16 = lane * 16;
   const bool one = t.foreign >= 1, two = t.foreign == 2, last = t.own_last;
 
-  f32x4_t others[DEPTH][2][8];   // [row mod DEPTH][f0 / f1][j]; written and read under the same conditions
-  auto fetch = [&](int i) {
-    if (one) {
+  // Four row slots of eight accumulator tiles each (128 registers).  One foreign part: row i lives in slot
+  // i mod 4 and is requested four rows ahead; two: rows i of f0 and f1 live in slots 2 (i mod 2) and
+  // 2 (i mod 2) + 1, two rows ahead.  Written and read under the same conditions.
+  f32x4_t slots[4][8];
+  auto fetch_row = [&](const __amdgpu_buffer_rsrc_t& from, int i, int slot) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        others[i % DEPTH][0][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(t.f0, lane16, (i * 8 + j) * 1024, AGENT));
-    }
+    for (int j = 0; j < 8; ++j)
+      slots[slot][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(from, lane16, (i * 8 + j) * 1024, AGENT));
+  };
+  // what has to be requested once row `done` (-1: nothing yet) has been consumed
+  auto fetch_after = [&](int done) {
     if (two) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        others[i % DEPTH][1][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(t.f1, lane16, (i * 8 + j) * 1024, AGENT));
+      const int i = done + 2;
+      if (done < 0) {
+        fetch_row(t.f0, 0, 0); fetch_row(t.f1, 0, 1); fetch_row(t.f0, 1, 2); fetch_row(t.f1, 1, 3);
+      } else if (i < 8) {
+        fetch_row(t.f0, i, 2 * (i % 2));
+        fetch_row(t.f1, i, 2 * (i % 2) + 1);
+      }
+    } else if (one) {
+      const int i = done + 4;
+      if (done < 0) {
+        fetch_row(t.f0, 0, 0); fetch_row(t.f0, 1, 1); fetch_row(t.f0, 2, 2); fetch_row(t.f0, 3, 3);
+      } else if (i < 8) {
+        fetch_row(t.f0, i, i % 4);
+      }
     }
   };
-#pragma unroll
-  for (int i = 0; i < DEPTH; ++i) fetch(i);
+  fetch_after(-1);
 
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
@@ -225,14 +238,14 @@ __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x
         // (f0 + u) + w with (u, w) = (own, f1) or (f1, own)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const f32x4_t f0 = others[i % DEPTH][0][j], f1 = others[i % DEPTH][1][j];
+          const f32x4_t f0 = slots[2 * (i % 2)][j], f1 = slots[2 * (i % 2) + 1][j];
 #pragma unroll
           for (int e = 0; e < 4; ++e) a[j][e] = (f0[e] + (last ? f1[e] : a[j][e])) + (last ? a[j][e] : f1[e]);
         }
       } else if (one) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const f32x4_t f0 = others[i % DEPTH][0][j];
+          const f32x4_t f0 = slots[i % 4][j];
 #pragma unroll
           for (int e = 0; e < 4; ++e) a[j][e] += f0[e];
         }
@@ -260,10 +273,8 @@ __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x
         const int c = 2 * j + (g >> 1);
         *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
       }
-      if (i + DEPTH < 8) {   // the row's registers are free again
-        SRT_FENCE();
-        fetch(i + DEPTH);
-      }
+      SRT_FENCE();
+      fetch_after(i);   // the row's registers are free again
     }
     SRT_FENCE();
     const bool fix = FIXUP && __builtin_amdgcn_ballot_w64(nan) != 0;
