@@ -282,20 +282,26 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
   const int n_rd = wave_n0 + 8 * rd_chunk;
   const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8 (checked on the host): the chunk is whole
 
+  // staging address of accumulator tile (ii, j): row 16 ii + jn, chunk (2 j + g / 2) ^ jn -- the lane's part of
+  // it is the same for every ii (a row group is 4096 bytes further: an immediate offset of the write)
+  uint32_t wr[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    wr[j] = stage + (uint32_t)jn * 256u + (uint32_t)(g & 1) * 8u + (uint32_t)(((2 * j + (g >> 1)) ^ jn) << 4);
+
 #pragma unroll
   for (int half = 0; half < TM * 16 / ROWS; ++half) {
     bool nan = false;
 #pragma unroll
     for (int ii = 0; ii < ROWS / 16; ++ii) {
       const int i = (ROWS / 16) * half + ii;
-      const int row = 16 * ii + jn;
-      const uint32_t row_addr = stage + (uint32_t)row * 256u + (uint32_t)(g & 1) * 8u;
       SRT_FENCE();
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         float a0 = acc[i][j][0], a1 = acc[i][j][1], a2 = acc[i][j][2], a3 = acc[i][j][3];
-        // one copy out of the accumulator registers, here, for both the test and the conversion
+#ifdef SRT_EPILOGUE_PIN   // measurement builds: pinning the copies costs three register moves per tile
         asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
+#endif
         if (HAS_BIAS) {
           const float br = T::to_float((S)(b[i].x & 0xffffu));
           a0 += per_row ? br : T::to_float((S)(b[j].x & 0xffffu));
@@ -313,8 +319,7 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
         }
         if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
         const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};
-        const int c = 2 * j + (g >> 1);
-        *reinterpret_cast<SRT_LDS u32x2_t*>(row_addr + (uint32_t)((c ^ (row & 15)) << 4)) = w;
+        *reinterpret_cast<SRT_LDS u32x2_t*>(wr[j] + (uint32_t)ii * 4096u) = w;
       }
     }
     SRT_FENCE();
