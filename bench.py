@@ -126,7 +126,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     ap.add_argument("--only", default=None,
                     help="run one configuration alone, a few launches, and exit (for profilers): headline, cfg3_tn, cfg3_nt, "
-                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, few_tiles, dense_backward, add, add_bias, tanh, cast")
+                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, few_tiles, fp16_4096, fp32_4096, dense_backward, add, "
+                         "add_bias, tanh, cast")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the single-GPU matmul path; run it with --gpus 1 "
@@ -223,7 +224,8 @@ def main():
 class Bench:
     """The configurations, each as one prepared foreign call per step."""
 
-    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1", "few_tiles")
+    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1", "few_tiles",
+                 "fp16_4096", "fp32_4096")
 
     def __init__(self, srt, native, q):
         self.srt, self.native, self.q = srt, native, q
@@ -331,6 +333,24 @@ class Bench:
             return {"name": "bf16 1024x4096x4096 (64 tiles of 256 x 256)", "call": call, "kernel": kernel,
                     "flops": 2.0 * 1024 * 4096 * 4096, "bytes": (1024 * 4096 * 2 + 4096 * 4096) * 2, "bound": "mfma",
                     "dtype": "bf16", "steps": 200}
+        if name == "fp16_4096":
+            # not a BASELINE configuration: the headline kernel's fp16 instantiation, one tile per compute unit
+            g = rng(6)
+            a = srt.Tensor((g.standard_normal((4096, 4096), dtype=np.float32) / np.float32(64)).astype(np.float16))
+            b = srt.Tensor(g.standard_normal((4096, 4096), dtype=np.float32).astype(np.float16))
+            c = srt.Tensor(shape=[4096, 4096], dtype=np.float16)
+            call, kernel = self.prepared(a, False, b, False, c)
+            return {"name": "fp16 4096^3", "call": call, "kernel": kernel, "flops": 2.0 * 4096 ** 3,
+                    "bytes": 3 * 4096 * 4096 * 2, "bound": "mfma", "dtype": "f16", "steps": 100}
+        if name == "fp32_4096":
+            # not a BASELINE configuration: the fp32 matrix path where it is not launch-sized
+            g = rng(7)
+            a = srt.Tensor(g.uniform(-1, 1, (4096, 4096)).astype(np.float32))
+            b = srt.Tensor(g.uniform(-1, 1, (4096, 4096)).astype(np.float32))
+            c = srt.Tensor(shape=[4096, 4096], dtype=np.float32)
+            call, kernel = self.prepared(a, False, b, False, c)
+            return {"name": "fp32 4096^3", "call": call, "kernel": kernel, "flops": 2.0 * 4096 ** 3,
+                    "bytes": 3 * 4096 * 4096 * 4, "bound": "mfma", "dtype": "f32", "steps": 20}
         if name == "cfg1":
             g = rng(0)
             a1 = srt.Tensor(g.uniform(-1, 1, (512, 512)).astype(np.float32))
