@@ -323,7 +323,7 @@ class Bench:
                     "flops": 2.0 * 32 * 256 ** 3, "bytes": 32 * 3 * 256 * 256 * 2, "bound": "mfma", "dtype": "f16",
                     "steps": 200}
         if name == "few_tiles":
-            # not a BASELINE configuration: a quarter-full device with a long k loop, the case of the
+            # not one of the five benchmark configurations: a quarter-full device with a long k loop, the case of the
             # tail-sharing form of the headline kernel (every tile cut along k into three parts)
             g = rng(5)
             a = srt.Tensor(bf16_encode(g.standard_normal((1024, 4096), dtype=np.float32) / np.float32(64)))
@@ -334,7 +334,7 @@ class Bench:
                     "flops": 2.0 * 1024 * 4096 * 4096, "bytes": (1024 * 4096 * 2 + 4096 * 4096) * 2, "bound": "mfma",
                     "dtype": "bf16", "steps": 200}
         if name == "fp16_4096":
-            # not a BASELINE configuration: the headline kernel's fp16 instantiation, one tile per compute unit
+            # not one of the five benchmark configurations: the headline kernel's fp16 instantiation, one tile per compute unit
             g = rng(6)
             a = srt.Tensor((g.standard_normal((4096, 4096), dtype=np.float32) / np.float32(64)).astype(np.float16))
             b = srt.Tensor(g.standard_normal((4096, 4096), dtype=np.float32).astype(np.float16))
@@ -343,7 +343,7 @@ class Bench:
             return {"name": "fp16 4096^3", "call": call, "kernel": kernel, "flops": 2.0 * 4096 ** 3,
                     "bytes": 3 * 4096 * 4096 * 2, "bound": "mfma", "dtype": "f16", "steps": 100}
         if name == "fp32_4096":
-            # not a BASELINE configuration: the fp32 matrix path where it is not launch-sized
+            # not one of the five benchmark configurations: the fp32 matrix path where it is not launch-sized
             g = rng(7)
             a = srt.Tensor(g.uniform(-1, 1, (4096, 4096)).astype(np.float32))
             b = srt.Tensor(g.uniform(-1, 1, (4096, 4096)).astype(np.float32))
