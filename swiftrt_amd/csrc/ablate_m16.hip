@@ -8,7 +8,7 @@
 //   -DABL_TAIL=1          (with ABL_DEEP) the tail-sharing form; every element of its result is then compared
 //                         with the plain 64-deep kernel's
 //   -DABL_AKC / -DABL_BKC operand layouts (defaults 1 / 0: the headline's row-major A and B)
-// Run: ablate_m16 [normal|zero] [M N K]; operands ~ N(0,1)/sqrt(K) (generated on the device) or zeros.
+// Run: ablate_m16 [normal|zero] [M N K [pad]]; pad: elements added to the pitch of the operands' rows; operands ~ N(0,1)/sqrt(K) (generated on the device) or zeros.
 // Prints one line: variant, data, median and minimum time per launch, TFLOP/s, and (unablated builds) the
 // largest error of 64 sampled results against a double-precision dot product.
 #define SRT_M16_ANY_RING_DEPTH 1
@@ -93,14 +93,18 @@ int main(int argc, char** argv) {
   const bool zero = argc > 1 && strcmp(argv[1], "zero") == 0;
   int M = 8192, N = 8192, K = 8192;
   if (argc > 4) { M = atoi(argv[2]); N = atoi(argv[3]); K = atoi(argv[4]); }
+  const int pad = argc > 5 ? atoi(argv[5]) : 0;   // elements added to the pitch of every operand row (a multiple of 8)
   if (M % 256 || N % 256 || K % 32 || K < 160) { fprintf(stderr, "M, N multiples of 256; K a multiple of 32, at least 160\n"); return 1; }
   uint16_t *a, *b, *c;
-  CHECK(hipMalloc(&a, (size_t)M * K * 2));
-  CHECK(hipMalloc(&b, (size_t)K * N * 2));
+  // pitches of the stored rows: A is [M][K] or [K][M], B is [N][K] or [K][N]
+  const size_t a_rows = ABL_AKC ? M : K, a_pitch = (ABL_AKC ? K : M) + pad;
+  const size_t b_rows = ABL_BKC ? N : K, b_pitch = (ABL_BKC ? K : N) + pad;
+  CHECK(hipMalloc(&a, a_rows * a_pitch * 2));
+  CHECK(hipMalloc(&b, b_rows * b_pitch * 2));
   CHECK(hipMalloc(&c, (size_t)M * N * 2));
   const float scale = 1.0f / sqrtf((float)K);
-  hipLaunchKernelGGL(fill_normal, dim3(4096), dim3(256), 0, 0, a, (size_t)M * K, scale, 0x1234567u, zero ? 1 : 0);
-  hipLaunchKernelGGL(fill_normal, dim3(4096), dim3(256), 0, 0, b, (size_t)K * N, scale, 0x89abcdeu, zero ? 1 : 0);
+  hipLaunchKernelGGL(fill_normal, dim3(4096), dim3(256), 0, 0, a, a_rows * a_pitch, scale, 0x1234567u, zero ? 1 : 0);
+  hipLaunchKernelGGL(fill_normal, dim3(4096), dim3(256), 0, 0, b, b_rows * b_pitch, scale, 0x89abcdeu, zero ? 1 : 0);
   CHECK(hipDeviceSynchronize());
 
   srt::GemmProblem p{};
@@ -108,8 +112,8 @@ int main(int argc, char** argv) {
   p.M = M; p.N = N; p.K = K; p.batch = 1;
   p.A = a; p.B = b; p.C = c;
   // A stored [M, K] (k-contiguous) or [K, M]; B stored [N, K] (k-contiguous) or [K, N]
-  if (ABL_AKC) { p.sam = K; p.sak = 1; } else { p.sam = 1; p.sak = M; }
-  if (ABL_BKC) { p.sbn = K; p.sbk = 1; } else { p.sbn = 1; p.sbk = N; }
+  if (ABL_AKC) { p.sam = (long long)a_pitch; p.sak = 1; } else { p.sam = 1; p.sak = (long long)a_pitch; }
+  if (ABL_BKC) { p.sbn = (long long)b_pitch; p.sbk = 1; } else { p.sbn = 1; p.sbk = (long long)b_pitch; }
   p.scm = N; p.scn = 1;
   p.activation = srtActivationIdentity;
 
@@ -143,7 +147,7 @@ int main(int argc, char** argv) {
   double worst = -1.0;
   if (SRT_ABLATE == 0 && !zero) {
     // 64 sampled results against double-precision dot products of the stored operands
-    std::vector<uint16_t> ha((size_t)M * K), hb((size_t)K * N), hc((size_t)M * N);
+    std::vector<uint16_t> ha(a_rows * a_pitch), hb(b_rows * b_pitch), hc((size_t)M * N);
     CHECK(hipMemcpy(ha.data(), a, ha.size() * 2, hipMemcpyDeviceToHost));
     CHECK(hipMemcpy(hb.data(), b, hb.size() * 2, hipMemcpyDeviceToHost));
     CHECK(hipMemcpy(hc.data(), c, hc.size() * 2, hipMemcpyDeviceToHost));
