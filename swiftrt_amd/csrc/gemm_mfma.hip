@@ -685,10 +685,13 @@ int mfma_select(const GemmProblem& p) {
   //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
   //    NN 1440 -> 1505 TFLOP/s, NT 1420 -> 1531, TN 1443 -> 1501, TT 1477 -> 1538), and of the 32x32x16
   //    64-deep kernel that two k-contiguous operands used to take for short k loops; it needs whole units
+  //    (K a multiple of 64, at least 512).  With an A that is not k-contiguous -- no half tiles -- it also takes
+  //    over from the 32x32x16 ring below half a device (2048 x 3072 x 1024, 96 tiles: 23-24 us against 26; 2048 x
+  //    2048 x 2048, 64 tiles: 38-40 against 40-41; 1024 x 2048 x 1024, 32 tiles: 23 against 25)
   const bool deep_ok = p.K % 64 == 0 && p.K >= 512;
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
-  else if (whole_ok && deep_ok && t256 >= 128) tile = 9;
+  else if (whole_ok && deep_ok && (t256 >= 128 || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
   else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
   else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
   else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout & 2) == 0))) tile = 1;
