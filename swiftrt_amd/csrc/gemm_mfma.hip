@@ -663,7 +663,9 @@ int mfma_select(const GemmProblem& p) {
   // 1024: 21 us against 28 us; 8 x 512 x 2048 x 256: 10.5 against 14.0; but 16 x 256 x 2048 x 2048: 81 us
   // against 51 us for whole tiles).
   const int m_rest = p.M % 256;
-  const bool half_nt = p.batch == 1 ? (th >= 96 && rounds_h == 1) : ((m_rest > 0 && m_rest <= 128) || p.K <= 512);
+  // (from 72 half tiles in one round: 1536 x 1536 x 1024 x . W^T, 72 of them: 14.8 us against 16.8 for 64 x 64 tiles;
+  // 1024 x 2048 x 2048, 64 of them: 25.7 against 22.9)
+  const bool half_nt = p.batch == 1 ? (th >= 72 && rounds_h == 1) : ((m_rest > 0 && m_rest <= 128) || p.K <= 512);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
@@ -680,7 +682,9 @@ int mfma_select(const GemmProblem& p) {
   // 6.6; but 64 x 128 x 1024 x 128: 12.3 against 18.5).
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
                                    (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
-  const long long ring_from = layout == 3 ? 96 : (p.K >= 1024 ? 24 : 32);
+  // (with neither operand k-contiguous the 64 x 64 kernel transposes both in registers: whole tiles from 12 up,
+  // 512 x 1536 x 1024: 22.7 us against 24.9)
+  const long long ring_from = layout == 3 ? 96 : layout == 0 ? (p.K >= 1024 ? 12 : 24) : (p.K >= 1024 ? 24 : 32);
   //  * the 64-deep form of the 16x16x32 kernel (whole-line loads of k-contiguous operands, one barrier per 128
   //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
   //    NN 1440 -> 1505 TFLOP/s, NT 1420 -> 1531, TN 1443 -> 1501, TT 1477 -> 1538), and of the 32x32x16
@@ -688,9 +692,15 @@ int mfma_select(const GemmProblem& p) {
   //    (K a multiple of 64, at least 512).  With an A that is not k-contiguous -- no half tiles -- it also takes
   //    over from the 32x32x16 ring below half a device (2048 x 3072 x 1024, 96 tiles: 23-24 us against 26; 2048 x
   //    2048 x 2048, 64 tiles: 38-40 against 40-41; 1024 x 2048 x 1024, 32 tiles: 23 against 25)
-  const bool deep_ok = p.K % 64 == 0 && p.K >= 512;
+  //    Four units (K = 256) are enough: 2048 x 3072 x 256 with A m-contiguous 11.8 us against 12.8-13.8 for the
+  //    32-deep kernels, 3072 x 8192 x 256 x . W^T 21.3 against 24.7.
+  const bool deep_ok = p.K % 64 == 0 && p.K >= 256;
+  // an m-contiguous A against a k-contiguous B, a short k loop and under 64 tiles: the 64 x 64 kernel (1024 x 2048
+  // x 256: 9.6 us against 12.4 for whole tiles; 512 x 4096 x 512: 13.2 against 15.0; at 64 tiles whole tiles win)
+  const bool small_tt = layout == 1 && p.K <= 512 && t256 < 64;
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
+  else if (small_tt) tile = 3;
   else if (whole_ok && deep_ok && (t256 >= 128 || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
   else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
   else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
@@ -792,11 +802,18 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   // k-contiguous the 64 x 64 kernel holds out longer -- 192 x 512 x 2048: 19 us against 22 us, but
   // 3072 x 128 x 3072: 33 us against 28 us)
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256);
-  if (t256 <= 24 && parts >= 4 && p.K >= (layout == 3 ? 3072 : 2048)) return true;
+  // (a k-contiguous A has half tiles: 1024 x 1536 x 2048, 24 tiles: 25.5 us in half tiles against 27.9 in four parts;
+  // with neither operand k-contiguous even two parts of a handful of tiles pay: 512 x 512 x 1024: 20 us against 25)
+  if (t256 <= 24 && parts >= 4 && p.K >= ((layout & 2) != 0 ? 3072 : 2048)) return true;
+  if (layout == 0 && t256 <= 8 && p.K >= 1024) return true;
+  if (layout == 2 && t256 <= 4 && parts >= 4 && p.K >= 2048) return true;  // (512 x 512 x 2048: 21 us against 25 in half tiles)
   if ((layout & 2) == 0 || p.M <= 128) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;
-  return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 192));
+  // (four parts also while half tiles would fill under 40 % of the device: 1536 x 1536 x 4096, 72 half tiles:
+  // 38 us against 46; 512 x 6144 x 4096, 96: 40 against 46)
+  const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256);
+  return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 192 || th <= 96));
 }
 
 // Whether the heuristic takes the tail-sharing form of the 64-deep kernel (tile 10): the tiles left over
@@ -813,17 +830,28 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
 //                             x . W: 57-59 against 55-57 (half tiles in one round: those stay), K = 8192: 98-103
 //                             against 103-110
 //   144 tiles                 3072 x 3072 x 4096: 67-69 against 71-73 (whole tiles)
-//   below 64 tiles split-K cuts deeper (32 tiles, K = 16384: 73 against 104); from 160 tiles up whole tiles
+//   48 tiles                  1536 x 2048 x 4096 x . W^T: 41 against 44 (split-K)
+//   below that split-K cuts deeper (32 tiles, K = 16384: 73 against 104); from 160 tiles up whole tiles
 //   are as good (160 tiles: 74-76 against 72-75)
 bool mfma_prefers_tail(const GemmProblem& p) {
-  if (p.K < 4096 || mfma_config(p, 10) == 0) return false;
+  if (p.K < 2048 || mfma_config(p, 10) == 0) return false;
   const int layout = mfma_layout(p);
   const long long cus = compute_units();
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
   const long long left = t256 % cus;
-  if (t256 >= cus) return left > 0 && 8 * left <= cus;   // a handful left over: see above
-  if (left < 64 || left > 160) return false;
+  if (p.K < 4096) {
+    // an A that is not k-contiguous has no half tiles to fall back on: from K = 2048 (1024 x 4096 x 2048, 64 tiles:
+    // 32.5 us against 37.7 for split-K; 1536 x 4096 x 2048, 96 tiles: 34.4 against 40.1 whole)
+    return (layout & 2) == 0 && t256 >= (p.M >= 512 ? 48 : 64) && t256 <= 128;
+  }
+  if (t256 >= cus) {
+    // a handful left over (see above), or one round and up to half of another with a k loop long enough to
+    // carry the adding up (3072 x 8192 x 8192, 384 tiles: 275 us against 298)
+    return left > 0 && (8 * left <= cus || (t256 < 2 * cus && 2 * left <= cus && p.K >= 8192));
+  }
+  if (left < 48 || left > 160) return false;
+  if (left < 64 && p.M < 512) return false;  // (the 48-tile figures are of 2-6 rows of tiles; one row stays with split-K)
   if (left <= 96) return true;
   return layout == 3 || (layout & 2) == 0 || p.K >= 8192 || th > cus;
 }

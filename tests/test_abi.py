@@ -216,8 +216,8 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_256x256_splitk"
     assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: from K = 2048
     assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x256_m16_k64"    # 32 tiles: whole tiles from 24 up
-    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_64x64"          # 16 tiles
-    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x256_m16_k64"    # two parts at K = 2048 do not pay
+    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_256x256_m16_k64"    # 16 tiles, neither operand k-contiguous: whole tiles from 12 up
+    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x256_m16_k64_tail"   # 128 tiles, K = 2048, no half tiles: cut in two
     # mid-size problems: the 256 x 256 kernels from 24 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16_k64"             # 144 tiles, long k loop
@@ -226,7 +226,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16"             # 128 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16"
     assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16"             # 256 half tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256_splitk" # A not k-contiguous: whole tiles, K split
+    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256_m16_k64_tail"   # A not k-contiguous: whole tiles cut along k
     assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x256_m16_k64"
     # 258 whole tiles: a whole round, and the two left over cut along k in three parts each
     assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_256x256_m16_k64_tail"
