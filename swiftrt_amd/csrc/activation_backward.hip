@@ -13,7 +13,7 @@
 //           rows w, w + 4, ... of its chunk, so every wave instruction moves one 1 KiB row segment
 //   sums    8 (V) fp32 column sums per lane in registers, waves combined through LDS, one fp32
 //           partial row per chunk in a workspace; a second tiny kernel adds the chunks in a fixed
-//           order (deterministic, no atomics)
+//           order (deterministic, no atomics), eight rows in flight per lane
 //   V = 1   same structure for layouts the vector path excludes (any strides)
 #include "gemm_common.h"
 #include "status.h"
@@ -62,7 +62,7 @@ __device__ __forceinline__ Pack<T, V> load_once(const typename T::storage* p) {
   }
 }
 
-template <typename T, int V>
+template <typename T, int V, int R>
 __global__ __launch_bounds__(256) void activation_backward_kernel(BackwardProblem p) {
   using S = typename T::storage;
   __shared__ float red[4][64 * V];
@@ -77,47 +77,44 @@ __global__ __launch_bounds__(256) void activation_backward_kernel(BackwardProble
 #pragma unroll
   for (int i = 0; i < V; ++i) sum[i] = 0.0f;
   if (n0 < p.N) {
-    // two rows per trip (both rows' loads are issued before either is used)
-    for (int m = m_begin + wave; m < m_end; m += 8) {
-      const int m2 = m + 4;
-      const bool second = m2 < m_end;
-      float fy[2][V], fd[2][V];
-      if (V > 1) {
-        const Pack<T, V> py0 = load_once<T, V>(y + (long long)m * p.sym + n0);
-        const Pack<T, V> pd0 = load_once<T, V>(dy + (long long)m * p.sdm + n0);
-        Pack<T, V> py1 = py0, pd1 = pd0;
-        if (second) {
-          py1 = load_once<T, V>(y + (long long)m2 * p.sym + n0);
-          pd1 = load_once<T, V>(dy + (long long)m2 * p.sdm + n0);
-        }
+    // R rows per trip (all their loads are issued before any is used); a row past the chunk's end repeats
+    // the trip's first row and is not stored or summed
+    for (int m = m_begin + wave; m < m_end; m += 4 * R) {
+      Pack<T, V> py[R], pd[R];
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          fy[0][i] = T::to_float(py0.v[i]); fd[0][i] = T::to_float(pd0.v[i]);
-          fy[1][i] = T::to_float(py1.v[i]); fd[1][i] = T::to_float(pd1.v[i]);
-        }
-      } else {
-        fy[0][0] = T::to_float(y[(long long)m * p.sym + (long long)n0 * p.syn]);
-        fd[0][0] = T::to_float(dy[(long long)m * p.sdm + (long long)n0 * p.sdn]);
-        fy[1][0] = fy[0][0]; fd[1][0] = fd[0][0];
-        if (second) {
-          fy[1][0] = T::to_float(y[(long long)m2 * p.sym + (long long)n0 * p.syn]);
-          fd[1][0] = T::to_float(dy[(long long)m2 * p.sdm + (long long)n0 * p.sdn]);
+      for (int r = 0; r < R; ++r) {
+        const int row = m + 4 * r < m_end ? m + 4 * r : m;
+        if (V > 1) {
+          py[r] = load_once<T, V>(y + (long long)row * p.sym + n0);
+          pd[r] = load_once<T, V>(dy + (long long)row * p.sdm + n0);
+        } else {
+          py[r].v[0] = y[(long long)row * p.sym + (long long)n0 * p.syn];
+          pd[r].v[0] = dy[(long long)row * p.sdm + (long long)n0 * p.sdn];
         }
       }
 #pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        if (r == 1 && !second) break;
-        const int row = r ? m2 : m;
+      for (int r = 0; r < R; ++r) {
+        const int row = m + 4 * r;
+        if (r > 0 && row >= m_end) break;
         Pack<T, V> out;
+        float gs[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          float g = fd[r][i] * activation_slope(p.activation, p.coef, fy[r][i]);
+          float g = T::to_float(pd[r].v[i]) * activation_slope(p.activation, p.coef, T::to_float(py[r].v[i]));
           // keep the product as an fp32 value: without this the compiler merges the multiply and
           // the conversion to half into one mixed-precision instruction that rounds the exact
           // product once, which differs from "fp32 product, then round" on ties
           asm volatile("" : "+v"(g));
-          out.v[i] = T::from_float(g);
+          gs[i] = g;
           sum[i] += g;
+        }
+        if constexpr (V > 1 && T::dtype == srtReal16BF) {
+          uint32_t w[V / 2];
+          encode_bf16<V>(gs, w);
+          out = __builtin_bit_cast(Pack<T, V>, w);
+        } else {
+#pragma unroll
+          for (int i = 0; i < V; ++i) out.v[i] = T::from_float(gs[i]);
         }
         if (V > 1) *reinterpret_cast<Pack<T, V>*>(dx + (long long)row * p.sxm + n0) = out;
         else dx[(long long)row * p.sxm + (long long)n0 * p.sxn] = out.v[0];
@@ -137,29 +134,38 @@ __global__ __launch_bounds__(256) void activation_backward_kernel(BackwardProble
   }
 }
 
-// Adds the chunks' partial rows: 64 columns per workgroup, the four waves take every fourth chunk
-// (four independent loads in flight per lane) and meet in LDS.  The order of the additions is fixed.
+// Adds the chunks' partial rows: 64 columns per workgroup of sixteen waves, wave w takes chunks w, w + 16, ...,
+// eight rows at a time (eight independent loads in flight per lane; a row past the last chunk is not loaded and
+// counts as zero), and the waves meet in LDS: up to 128 chunks cost one round of loads.  The order of the
+// additions is fixed.
+constexpr int kFinishWaves = 16;
 template <typename T>
-__global__ __launch_bounds__(256) void bias_gradient_finish_kernel(const float* partial, int chunks, int N,
-                                                                   typename T::storage* dbias, long long stride) {
-  __shared__ float red[4][64];
+__global__ __launch_bounds__(64 * kFinishWaves) void bias_gradient_finish_kernel(const float* partial, int chunks, int N,
+                                                                                 typename T::storage* dbias, long long stride) {
+  __shared__ float red[kFinishWaves][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = blockIdx.x * 64 + lane;
-  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = 0.0f;
   if (n < N) {
-    int c = wave;
-    for (; c + 12 < chunks; c += 16) {
-      s0 += partial[(long long)c * N + n];
-      s1 += partial[(long long)(c + 4) * N + n];
-      s2 += partial[(long long)(c + 8) * N + n];
-      s3 += partial[(long long)(c + 12) * N + n];
+    for (int c = wave; c < chunks; c += 8 * kFinishWaves) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        v[i] = c + kFinishWaves * i < chunks ? partial[(long long)(c + kFinishWaves * i) * N + n] : 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s[i] += v[i];
     }
-    for (; c < chunks; c += 4) s0 += partial[(long long)c * N + n];
   }
-  red[wave][lane] = (s0 + s1) + (s2 + s3);
+  red[wave][lane] = ((s[0] + s[1]) + (s[2] + s[3])) + ((s[4] + s[5]) + (s[6] + s[7]));
   __syncthreads();
-  if (wave == 0 && n < N)
-    dbias[(long long)n * stride] = T::from_float((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]));
+  if (wave == 0 && n < N) {
+    float t[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = (red[4 * i][lane] + red[4 * i + 1][lane]) + (red[4 * i + 2][lane] + red[4 * i + 3][lane]);
+    dbias[(long long)n * stride] = T::from_float((t[0] + t[1]) + (t[2] + t[3]));
+  }
 }
 
 // Scratch of the entry point that allocates nothing (srtActivationBackwardBiasNoAlloc): the chunks'
@@ -205,7 +211,9 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
   const int V = vec ? VEC : 1;
   const int strips = (p.N + 64 * V - 1) / (64 * V);
   // enough workgroups to keep every memory channel busy, but at least 16 rows per chunk
-  int chunks = (4096 + strips - 1) / strips;
+  // (1024 to 6144 workgroups and one, two or four rows per trip all measure the same on 4096 x 11008; fewer chunks
+  // are fewer partial rows for the second kernel)
+  int chunks = (2048 + strips - 1) / strips;
   const int max_chunks = (p.M + 15) / 16;
   if (chunks > max_chunks) chunks = max_chunks;
   if (chunks > 65535) chunks = 65535;
@@ -231,11 +239,11 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
   }
   p.partial = (float*)workspace;
   const dim3 grid(strips, chunks);
-  if (vec) hipLaunchKernelGGL((activation_backward_kernel<T, VEC>), grid, dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL((activation_backward_kernel<T, 1>), grid, dim3(256), 0, stream, p);
+  if (vec) hipLaunchKernelGGL((activation_backward_kernel<T, VEC, 2>), grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((activation_backward_kernel<T, 1, 2>), grid, dim3(256), 0, stream, p);
   hipError_t e = launch_status(stream);
   if (e == hipSuccess && dbias) {
-    hipLaunchKernelGGL((bias_gradient_finish_kernel<T>), dim3((p.N + 63) / 64), dim3(256), 0, stream,
+    hipLaunchKernelGGL((bias_gradient_finish_kernel<T>), dim3((p.N + 63) / 64), dim3(64 * kFinishWaves), 0, stream,
                        (const float*)workspace, chunks, p.N, (typename T::storage*)dbias, dbias_stride);
     e = launch_status(stream);
   }

@@ -57,6 +57,24 @@ struct BF16 {
   }
 };
 
+// V fp32 values (V even) -> V bfloat16 in V / 2 dwords, bit for bit what BF16::from_float gives for each: when none
+// of them is a NaN (one unordered compare per pair) the hardware converter does two values per instruction;
+// the scalar encoder (NaN -> 0x7FFF) runs only for a lane that holds a NaN.
+template <int V>
+__device__ __forceinline__ void encode_bf16(const float (&r)[V], uint32_t (&w)[V / 2]) {
+  static_assert(V % 2 == 0, "pairs");
+  bool clean = true;
+#pragma unroll
+  for (int i = 0; i < V; i += 2) clean &= !__builtin_isunordered(r[i], r[i + 1]);
+  if (clean) {
+#pragma unroll
+    for (int i = 0; i < V; i += 2) w[i / 2] = BF16::pack2<false>(r[i], r[i + 1]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < V; i += 2) w[i / 2] = BF16::pack2<true>(r[i], r[i + 1]);
+  }
+}
+
 struct F16 {
   using storage = uint16_t;
   static constexpr int dtype = srtReal16F;
@@ -109,6 +127,10 @@ __device__ __forceinline__ float apply_activation(int activation, float coef, fl
 // at fp32 rounding level everywhere.  NaN in, NaN out; +-inf give the limits.
 template <int ACT>
 __device__ __forceinline__ float activation16_ct(float coef, float x) {
+  // fused multiply-adds here whatever the translation unit's setting (the element-wise kernels are compiled
+  // without contraction for their basic operations): three instructions fewer per tanh, and the same bits
+  // as the GEMM epilogues' use of this function
+#pragma clang fp contract(fast)
   if (ACT == srtActivationSigmoid) return __fdividef(1.0f, 1.0f + __expf(-x));
   if (ACT == srtActivationTanh) {
     // tanh|x| = 1 - 2 / (exp(2|x|) + 1): exp overflows to +inf for large |x|, giving exactly 1

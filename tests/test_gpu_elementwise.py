@@ -46,6 +46,55 @@ def test_binary_dense_bit_exact(op, fn, dt):
 
 
 @pytest.mark.parametrize("dt", DTS)
+def test_vector_path_special_values_bit_exact(dt):
+    """NaNs, infinities, sums that overflow to infinity, products that land among the subnormals and exact
+    ties, scattered over rows that the 16-byte path handles: the 16-bit encoders must agree with the oracle's
+    (NaN -> 0x7FFF for bfloat16, round to nearest even) whichever lanes share a vector with a NaN."""
+    g = H.rng(21)
+    shape = (96, 512)
+    a = (g.standard_normal(shape) * 2.0).astype(np.float32)
+    b = (g.standard_normal(shape) * 2.0).astype(np.float32)
+    big = {H.F32: 3.0e38, H.F16: 60000.0, H.BF16: 3.0e38}[dt]
+    tiny = {H.F32: 1.0e-19, H.F16: 2.0e-4, H.BF16: 1.0e-19}[dt]
+    where = g.integers(0, 12, shape)
+    a[where == 0] = np.nan
+    b[where == 1] = np.nan
+    a[where == 2] = np.inf
+    b[where == 3] = -np.inf
+    a[where == 4] = big
+    b[where == 4] = big            # the sum overflows
+    a[where == 5] = tiny
+    b[where == 5] = tiny * 0.37    # the product is a subnormal of the element type (or underflows)
+    a[where == 6] = 1.0
+    b[where == 6] = {H.F32: 2.0 ** -24, H.F16: 2.0 ** -11, H.BF16: 2.0 ** -8}[dt]   # 1 + half a step: a tie
+    a[where == 7] = -0.0
+    b[where == 7] = 0.0
+    a_st, b_st = H.encode(a, dt), H.encode(b, dt)
+    ta, tb = srt.Tensor(a_st), srt.Tensor(b_st)
+    q = srt.current_queue()
+
+    def same(got_st, want_st):
+        # bfloat16 has one NaN (0x7FFF); fp32 and fp16 NaNs may differ in sign between host and device
+        if dt == H.BF16:
+            return np.array_equal(got_st, want_st)
+        nan_g, nan_w = np.isnan(H.decode(got_st)), np.isnan(H.decode(want_st))
+        return np.array_equal(nan_g, nan_w) and np.array_equal(got_st[~nan_g], want_st[~nan_w])
+
+    for op, fn in EXACT_BINARY:
+        out = srt.Tensor(shape=ta.shape, dtype=ta.dtype)
+        getattr(q, fn)(ta, tb, out)
+        assert same(out.array(), ora.elementwise(op, a_st, b_st)), op
+    out = srt.Tensor(shape=ta.shape, dtype=ta.dtype)
+    q.neg(ta, out)
+    assert same(out.array(), ora.elementwise("neg", a_st))
+    # the backward epilogue's dx goes through the same encoder
+    dx = srt.Tensor(shape=ta.shape, dtype=ta.dtype)
+    db = srt.Tensor(shape=[shape[1]], dtype=ta.dtype)
+    q.activation_backward(ta, tb, srt.ActivationType.identity, 0.0, dx, db)
+    assert same(dx.array(), ora.elementwise("mul", b_st, H.encode(np.ones(shape, np.float32), dt)))
+
+
+@pytest.mark.parametrize("dt", DTS)
 def test_binary_odd_sizes_and_misaligned_views(dt):
     """Extents that are not a multiple of the vector width and views that start off a 16-byte
     boundary take the element-at-a-time path of the same kernel."""
