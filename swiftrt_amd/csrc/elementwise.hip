@@ -20,6 +20,7 @@ namespace srt {
 namespace ew {
 
 constexpr int MAX_RANK = 4;   // after collapsing adjacent dimensions
+constexpr int kVectorsPerLane = 4;   // (two: sigmoid 32.2 -> 30.7 us, bias-broadcast add 33.3 -> 36.8, the rest unchanged)
 
 // ---- operations -----------------------------------------------------------------------------
 struct Add { static __device__ __forceinline__ float apply(float a, float b) { return a + b; } };
@@ -94,9 +95,9 @@ __global__ __launch_bounds__(256) void map_kernel(Map m) {
   // this device the memory parallelism of a streaming kernel comes from the waves: the same kernel with all
   // four vectors' loads issued before the first use needs 92 registers (five waves) and ran 15-20 % slower,
   // and four consecutive rows per lane with a row-broadcast operand loaded once were no faster either.
-  const unsigned long long base = (unsigned long long)blockIdx.x * (256 * 4) + threadIdx.x;
+  const unsigned long long base = (unsigned long long)blockIdx.x * (256 * kVectorsPerLane) + threadIdx.x;
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
+  for (int u = 0; u < kVectorsPerLane; ++u) {
     const unsigned long long id = base + (unsigned long long)u * 256;
     if (id >= m.total) break;
     // decompose the vector id over the collapsed dimensions
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(256) void map_kernel(Map m) {
 
 template <typename TI, typename TO, typename Op, int V>
 hipError_t launch_v(const Map& m, hipStream_t stream) {
-  const unsigned long long blocks = (m.total + 1023) / 1024;
+  const unsigned long long blocks = (m.total + 256 * kVectorsPerLane - 1) / (256 * kVectorsPerLane);
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
   hipLaunchKernelGGL((map_kernel<TI, TO, Op, V>), dim3((unsigned)blocks), dim3(256), 0, stream, m);
