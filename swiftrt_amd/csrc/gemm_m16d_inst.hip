@@ -17,6 +17,11 @@ hipError_t SRT_CAT(launch_m16d_tail, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(con
   return m16d::launch_tail<SRT_M16_TYPE, SRT_M16_AKC != 0, SRT_M16_BKC != 0>(p, stream);
 }
 
+// launch_m16d_partial_<type>_<akc><bkc>: the split-K pass (fp32 accumulators to a workspace)
+hipError_t SRT_CAT(launch_m16d_partial, SRT_M16_TYPE, SRT_M16_AKC, SRT_M16_BKC)(const GemmProblem& p, hipStream_t stream) {
+  return m16d::launch_partial<SRT_M16_TYPE, SRT_M16_AKC != 0, SRT_M16_BKC != 0>(p, stream);
+}
+
 // whether the tail-sharing form applies to `p` (defined once)
 #if SRT_M16_AKC == 0 && SRT_M16_BKC == 0
 bool SRT_CAT(m16d_tail_fits, SRT_M16_TYPE, x, x)(const GemmProblem& p) { return m16d::tail_fits(p); }

@@ -942,5 +942,11 @@ hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   return launch_kernel<T, A_KC, B_KC, EPI_PLAIN>(p, stream);
 }
 
+// The split-K pass: fp32 accumulators to a workspace, no epilogue arithmetic.
+template <typename T, bool A_KC, bool B_KC>
+hipError_t launch_partial(const GemmProblem& p, hipStream_t stream) {
+  return launch_kernel<T, A_KC, B_KC, EPI_PARTIAL>(p, stream);
+}
+
 }  // namespace m16d
 }  // namespace srt
