@@ -684,10 +684,12 @@ int mfma_select(const GemmProblem& p) {
   // in one round; a batch whenever whole tiles would be padding or the k loop is short (8 x 128 x 4096 x
   // 1024: 21 us against 28 us; 8 x 512 x 2048 x 256: 10.5 against 14.0; but 16 x 256 x 2048 x 2048: 81 us
   // against 51 us for whole tiles).
-  const int m_rest = p.M % 256;
   // (from 72 half tiles in one round: 1536 x 1536 x 1024 x . W^T, 72 of them: 14.8 us against 16.8 for 64 x 64 tiles;
   // 1024 x 2048 x 2048, 64 of them: 25.7 against 22.9)
-  const bool half_nt = p.batch == 1 ? (th >= 72 && rounds_h == 1) : ((m_rest > 0 && m_rest <= 128) || p.K <= 512);
+  // (a batch goes by the same count: 64 x 256 x 256 x 1024, 128 half tiles: 20.4 us against 31.9 for 64 x 64 tiles; 16 x 128 x
+  // 128 x 1024, 16 of them: 14.2 against 12.0; 64 x 256 x 1024 x 256, 512 of them: 27.4 against 18.4 for whole tiles;
+  // with 64 rows or fewer half of a half tile is padding: 64 x 64 x 512 x 256 9.3 against 8.2)
+  const bool half_nt = th >= 72 && rounds_h == 1 && p.M > 64;
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
@@ -702,11 +704,19 @@ int mfma_select(const GemmProblem& p) {
   // short k loop and few tiles, or a k-contiguous B and under 128 rows, it is not (48 x 16384 x 768: 20.5 us
   // against 15.9 us for 64 x 64 tiles; 128 x 14336 x 128: 10.2 against 8.0; 8 x 32 x 4096 x 64: 8.6 against
   // 6.6; but 64 x 128 x 1024 x 128: 12.3 against 18.5).
+  // (an A that is not k-contiguous has no half tiles and the 64 x 64 kernel's k loop is slow on it: from K = 1024 whole
+  // tiles even when most of their rows are padding -- 64 x 128 x 128 x 1024 with A m-contiguous 22.6 us against 30.9,
+  // 64 x 64 x 512 x 1024 22.7 against 28.4)
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
+                                   ((layout & 2) == 0 && p.K >= 1024 && p.M >= 64 && p.N >= 64) ||
                                    (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
   // (with neither operand k-contiguous the 64 x 64 kernel transposes both in registers: whole tiles from 12 up,
   // 512 x 1536 x 1024: 22.7 us against 24.9)
-  const long long ring_from = layout == 3 ? 96 : layout == 0 ? (p.K >= 1024 ? 12 : 24) : (p.K >= 1024 ? 24 : 32);
+  // (x^T . W^T at K = 1024: a single matrix of 16-32 tiles is 6-10 % faster in 64 x 64 tiles -- 1024 x 2048 x 1024 20.9 us
+  // against 22.8 --, a batch, whose tiles share no operand, in whole ones from 16: 16 x 256 x 256 x 1024 21.9 against 24.3)
+  const long long ring_from = layout == 3 ? 96
+                            : layout == 0 ? (p.K >= 1024 ? 4 : p.K >= 512 ? 8 : 24)
+                            : p.K < 1024 ? 32 : layout == 1 ? (p.batch > 1 ? 16 : 40) : 24;
   //  * the 64-deep form of the 16x16x32 kernel (whole-line loads of k-contiguous operands, one barrier per 128
   //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
   //    NN 1440 -> 1505 TFLOP/s, NT 1420 -> 1531, TN 1443 -> 1501, TT 1477 -> 1538), and of the 32x32x16
@@ -720,12 +730,19 @@ int mfma_select(const GemmProblem& p) {
   // an m-contiguous A against a k-contiguous B, a short k loop and under 64 tiles: the 64 x 64 kernel (1024 x 2048
   // x 256: 9.6 us against 12.4 for whole tiles; 512 x 4096 x 512: 13.2 against 15.0; at 64 tiles whole tiles win)
   const bool small_tt = layout == 1 && p.K <= 512 && t256 < 64;
+  // two k-contiguous operands and a last row of tiles that is half padding or more: the 32x32x16 64-deep kernel loses
+  // less to the padding (64 x 384 x 384 x 4096: 130 us against 155 for the 16x16x32 one, K = 256: 14.9 against 16.9)
+  const int m_rest = p.M % 256;
+  const bool padded_nt = layout == 3 && m_rest >= 1 && m_rest <= 128 && p.M < 1024 && t256 >= 128 && p.K % 64 == 0;
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
+  else if (whole_ok && padded_nt) tile = 4;
   else if (small_tt) tile = 3;
   else if (whole_ok && deep_ok && (t256 >= 128 || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
   else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
   else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
+  // (k loops too short for the 64-deep kernel, A not k-contiguous: the 16x16x32 ring, 4 x 1024 x 1024 x 64: 9.1 us against 10.1)
+  else if (whole_ok && !deep_ok && (layout & 2) == 0 && t256 >= ring_from && mfma_config(p, 5) != 0) tile = 5;
   else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout & 2) == 0))) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
@@ -867,13 +884,26 @@ bool mfma_prefers_tail(const GemmProblem& p) {
     // 32.5 us against 37.7 for split-K; 1536 x 4096 x 2048, 96 tiles: 34.4 against 40.1 whole)
     return (layout & 2) == 0 && t256 >= (p.M >= 512 ? 48 : 64) && t256 <= 128;
   }
+  // a batch has no split-K pass: with few tiles this is its only way of cutting k (4 x 256 x 256 x 4096: 40 us against
+  // 44 in half tiles, 70 whole with an A that is not k-contiguous; 16 x 64 x 512 x 4096, 32 tiles: 40-42 against 46-70)
+  // tiles that are mostly padding rows, both operands k-contiguous: 64 x 64 x 512 x 4096, 128 tiles, 95 us against 77
+  // for 64 x 64 tiles; 4 x 128 x 128 x 4096 39 against 32
+  if (p.M <= 128 && layout == 3) return false;
+  if (p.batch > 1 && t256 < 48) return true;
+  if (p.M <= 128) return false;   // (64 x 64 x 512 x 4096 with A m-contiguous, 128 tiles: 92 us against 81-82 whole)
+  // a last row of tiles that is half padding or more, and half tiles that fit one round (16 x 384 x 384 x 4096: 56 us
+  // against 51 in half tiles)
+  const int m_rest = p.M % 256;
+  if ((layout & 2) != 0 && m_rest >= 1 && m_rest <= 128 && th <= cus) return false;
   if (t256 >= cus) {
     // a handful left over (see above), or one round and up to half of another with a k loop long enough to
     // carry the adding up (3072 x 8192 x 8192, 384 tiles: 275 us against 298)
     return left > 0 && (8 * left <= cus || (t256 < 2 * cus && 2 * left <= cus && p.K >= 8192));
   }
   if (left < 48 || left > 160) return false;
-  if (left < 64 && p.M < 512) return false;  // (the 48-tile figures are of 2-6 rows of tiles; one row stays with split-K)
+  // (the 48-tile figures are of 2-6 rows of tiles, one row stays with split-K; so does K = 8192, which four parts cut
+  // deeper: 512 x 6144 x 8192 with A m-contiguous 58 us against 62)
+  if (left < 64 && (p.M < 512 || (p.K > 4096 && p.batch == 1))) return false;
   if (left <= 96) return true;
   return layout == 3 || (layout & 2) == 0 || p.K >= 8192 || th > cus;
 }
