@@ -303,6 +303,25 @@ def test_tail_sharing_batched_clipped_and_repeatable(tmp_path):
     assert tail.max() == 0.75 and tail.min() == 0.0
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_few_tile_batches_with_long_k_share_their_tiles(ta, tb):
+    """A batch has no split-K pass; the heuristic cuts its few tiles along k with the tail-sharing kernel.
+    Every tile of the launch is a shared one here (three parts each), the batches have their own operands,
+    and the tiles have ragged edges: integer operands, bit-exact in every layout, unpinned."""
+    srt.PlanCache.clear()
+    r = H.rng(515)
+    for (B_, M, N, K, dt) in [(4, 256, 256, 4096, H.BF16), (5, 200, 520, 4096, H.F16), (16, 136, 144, 8192, H.BF16)]:
+        a = r.integers(-2, 3, (B_, K, M) if ta else (B_, M, K)).astype(np.float32)
+        w = r.integers(-2, 3, (B_, N, K) if tb else (B_, K, N)).astype(np.float32)
+        at, wt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(w, dt))
+        out = srt.matmul(at, wt, ta, tb)
+        assert query_kernel(at, ta, wt, tb, out) == TAIL, (B_, M, N, K)
+        am = np.swapaxes(a, 1, 2) if ta else a
+        wm = np.swapaxes(w, 1, 2) if tb else w
+        exact = np.einsum("bmk,bkn->bmn", am.astype(np.int64), wm.astype(np.int64))
+        assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt)), (B_, M, N, K)
+
+
 def test_tail_sharing_every_way_of_cutting(tmp_path):
     """Left-over counts that reach every branch of the cutting rule -- three parts, two parts, one short part
     taken two, three and four at a time, counts that are not multiples of 8, a single left-over tile, with and
