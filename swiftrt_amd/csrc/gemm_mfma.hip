@@ -689,7 +689,9 @@ int mfma_select(const GemmProblem& p) {
   // (a batch goes by the same count: 64 x 256 x 256 x 1024, 128 half tiles: 20.4 us against 31.9 for 64 x 64 tiles; 16 x 128 x
   // 128 x 1024, 16 of them: 14.2 against 12.0; 64 x 256 x 1024 x 256, 512 of them: 27.4 against 18.4 for whole tiles;
   // with 64 rows or fewer half of a half tile is padding: 64 x 64 x 512 x 256 9.3 against 8.2)
-  const bool half_nt = th >= 72 && rounds_h == 1 && p.M > 64;
+  // (a batch of 128 whole tiles or more stays whole: its tiles share no operand, and the half tile's lower arithmetic
+  // intensity shows -- 16 x 640 x 640 x 8192: 264 us against 169-174)
+  const bool half_nt = th >= 72 && rounds_h == 1 && p.M > 64 && (p.batch == 1 || t256 < 128);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
@@ -708,7 +710,7 @@ int mfma_select(const GemmProblem& p) {
   // tiles even when most of their rows are padding -- 64 x 128 x 128 x 1024 with A m-contiguous 22.6 us against 30.9,
   // 64 x 64 x 512 x 1024 22.7 against 28.4)
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
-                                   ((layout & 2) == 0 && p.K >= 1024 && p.M >= 64 && p.N >= 64) ||
+                                   ((layout & 2) == 0 && p.K >= (p.batch > 1 ? 512 : 1024) && p.M >= 64 && p.N >= 64) ||
                                    (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
   // (with neither operand k-contiguous the 64 x 64 kernel transposes both in registers: whole tiles from 12 up,
   // 512 x 1536 x 1024: 22.7 us against 24.9)
@@ -729,7 +731,9 @@ int mfma_select(const GemmProblem& p) {
   const bool deep_ok = p.K % 64 == 0 && p.K >= 256;
   // an m-contiguous A against a k-contiguous B, a short k loop and under 64 tiles: the 64 x 64 kernel (1024 x 2048
   // x 256: 9.6 us against 12.4 for whole tiles; 512 x 4096 x 512: 13.2 against 15.0; at 64 tiles whole tiles win)
-  const bool small_tt = layout == 1 && p.K <= 512 && t256 < 64;
+  // (a single matrix: the tiles of a batch share no operand and whole tiles win there -- 48 x 256 x 256 x 512: 14.7 us
+  // against 19.4)
+  const bool small_tt = layout == 1 && p.K <= 512 && t256 < 64 && p.batch == 1;
   // two k-contiguous operands and a last row of tiles that is half padding or more: the 32x32x16 64-deep kernel loses
   // less to the padding (64 x 384 x 384 x 4096: 130 us against 155 for the 16x16x32 one, K = 256: 14.9 against 16.9)
   const int m_rest = p.M % 256;
@@ -879,18 +883,22 @@ bool mfma_prefers_tail(const GemmProblem& p) {
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
   const long long left = t256 % cus;
+  // A batch has no split-K pass: under a quarter of a round of tiles this is its only way of cutting k.  From K = 2048
+  // when A is not k-contiguous (16 x 256 x 256 x 2048: 29-30 us against 37-39 whole), from 4096 otherwise (4 x 256 x 256 x
+  // 4096: 40 us against 44 in half tiles; 48 x 256 x 256 x 8192: 96 against 165), from 8192 for x . W^T of 128 rows or
+  // fewer, which the 64 x 64 tiles do well (4 x 128 x 128 x 4096: 39 against 32; 16 x 128 x 128 x 8192: 58 against 72).
+  if (p.batch > 1 && t256 < 64) {
+    const int from = (layout & 2) == 0 ? 2048 : (layout == 3 && p.M <= 128) ? 8192 : 4096;
+    return p.K >= from;
+  }
   if (p.K < 4096) {
     // an A that is not k-contiguous has no half tiles to fall back on: from K = 2048 (1024 x 4096 x 2048, 64 tiles:
     // 32.5 us against 37.7 for split-K; 1536 x 4096 x 2048, 96 tiles: 34.4 against 40.1 whole)
     return (layout & 2) == 0 && t256 >= (p.M >= 512 ? 48 : 64) && t256 <= 128;
   }
-  // a batch has no split-K pass: with few tiles this is its only way of cutting k (4 x 256 x 256 x 4096: 40 us against
-  // 44 in half tiles, 70 whole with an A that is not k-contiguous; 16 x 64 x 512 x 4096, 32 tiles: 40-42 against 46-70)
-  // tiles that are mostly padding rows, both operands k-contiguous: 64 x 64 x 512 x 4096, 128 tiles, 95 us against 77
-  // for 64 x 64 tiles; 4 x 128 x 128 x 4096 39 against 32
-  if (p.M <= 128 && layout == 3) return false;
-  if (p.batch > 1 && t256 < 48) return true;
-  if (p.M <= 128) return false;   // (64 x 64 x 512 x 4096 with A m-contiguous, 128 tiles: 92 us against 81-82 whole)
+  // tiles that are mostly padding rows: 64 x 64 x 512 x 4096, 128 tiles, x . W^T 95 us against 77 for 64 x 64 tiles, with
+  // A m-contiguous 92 against 81-82 whole (but 64 x 128 x 128 x 4096 with A m-contiguous: 46 against 70 whole)
+  if (p.M <= 64 || (p.M <= 128 && layout == 3)) return false;
   // a last row of tiles that is half padding or more, and half tiles that fit one round (16 x 384 x 384 x 4096: 56 us
   // against 51 in half tiles)
   const int m_rest = p.M % 256;
