@@ -849,7 +849,9 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   // with neither operand k-contiguous even two parts of a handful of tiles pay: 512 x 512 x 1024: 20 us against 25)
   if (t256 <= 24 && parts >= 4 && p.K >= ((layout & 2) != 0 ? 3072 : 2048)) return true;
   if (layout == 0 && t256 <= 8 && p.K >= 1024) return true;
-  if (layout == 2 && t256 <= 4 && parts >= 4 && p.K >= 2048) return true;  // (512 x 512 x 2048: 21 us against 25 in half tiles)
+  // (512 x 512 x 2048: 21 us against 25 in half tiles; 192 x 2048 x 2048, 8 tiles: 22.0 against 25.1; 384 x 2048 x 2048, 16:
+  // 23.5 against 25.5; at 24 tiles the half tiles are ahead)
+  if (layout == 2 && t256 <= 16 && parts >= 4 && p.K >= 2048) return true;
   if ((layout & 2) == 0 || p.M <= 128) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;
