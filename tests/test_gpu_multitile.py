@@ -322,6 +322,34 @@ def test_few_tile_batches_with_long_k_share_their_tiles(ta, tb):
         assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt)), (B_, M, N, K)
 
 
+def test_tail_sharing_on_two_queues_at_once():
+    """Two queues launch tail-sharing matmuls of different shapes back to back without waiting for each other:
+    every launch has its own partial sums and flags (stream-ordered workspace, a launch-unique flag value), so
+    the results are the ones each queue gets alone -- bit for bit, on integer operands the exact product."""
+    srt.PlanCache.clear()
+    p = srt.HipPlatform.local()
+    q0, q1 = p.devices[1].queues[0], p.devices[1].queues[1]
+    r = H.rng(616)
+    jobs = []
+    for (q, (M, N, K)) in [(q0, (1024, 4096, 4096)), (q1, (2048, 2048, 8192))]:
+        a = r.integers(-2, 3, (M, K)).astype(np.float32)
+        w = r.integers(-2, 3, (N, K)).astype(np.float32)
+        at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+        outs = [srt.Tensor(shape=[M, N], dtype=np.uint16) for _ in range(6)]
+        assert query_kernel(at, False, wt, True, outs[0]) == TAIL, (M, N, K)
+        at.device_read(q); wt.device_read(q)
+        want = H.encode((a.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32), H.BF16)
+        jobs.append((q, at, wt, outs, want))
+    q0.wait_for_completion(); q1.wait_for_completion()
+    for i in range(6):
+        for (q, at, wt, outs, _) in jobs:
+            q.matmul(at, False, wt, True, outs[i])
+    for (q, _, _, outs, want) in jobs:
+        q.wait_for_completion()
+        for o in outs:
+            assert np.array_equal(o.array(), want)
+
+
 def test_tail_sharing_every_way_of_cutting(tmp_path):
     """Left-over counts that reach every branch of the cutting rule -- three parts, two parts, one short part
     taken two, three and four at a time, counts that are not multiples of 8, a single left-over tile, with and
