@@ -265,9 +265,13 @@ __device__ __forceinline__ void load_bias(const GemmProblem& p, int wave_m0, int
 // lane of the wave saw a NaN the staged patterns are rewritten to 0x7FFF on the way out.
 // Bias and the clamps (CLAMP 1: relu, 2: clipped relu) are applied to the copy that leaves the
 // accumulator registers, so the accumulators themselves are only read.
-template <typename T, int TM, bool HAS_BIAS, int CLAMP>
+// FLIP: the accumulator of the tile in row group i, column group j of the result is acc[j][i] (the kernel computed
+// the transposed product with the operands' roles exchanged; each 16 x 16 tile lies in the registers as it does
+// otherwise).
+template <typename T, int TM, bool HAS_BIAS, int CLAMP, bool FLIP = false>
 __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[TM][8], int wave_m0, int wave_n0,
                                            int bz, int lane, uint32_t stage, const u32x2_t (&b)[8]) {
+  static_assert(!FLIP || TM == 8, "a square block of accumulator tiles");
   constexpr int ROWS = TM == 8 ? 64 : 32;
   using S = typename T::storage;
   const bool per_row = p.bias_per_row != 0;
@@ -298,7 +302,8 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
       SRT_FENCE();
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        float a0 = acc[i][j][0], a1 = acc[i][j][1], a2 = acc[i][j][2], a3 = acc[i][j][3];
+        const f32x4_t& tile = FLIP ? acc[j][i] : acc[i][j];
+        float a0 = tile[0], a1 = tile[1], a2 = tile[2], a3 = tile[3];
 #ifdef SRT_EPILOGUE_PIN   // measurement builds: pinning the copies costs three register moves per tile
         asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
 #endif
