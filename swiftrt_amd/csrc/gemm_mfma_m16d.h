@@ -169,7 +169,9 @@ __device__ __forceinline__ void publish_accumulators(const f32x4_t (&acc)[8][8],
                    :: "a"(acc[i][j]), "v"(lane16), "s"(mine), "s"((i * 8 + j) * 1024) : "memory");
 }
 
-template <typename T, bool HAS_BIAS, int CLAMP>
+// FLIP: as m16::store_tile's -- the tile of row group i, column group j is acc[j][i], here and in what the other pieces
+// published (every piece of a launch publishes its accumulators by their register index).
+template <typename T, bool HAS_BIAS, int CLAMP, bool FLIP = false>
 __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x4_t (&acc)[8][8], int wave_m0, int wave_n0,
                                                 int bz, int lane, uint32_t stage, const u32x2_t (&b)[8], const TailStore& t) {
   constexpr int AGENT = 16;
@@ -195,7 +197,7 @@ __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x
   auto fetch_row = [&](const __amdgpu_buffer_rsrc_t& from, int i, int slot) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      slots[slot][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(from, lane16, (i * 8 + j) * 1024, AGENT));
+      slots[slot][j] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(from, lane16, (FLIP ? j * 8 + i : i * 8 + j) * 1024, AGENT));
   };
   // what has to be requested once row `done` (-1: nothing yet) has been consumed
   auto fetch_after = [&](int done) {
@@ -231,7 +233,8 @@ __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x
       float a[8][4];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        a[j][0] = acc[i][j][0]; a[j][1] = acc[i][j][1]; a[j][2] = acc[i][j][2]; a[j][3] = acc[i][j][3];
+        const f32x4_t& tile = FLIP ? acc[j][i] : acc[i][j];
+        a[j][0] = tile[0]; a[j][1] = tile[1]; a[j][2] = tile[2]; a[j][3] = tile[3];
         asm volatile("" : "+v"(a[j][0]), "+v"(a[j][1]), "+v"(a[j][2]), "+v"(a[j][3]));
       }
       if (two) {
@@ -344,7 +347,6 @@ constexpr int TAIL_MAX_PARTS = 3;
 // 8192^3: the kernel runs 2 % faster whenever its B is k-contiguous, whatever A is).
 template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false>
 __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailShare& ts) {
-  static_assert(!(FLIP && SK), "the tail-sharing form is not flipped");
   static_assert(!FLIP || (EPI != EPI_PARTIAL && EPI != EPI_TRANS), "flipped: the store_tile epilogues only");
   constexpr int TM = 8;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
@@ -770,7 +772,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
             how.own_last = mine == 2;
           }
           m16::pin_all<TM>(acc);   // (nothing read from the accumulators moves out of the loop)
-          store_tile_tail<T, HAS_BIAS, CLAMP>(p, acc, em0, en0, bz, lane_id(), stage, bias_regs, how);
+          store_tile_tail<T, HAS_BIAS, CLAMP, FLIP>(pe, acc, em0, en0, bz, lane_id(), stage, bias_regs, how);
           break;
         }
         publish_accumulators(acc, ring::make_rsrc(ts.partial + ((size_t)((place0 + mine) * 4 + wave) * 64) * 256, 65536), lane_id());
@@ -811,9 +813,9 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
   gemm_m16d_body<T, A_KC, B_KC, EPI, false, FLIP>(p, TailShare{});
 }
 
-template <typename T, bool A_KC, bool B_KC, int EPI>
+template <typename T, bool A_KC, bool B_KC, int EPI, bool FLIP = false>
 __global__ __launch_bounds__(NT) void gemm_m16d_tail_kernel(GemmProblem p, TailShare ts) {
-  gemm_m16d_body<T, A_KC, B_KC, EPI, true>(p, ts);
+  gemm_m16d_body<T, A_KC, B_KC, EPI, true, FLIP>(p, ts);
 }
 
 #undef SRT_FENCE
@@ -831,6 +833,15 @@ hipError_t launch_kernel(const GemmProblem& p, hipStream_t stream) {
   const int grid = ring::persistent_grid(tiles);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
   return launch_status(stream);
+}
+
+// The transposed product of `p` with the operands' roles exchanged and the result fields kept (see gemm_m16d_body, FLIP).
+inline GemmProblem flipped(const GemmProblem& p) {
+  GemmProblem q = p;
+  q.M = p.N; q.N = p.M;
+  q.A = p.B; q.sam = p.sbn; q.sak = p.sbk; q.sab = p.sbb;
+  q.B = p.A; q.sbk = p.sak; q.sbn = p.sam; q.sbb = p.sab;
+  return q;
 }
 
 // ---- the tail-sharing form ----------------------------------------------------------------------------
@@ -898,9 +909,9 @@ inline unsigned long long next_tail_epoch() {
   return 0x5ca1ab1e00000000ull | (++counter & 0xffffffffull);
 }
 
-template <typename T, bool A_KC, bool B_KC, int EPI>
+template <typename T, bool A_KC, bool B_KC, int EPI, bool FLIP = false>
 hipError_t launch_tail_kernel(const GemmProblem& p, hipStream_t stream) {
-  auto kernel = gemm_m16d_tail_kernel<T, A_KC, B_KC, EPI>;
+  auto kernel = gemm_m16d_tail_kernel<T, A_KC, B_KC, EPI, FLIP>;
   constexpr int lds_bytes = UNITS * UNIT;
   static std::atomic<uint32_t> configured{0};
   if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
@@ -931,22 +942,16 @@ hipError_t launch_tail(const GemmProblem& p, hipStream_t stream) {
   const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
                      p.activation == srtActivationElu;
   if (trans) return hipErrorInvalidValue;
-  if (p.activation == srtActivationClippedRelu) return launch_tail_kernel<T, A_KC, B_KC, EPI_CLIPPED>(p, stream);
+  constexpr bool FLIP = A_KC && !B_KC;   // x . W as the transposed product, as in launch()
+  constexpr bool KA = FLIP ? false : A_KC, KB = FLIP ? true : B_KC;
+  const GemmProblem q = FLIP ? flipped(p) : p;
+  if (p.activation == srtActivationClippedRelu) return launch_tail_kernel<T, KA, KB, EPI_CLIPPED, FLIP>(q, stream);
   if (p.activation == srtActivationRelu) {
-    if (p.bias) return launch_tail_kernel<T, A_KC, B_KC, EPI_BIAS_RELU>(p, stream);
-    return launch_tail_kernel<T, A_KC, B_KC, EPI_RELU>(p, stream);
+    if (p.bias) return launch_tail_kernel<T, KA, KB, EPI_BIAS_RELU, FLIP>(q, stream);
+    return launch_tail_kernel<T, KA, KB, EPI_RELU, FLIP>(q, stream);
   }
-  if (p.bias) return launch_tail_kernel<T, A_KC, B_KC, EPI_BIAS>(p, stream);
-  return launch_tail_kernel<T, A_KC, B_KC, EPI_PLAIN>(p, stream);
-}
-
-// The transposed product of `p` with the operands' roles exchanged and the result fields kept (see gemm_m16d_body, FLIP).
-inline GemmProblem flipped(const GemmProblem& p) {
-  GemmProblem q = p;
-  q.M = p.N; q.N = p.M;
-  q.A = p.B; q.sam = p.sbn; q.sak = p.sbk; q.sab = p.sbb;
-  q.B = p.A; q.sbk = p.sak; q.sbn = p.sam; q.sbb = p.sab;
-  return q;
+  if (p.bias) return launch_tail_kernel<T, KA, KB, EPI_BIAS, FLIP>(q, stream);
+  return launch_tail_kernel<T, KA, KB, EPI_PLAIN, FLIP>(q, stream);
 }
 
 template <typename T, bool A_KC, bool B_KC>
