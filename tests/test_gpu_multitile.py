@@ -226,6 +226,28 @@ def test_k64_m16_batched_column_major_and_nan(tmp_path):
 
 
 @pytest.mark.parametrize("dt", [H.BF16, H.F16])
+def test_column_major_dense_through_the_flipped_kernels(dt):
+    """Column-major operands and result: the call is computed as the transposed problem, whose A is k-contiguous and
+    whose B is n-contiguous -- the layout the 64-deep kernel and its tail-sharing form run flipped -- with the bias
+    running along the rows of what the kernel stores.  Integer operands and bias, relu, ragged edges: bit-exact."""
+    srt.PlanCache.clear()
+    r = H.rng(808)
+    relu = srt.ActivationType.relu
+    for (M, N, K, want) in [(2056, 4088, 512, DEEP), (1024, 4096, 4096, TAIL), (1032, 4088, 4096, TAIL)]:
+        a = r.integers(-2, 3, (M, K)).astype(np.float32)
+        w = r.integers(-2, 3, (K, N)).astype(np.float32)
+        bias = r.integers(-40, 41, N).astype(np.float32)
+        at = srt.Tensor(H.encode(a, dt), order=srt.Order.col)
+        wt = srt.Tensor(H.encode(w, dt), order=srt.Order.col)
+        bt = srt.Tensor(H.encode(bias, dt))
+        out = srt.Tensor(shape=[M, N], dtype=at.dtype, order=srt.Order.col)
+        assert query_kernel(at, False, wt, False, out) == want, (M, N, K)
+        srt.current_queue().matmul(at, False, wt, False, out, bias=bt, activation=relu)
+        exact = np.maximum(a.astype(np.float64) @ w.astype(np.float64) + bias, 0)   # (integers: exact in fp64)
+        assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt)), (M, N, K)
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
 def test_dense_shape_bias_relu_integer_bit_exact(dt, tmp_path):
     """The Dense configuration's shape, 4096 x 11008 x 4096 with an integer bias and relu: 688 tiles run as
     three even rounds of 232 workgroups."""
