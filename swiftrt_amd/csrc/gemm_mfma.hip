@@ -691,7 +691,12 @@ int mfma_select(const GemmProblem& p) {
   // with 64 rows or fewer half of a half tile is padding: 64 x 64 x 512 x 256 9.3 against 8.2)
   // (a batch of 128 whole tiles or more stays whole: its tiles share no operand, and the half tile's lower arithmetic
   // intensity shows -- 16 x 640 x 640 x 8192: 264 us against 169-174)
-  const bool half_nt = th >= 72 && rounds_h == 1 && p.M > 64 && (p.batch == 1 || t256 < 128);
+  // (a last row of half tiles that is mostly padding: 169 x 9824 x 504, 78 half tiles, 11.1 us against 9.8 for 64 x 64)
+  // (likewise a last column of tiles: 4488 x 320 x 6352, 72 half tiles, 74 us against 65); up to a quarter of padding is fine
+  // (664 x 7536 x 352: 10.2 us against 16.3)
+  const long long m_pad = (p.M + 127) / 128 * 128, n_pad = (p.N + 255) / 256 * 256;
+  const bool half_fill_ok = 4 * (m_pad - p.M) <= m_pad && 4 * (n_pad - p.N) <= n_pad;
+  const bool half_nt = th >= 72 && rounds_h == 1 && p.M > 64 && half_fill_ok && (p.batch == 1 || t256 < 128);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
@@ -711,13 +716,14 @@ int mfma_select(const GemmProblem& p) {
   // 64 x 64 x 512 x 1024 22.7 against 28.4)
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
                                    ((layout & 2) == 0 && p.K >= (p.batch > 1 ? 512 : 1024) && p.M >= 64 && p.N >= 64) ||
+                                   (layout == 0 && p.K >= 512) ||   // (8 x 88 x 2576, one tile: 51 us against 63; 16 x 2560 x 960: 22 against 25)
                                    (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
   // (with neither operand k-contiguous the 64 x 64 kernel transposes both in registers: whole tiles from 12 up,
   // 512 x 1536 x 1024: 22.7 us against 24.9)
   // (x^T . W^T at K = 1024: a single matrix of 16-32 tiles is 6-10 % faster in 64 x 64 tiles -- 1024 x 2048 x 1024 20.9 us
   // against 22.8 --, a batch, whose tiles share no operand, in whole ones from 16: 16 x 256 x 256 x 1024 21.9 against 24.3)
   const long long ring_from = layout == 3 ? 96
-                            : layout == 0 ? (p.K >= 1024 ? 4 : p.K >= 512 ? 8 : 24)
+                            : layout == 0 ? (p.K >= 1024 ? 1 : p.K >= 512 ? 8 : 64)   // (312 x 6136 x 80, 48 tiles: 9.9 us against 8.7)
                             : p.K < 1024 ? 32 : layout == 1 ? (p.batch > 1 ? 16 : 40) : 24;
   //  * the 64-deep form of the 16x16x32 kernel (whole-line loads of k-contiguous operands, one barrier per 128
   //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
@@ -743,8 +749,11 @@ int mfma_select(const GemmProblem& p) {
   else if (whole_ok && padded_nt) tile = 4;
   else if (small_tt) tile = 3;
   else if (whole_ok && deep_ok && (t256 >= 128 || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
+  // (two k-contiguous operands and a k extent that is not a whole number of 32-deep stages: the 16x16x32 ring loses its
+  // prefetch across tiles there, 4826 x 12408 x 7056: 833 us against 703 for the 32x32x16 64-deep kernel)
+  else if (whole_ok && layout == 3 && t256 >= 128 && p.K % 32 != 0) tile = 4;
   else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
-  else if (whole_ok && layout == 3 && t256 >= 192) tile = 4;
+  else if (whole_ok && layout == 3 && t256 >= 128) tile = 4;   // (1480 x 7920 x 128, 186 tiles: 11.8 us against 14.2 for the ring)
   // (k loops too short for the 64-deep kernel, A not k-contiguous: the 16x16x32 ring, 4 x 1024 x 1024 x 64: 9.1 us against 10.1)
   else if (whole_ok && !deep_ok && (layout & 2) == 0 && t256 >= ring_from && mfma_config(p, 5) != 0) tile = 5;
   else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout & 2) == 0))) tile = 1;
@@ -852,7 +861,11 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   // (512 x 512 x 2048: 21 us against 25 in half tiles; 192 x 2048 x 2048, 8 tiles: 22.0 against 25.1; 384 x 2048 x 2048, 16:
   // 23.5 against 25.5; at 24 tiles the half tiles are ahead)
   if (layout == 2 && t256 <= 16 && parts >= 4 && p.K >= 2048) return true;
-  if ((layout & 2) == 0 || p.M <= 128) return p.K >= 4096 || (p.K >= 2048 && parts >= 4);
+  // (two parts at K = 2048-4095 pay up to a quarter round of tiles -- 192 x 12568 x 3264 with A m-contiguous, 50 tiles: 42 us
+  // against 55 whole; 1496 x 80 x 3904: 41 against 63 -- and lose on half a device, 1024 x 8192 x 2048: 56 against 47; with
+  // 128 rows or fewer from K = 1024: 8 x 2184 x 1536 with A m-contiguous 24 us against 30, 72 x 2536 x 1408 16 against 19)
+  if ((layout & 2) == 0 || p.M <= 128)
+    return p.K >= 4096 || (p.K >= 2048 && (parts >= 4 || t256 <= 64)) || (p.M <= 128 && p.K >= 1024 && t256 <= 64);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;
   // (four parts also while half tiles would fill under 40 % of the device: 1536 x 1536 x 4096, 72 half tiles:
@@ -914,7 +927,9 @@ bool mfma_prefers_tail(const GemmProblem& p) {
   // (the 48-tile figures are of 2-6 rows of tiles, one row stays with split-K; so does K = 8192, which four parts cut
   // deeper: 512 x 6144 x 8192 with A m-contiguous 58 us against 62)
   if (left < 64 && (p.M < 512 || (p.K > 4096 && p.batch == 1))) return false;
-  if (left <= 96) return true;
+  // x . W has half tiles to fall back on: while they fit one round they are as good or better below K = 8192 from 72 tiles
+  // up (1536 x 3072 x 4096: 46-53 us in half tiles, 53 shared; 2048 x 3072 x 4096: 48-52 against 51-55)
+  if (left <= (layout == 2 ? 64 : 96)) return true;
   return layout == 3 || (layout & 2) == 0 || p.K >= 8192 || th > cus;
 }
 

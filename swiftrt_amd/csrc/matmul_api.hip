@@ -145,7 +145,14 @@ Plan heuristic_plan(const GemmProblem& p) {
   // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units
   if (srt::mfma_prefers_tail(p)) return kPlanM16DTail;
   // few 256 x 256 tiles and a long k loop: K split over the idle compute units
+  // up to 64 rows against a long k loop that split-K cannot cut, or only in two (K / 4 not a whole number of stages): one
+  // round of the streaming kernel's workgroups beats tiles that leave most of the device idle (24 x 96 x 10320: 32 us
+  // against 121 in half tiles; 64 x 144 x 8400 x . W^T: 26 against 61 in 64 x 64 tiles; 8 x 1288 x 10432: 44 against 58 in
+  // two parts)
+  const bool streams = p.K >= 2048 && srt::skinny_supported(p) && (long long)((p.N + 63) / 64) * p.batch <= 256;
+  if (streams && srt::mfma_splitk_parts(p) <= 2) return kPlanSkinny;
   if (srt::mfma_prefers_splitk(p)) return kPlanSplitK;
+  if (streams) return kPlanSkinny;
   const int c = srt::mfma_select(p);
   if (c) {
     switch (c >> 2) {
