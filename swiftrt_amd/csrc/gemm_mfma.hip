@@ -691,12 +691,20 @@ int mfma_select(const GemmProblem& p) {
   // with 64 rows or fewer half of a half tile is padding: 64 x 64 x 512 x 256 9.3 against 8.2)
   // (a batch of 128 whole tiles or more stays whole: its tiles share no operand, and the half tile's lower arithmetic
   // intensity shows -- 16 x 640 x 640 x 8192: 264 us against 169-174)
-  // (a last row of half tiles that is mostly padding: 169 x 9824 x 504, 78 half tiles, 11.1 us against 9.8 for 64 x 64)
-  // (likewise a last column of tiles: 4488 x 320 x 6352, 72 half tiles, 74 us against 65); up to a quarter of padding is fine
-  // (664 x 7536 x 352: 10.2 us against 16.3)
-  const long long m_pad = (p.M + 127) / 128 * 128, n_pad = (p.N + 255) / 256 * 256;
-  const bool half_fill_ok = 4 * (m_pad - p.M) <= m_pad && 4 * (n_pad - p.N) <= n_pad;
-  const bool half_nt = th >= 72 && rounds_h == 1 && p.M > 64 && half_fill_ok && (p.batch == 1 || t256 < 128);
+  // (a last row of half tiles that is mostly padding: 169 x 9824 x 504, 78 half tiles, 11.1 us against 9.8 for 64 x 64; up to
+  // a quarter of padding is fine: 664 x 7536 x 352 10.2 us against 16.3.  A long k loop wants more of the device: 5 x 1020 x
+  // 408 x 3368, 80 half tiles, 70 us against 44 for 64 x 64 tiles.  With 128 rows or fewer whole tiles are no alternative, and
+  // a short k loop is all stores: half tiles whatever the rounds, 45 x 72 x 2240 x 64 10.4 us against 18.3)
+  const long long m_pad = (p.M + 127) / 128 * 128;
+  const bool half_fill_ok = 4 * (m_pad - p.M) <= m_pad;
+  // (3205 x 984 x 3800, 104 half tiles: 48 us against 56; short rows with k loops from 1024: 3 x 194 x 3080 x 1672, 78 half
+  // tiles, 38 us against 25 for 64 x 64 tiles)
+  // (those two are of batches; a single matrix shares its operands between tiles and takes half tiles from 72: 397 x 7528 x
+  // 1056, 120 of them, 15 us against 21; 664 x 3208 x 8544, 78, 87 against 97)
+  const long long th_min = p.batch == 1 ? 72 : p.K >= 2048 ? 96 : (p.K >= 1024 && p.M < 512) ? 128 : 72;
+  const bool one_round = th >= th_min && rounds_h == 1 && half_fill_ok && (p.batch == 1 || t256 < 128);
+  const bool small_rows = p.M <= 128 && p.K <= 512 && th >= 72;
+  const bool half_nt = p.M > 64 && (one_round || small_rows);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
@@ -717,7 +725,9 @@ int mfma_select(const GemmProblem& p) {
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
                                    ((layout & 2) == 0 && p.K >= (p.batch > 1 ? 512 : 1024) && p.M >= 64 && p.N >= 64) ||
                                    (layout == 0 && p.K >= 512) ||   // (8 x 88 x 2576, one tile: 51 us against 63; 16 x 2560 x 960: 22 against 25)
-                                   (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 128 && p.N >= 128))));
+                                   (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 72 && p.N >= 72))));
+  // (a device's worth of tiles that are two thirds padding still beats 64 x 64 tiles: 41 x 1480 x 72 x 1248 x . W^T 37 us
+  // against 68, 21 x 1840 x 88 x 152 11 against 17; not with a handful of rows: 35 x 8 x 2024 x 1144 52 against 38)
   // (with neither operand k-contiguous the 64 x 64 kernel transposes both in registers: whole tiles from 12 up,
   // 512 x 1536 x 1024: 22.7 us against 24.9)
   // (x^T . W^T at K = 1024: a single matrix of 16-32 tiles is 6-10 % faster in 64 x 64 tiles -- 1024 x 2048 x 1024 20.9 us
@@ -743,7 +753,7 @@ int mfma_select(const GemmProblem& p) {
   // two k-contiguous operands and a last row of tiles that is half padding or more: the 32x32x16 64-deep kernel loses
   // less to the padding (64 x 384 x 384 x 4096: 130 us against 155 for the 16x16x32 one, K = 256: 14.9 against 16.9)
   const int m_rest = p.M % 256;
-  const bool padded_nt = layout == 3 && m_rest >= 1 && m_rest <= 128 && p.M < 1024 && t256 >= 128 && p.K % 64 == 0;
+  const bool padded_nt = layout == 3 && m_rest >= 1 && m_rest <= 128 && p.M < 1024 && t256 >= 128;
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
   else if (whole_ok && padded_nt) tile = 4;
@@ -756,7 +766,8 @@ int mfma_select(const GemmProblem& p) {
   else if (whole_ok && layout == 3 && t256 >= 128) tile = 4;   // (1480 x 7920 x 128, 186 tiles: 11.8 us against 14.2 for the ring)
   // (k loops too short for the 64-deep kernel, A not k-contiguous: the 16x16x32 ring, 4 x 1024 x 1024 x 64: 9.1 us against 10.1)
   else if (whole_ok && !deep_ok && (layout & 2) == 0 && t256 >= ring_from && mfma_config(p, 5) != 0) tile = 5;
-  else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout & 2) == 0))) tile = 1;
+  // (a handful of rows against a k-contiguous B: the 64 x 64 tiles, 4 x 8 x 104 x 7264 103 us against 116)
+  else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout == 0 || (layout == 1 && p.M > 64))))) tile = 1;
   else if (!big_ok && tiles(128) >= 256) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
@@ -857,7 +868,7 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   // (a k-contiguous A has half tiles: 1024 x 1536 x 2048, 24 tiles: 25.5 us in half tiles against 27.9 in four parts;
   // with neither operand k-contiguous even two parts of a handful of tiles pay: 512 x 512 x 1024: 20 us against 25)
   if (t256 <= 24 && parts >= 4 && p.K >= ((layout & 2) != 0 ? 3072 : 2048)) return true;
-  if (layout == 0 && t256 <= 8 && p.K >= 1024) return true;
+  if ((layout & 2) == 0 && t256 <= 8 && p.K >= 1024) return true;   // (1224 x 136 x 1600 with B k-contiguous: 24 us against 30)
   // (512 x 512 x 2048: 21 us against 25 in half tiles; 192 x 2048 x 2048, 8 tiles: 22.0 against 25.1; 384 x 2048 x 2048, 16:
   // 23.5 against 25.5; at 24 tiles the half tiles are ahead)
   if (layout == 2 && t256 <= 16 && parts >= 4 && p.K >= 2048) return true;
@@ -865,7 +876,9 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   // against 55 whole; 1496 x 80 x 3904: 41 against 63 -- and lose on half a device, 1024 x 8192 x 2048: 56 against 47; with
   // 128 rows or fewer from K = 1024: 8 x 2184 x 1536 with A m-contiguous 24 us against 30, 72 x 2536 x 1408 16 against 19)
   if ((layout & 2) == 0 || p.M <= 128)
-    return p.K >= 4096 || (p.K >= 2048 && (parts >= 4 || t256 <= 64)) || (p.M <= 128 && p.K >= 1024 && t256 <= 64);
+    // (few columns likewise: 4968 x 128 x 1856 with B k-contiguous, 20 tiles, 27 us in two parts against 35)
+    return p.K >= 4096 || (p.K >= 2048 && (parts >= 4 || t256 <= 96)) ||
+           ((p.M <= 128 || p.N <= 128) && p.K >= 1024 && t256 <= 64);
   if (p.K < 4096) return false;
   if (layout == 3) return parts >= 4 || p.K >= 8192;
   // (four parts also while half tiles would fill under 40 % of the device: 1536 x 1536 x 4096, 72 half tiles:

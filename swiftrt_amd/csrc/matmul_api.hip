@@ -143,6 +143,11 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 Plan heuristic_plan(const GemmProblem& p) {
   if (srt::skinny_supported(p) && srt::skinny_preferred(p)) return kPlanSkinny;
   // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units
+  // up to 32 rows against a long k loop, one round of the streaming kernel's workgroups: ahead of sharing tiles that are
+  // nearly all padding (28 x 8 x 88 x 7680: 32 us against 59)
+  if (p.M <= 32 && p.K >= 2048 && srt::skinny_supported(p) && (long long)((p.N + 63) / 64) * p.batch <= 256 &&
+      srt::mfma_splitk_parts(p) <= 2)
+    return kPlanSkinny;
   if (srt::mfma_prefers_tail(p)) return kPlanM16DTail;
   // few 256 x 256 tiles and a long k loop: K split over the idle compute units
   // up to 64 rows against a long k loop that split-K cannot cut, or only in two (K / 4 not a whole number of stages): one
