@@ -254,6 +254,35 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 8, 28672, 1024) == "mfma_128x256_m16"               # 448 workgroups: not one round
     assert query(native.REAL16BF, 64, 14336, 4096) == "skinny"
     assert query(native.REAL16BF, 64, 11008, 4096) == "mfma_256x256_splitk"
+    # what sweeps against every pinned plan found (the measured pairs stand next to the rules in csrc/gemm_mfma.hip)
+    assert query(native.REAL16BF, 24, 96, 10320) == "skinny"                          # K / 2 is not a whole number of stages: no split-K
+    assert query(native.REAL16BF, 8, 1288, 10432) == "skinny"                         # only two parts possible
+    assert query(native.REAL16BF, 8, 88, 2576, ta=True) == "mfma_256x256_m16"           # one whole tile beats 64 x 64 tiles on an m-contiguous A
+    assert query(native.REAL16BF, 4826, 12408, 7056, tb=True) == "mfma_256x256_k64"   # k extent not a whole number of 32-deep stages
+    assert query(native.REAL16BF, 192, 12568, 3264, ta=True, tb=True) == "mfma_256x256_splitk"   # two parts up to a quarter round
+    assert query(native.REAL16BF, 664, 7536, 352, tb=True) == "mfma_128x256_m16"      # 13 % padding rows are fine for half tiles
+    assert query(native.REAL16BF, 169, 9824, 504, tb=True) == "mfma_64x64"            # a second row of half tiles that is mostly padding is not
+    assert query(native.REAL16BF, 512, 512, 1024, ta=True) == "mfma_256x256_splitk"   # four tiles, neither operand k-contiguous
+    # batches (no split-K pass)
+    def query_batched(dt, B, M, N, K, ta=False, tb=False):
+        ashape = (B, K, M) if ta else (B, M, K)
+        bshape = (B, N, K) if tb else (B, K, N)
+        ad, k1 = native.make_descriptor(dt, ashape, (ashape[1] * ashape[2], ashape[2], 1), native.ORDER_ROW)
+        bd, k2 = native.make_descriptor(dt, bshape, (bshape[1] * bshape[2], bshape[2], 1), native.ORDER_ROW)
+        od, k3 = native.make_descriptor(dt, (B, M, N), (M * N, N, 1), native.ORDER_ROW)
+        buf = ctypes.create_string_buffer(64)
+        p = ctypes.c_void_p(256)
+        assert L.srtMatmulQueryKernel(ctypes.byref(ad), int(ta), ctypes.byref(bd), int(tb), ctypes.byref(od), p, p, p, buf, 64) == 0
+        return buf.value.decode()
+    assert query_batched(native.REAL16BF, 4, 256, 256, 4096, ta=True) == "mfma_256x256_m16_k64_tail"   # four tiles cut along k
+    assert query_batched(native.REAL16BF, 16, 256, 256, 2048, ta=True, tb=True) == "mfma_256x256_m16_k64_tail"
+    assert query_batched(native.REAL16BF, 4, 128, 128, 4096, tb=True) == "mfma_64x64"                  # mostly padding, both k-contiguous
+    assert query_batched(native.REAL16BF, 64, 256, 256, 1024, tb=True) == "mfma_128x256_m16"           # 128 half tiles in one round
+    assert query_batched(native.REAL16BF, 64, 256, 1024, 256, tb=True) == "mfma_256x256_m16_k64"       # 512 half tiles: whole tiles
+    assert query_batched(native.REAL16BF, 64, 384, 384, 4096, tb=True) == "mfma_256x256_k64"           # a last row of tiles half padding
+    assert query_batched(native.REAL16BF, 28, 8, 88, 7680) == "skinny"                                 # ahead of sharing padded tiles
+    assert query_batched(native.REAL16BF, 41, 1480, 72, 1248, tb=True) == "mfma_256x256_k64"           # a device's worth of padded whole tiles
+    assert query_batched(native.REAL16BF, 36, 8, 768, 328, tb=True) == "mfma_64x64"                    # 864 streaming workgroups: not worth it
     # 16-bit operands that miss the 16-byte rules: the matrix-core kernel with element-wise staging
     assert query(native.REAL16BF, 33, 33, 33) == "mfma_64x64_any"
     assert query(native.REAL16BF, 64, 64, 64, align=2) == "mfma_64x64_any"            # misaligned view
