@@ -680,10 +680,8 @@ int mfma_select(const GemmProblem& p) {
   //    operands, where the 64-deep kernel keeps short k loops (8192 x 8192 x 1024: 138 us against 146).
   // Half tiles: with 64 columns or fewer only for longer k loops and an n-contiguous B (1536 x 64 x 128:
   // 10.4 us against 6.7 us for 64 x 64 tiles, 1536 x 64 x 768: 12.8 against 15.1; 32 x 1024 x 64 x 4096
-  // with B k-contiguous: 97 against 67).  With two k-contiguous operands a single matrix takes them only
-  // in one round; a batch whenever whole tiles would be padding or the k loop is short (8 x 128 x 4096 x
-  // 1024: 21 us against 28 us; 8 x 512 x 2048 x 256: 10.5 against 14.0; but 16 x 256 x 2048 x 2048: 81 us
-  // against 51 us for whole tiles).
+  // with B k-contiguous: 97 against 67).  With two k-contiguous operands they are taken only in one round (8 x 128 x
+  // 4096 x 1024: 21 us against 28 us; 8 x 512 x 2048 x 256: 10.5 against 14.0), by the counts below.
   // (from 72 half tiles in one round: 1536 x 1536 x 1024 x . W^T, 72 of them: 14.8 us against 16.8 for 64 x 64 tiles;
   // 1024 x 2048 x 2048, 64 of them: 25.7 against 22.9)
   // (a batch goes by the same count: 64 x 256 x 256 x 1024, 128 half tiles: 20.4 us against 31.9 for 64 x 64 tiles; 16 x 128 x
