@@ -142,20 +142,18 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 
 Plan heuristic_plan(const GemmProblem& p) {
   if (srt::skinny_supported(p) && srt::skinny_preferred(p)) return kPlanSkinny;
-  // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units
-  // up to 32 rows against a long k loop, one round of the streaming kernel's workgroups: ahead of sharing tiles that are
-  // nearly all padding (28 x 8 x 88 x 7680: 32 us against 59)
-  if (p.M <= 32 && p.K >= 2048 && srt::skinny_supported(p) && (long long)((p.N + 63) / 64) * p.batch <= 256 &&
-      srt::mfma_splitk_parts(p) <= 2)
-    return kPlanSkinny;
-  if (srt::mfma_prefers_tail(p)) return kPlanM16DTail;
-  // few 256 x 256 tiles and a long k loop: K split over the idle compute units
-  // up to 64 rows against a long k loop that split-K cannot cut, or only in two (K / 4 not a whole number of stages): one
-  // round of the streaming kernel's workgroups beats tiles that leave most of the device idle (24 x 96 x 10320: 32 us
-  // against 121 in half tiles; 64 x 144 x 8400 x . W^T: 26 against 61 in 64 x 64 tiles; 8 x 1288 x 10432: 44 against 58 in
-  // two parts)
+  // Up to 64 rows against a long k loop, one round of the streaming kernel's workgroups: when split-K cannot cut the k
+  // loop, or only in two (K / 4 not a whole number of stages; a batch has no split-K pass at all), the streaming kernel beats
+  // tiles that leave most of the device idle (24 x 96 x 10320: 32 us against 121 in half tiles; 64 x 144 x 8400 x . W^T: 26
+  // against 61 in 64 x 64 tiles; 8 x 1288 x 10432: 44 against 58 in two parts).  With up to 32 rows that is decided ahead
+  // of tail sharing, whose tiles would be nearly all padding (28 x 8 x 88 x 7680: 32 us against 59).
   const bool streams = p.K >= 2048 && srt::skinny_supported(p) && (long long)((p.N + 63) / 64) * p.batch <= 256;
-  if (streams && srt::mfma_splitk_parts(p) <= 2) return kPlanSkinny;
+  const bool few_parts = srt::mfma_splitk_parts(p) <= 2;
+  if (streams && few_parts && p.M <= 32) return kPlanSkinny;
+  // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units
+  if (srt::mfma_prefers_tail(p)) return kPlanM16DTail;
+  if (streams && few_parts) return kPlanSkinny;
+  // few 256 x 256 tiles and a long k loop: K split over the idle compute units
   if (srt::mfma_prefers_splitk(p)) return kPlanSplitK;
   if (streams) return kPlanSkinny;
   const int c = srt::mfma_select(p);
