@@ -94,6 +94,21 @@ def test_vector_path_special_values_bit_exact(dt):
     assert same(dx.array(), ora.elementwise("mul", b_st, H.encode(np.ones(shape, np.float32), dt)))
 
 
+def test_every_float_converts_to_bfloat16_as_the_reference_codec_does():
+    """All 2^32 fp32 bit patterns through the device's fp32 -> bfloat16 copy (the 16-byte path: hardware converter for
+    vectors without a NaN, the scalar encoder for the others) against the oracle's restatement of BFloat16.init
+    (platform/common/BFloat16.swift:53-80), in 16 slabs of 2^28."""
+    q = srt.current_queue()
+    n = 1 << 28
+    out = srt.Tensor(shape=[n // 4096, 4096], dtype=np.uint16)
+    for slab in range(16):
+        bits = np.arange(slab * n, (slab + 1) * n, dtype=np.uint64).astype(np.uint32)
+        x = bits.view(np.float32).reshape(n // 4096, 4096)
+        q.copy(srt.Tensor(x), out)
+        want = ora.encode(x, H.BF16)
+        assert np.array_equal(out.array(), want), slab
+
+
 @pytest.mark.parametrize("dt", DTS)
 def test_binary_odd_sizes_and_misaligned_views(dt):
     """Extents that are not a multiple of the vector width and views that start off a 16-byte
