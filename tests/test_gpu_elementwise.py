@@ -109,6 +109,30 @@ def test_every_float_converts_to_bfloat16_as_the_reference_codec_does():
         assert np.array_equal(out.array(), want), slab
 
 
+def test_floats_convert_to_float16_as_ieee_does():
+    """fp32 -> fp16 copy on the device against numpy's binary16 (round to nearest even, subnormals kept, overflow to
+    infinity): every combination of sign, exponent and upper mantissa bits with the thirteen dropped bits at and next to
+    the tie (0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF), the same around the ten further bits a subnormal result drops, and
+    2^24 random patterns.  NaNs are compared as NaNs (their payloads are not part of the contract)."""
+    q = srt.current_queue()
+    upper = np.arange(1 << 19, dtype=np.uint32) << 13
+    lows = np.array([0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF], np.uint32)
+    bits = (upper[:, None] | lows[None, :]).reshape(-1)
+    sub = (np.arange(1 << 9, dtype=np.uint32) << 23)[:, None] | np.array(
+        [0x7FFFFF, 0x400000, 0x400001, 0x3FFFFF, 0x200000, 0x600000, 0x100000, 0x300000], np.uint32)[None, :]
+    bits = np.concatenate([bits, sub.reshape(-1), H.rng(5).integers(0, 1 << 32, 1 << 24, dtype=np.uint64).astype(np.uint32)])
+    bits = bits[: bits.size // 4096 * 4096]
+    x = bits.view(np.float32).reshape(-1, 4096)
+    out = srt.Tensor(shape=list(x.shape), dtype=np.float16)
+    q.copy(srt.Tensor(x), out)
+    with np.errstate(all="ignore"):
+        want = x.astype(np.float16)
+    got = out.array()
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint16)[~nan], want.view(np.uint16)[~nan])
+
+
 @pytest.mark.parametrize("dt", DTS)
 def test_binary_odd_sizes_and_misaligned_views(dt):
     """Extents that are not a multiple of the vector width and views that start off a 16-byte
