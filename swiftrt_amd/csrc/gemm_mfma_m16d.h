@@ -942,16 +942,29 @@ hipError_t launch_tail(const GemmProblem& p, hipStream_t stream) {
   const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
                      p.activation == srtActivationElu;
   if (trans) return hipErrorInvalidValue;
-  constexpr bool FLIP = A_KC && !B_KC;   // x . W as the transposed product, as in launch()
-  constexpr bool KA = FLIP ? false : A_KC, KB = FLIP ? true : B_KC;
-  const GemmProblem q = FLIP ? flipped(p) : p;
-  if (p.activation == srtActivationClippedRelu) return launch_tail_kernel<T, KA, KB, EPI_CLIPPED, FLIP>(q, stream);
-  if (p.activation == srtActivationRelu) {
-    if (p.bias) return launch_tail_kernel<T, KA, KB, EPI_BIAS_RELU, FLIP>(q, stream);
-    return launch_tail_kernel<T, KA, KB, EPI_RELU, FLIP>(q, stream);
+  // x . W as the transposed product, as in launch() -- from 96 tiles up: on a device a quarter full the flipped walk costs
+  // more than the cheaper fragment reads give (1024 x 4096 x 4096, 64 tiles: 44.7 us against 44.1; 1536 x 4096 x 11008, 96
+  // tiles: 112 against 115)
+  if constexpr (A_KC && !B_KC) {
+    const long long tiles = (long long)((p.M + 255) / 256) * ((p.N + BN - 1) / BN) * p.batch;
+    if (tiles >= 96) {
+      const GemmProblem q = flipped(p);
+      if (p.activation == srtActivationClippedRelu) return launch_tail_kernel<T, false, true, EPI_CLIPPED, true>(q, stream);
+      if (p.activation == srtActivationRelu) {
+        if (p.bias) return launch_tail_kernel<T, false, true, EPI_BIAS_RELU, true>(q, stream);
+        return launch_tail_kernel<T, false, true, EPI_RELU, true>(q, stream);
+      }
+      if (p.bias) return launch_tail_kernel<T, false, true, EPI_BIAS, true>(q, stream);
+      return launch_tail_kernel<T, false, true, EPI_PLAIN, true>(q, stream);
+    }
   }
-  if (p.bias) return launch_tail_kernel<T, KA, KB, EPI_BIAS, FLIP>(q, stream);
-  return launch_tail_kernel<T, KA, KB, EPI_PLAIN, FLIP>(q, stream);
+  if (p.activation == srtActivationClippedRelu) return launch_tail_kernel<T, A_KC, B_KC, EPI_CLIPPED>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_tail_kernel<T, A_KC, B_KC, EPI_BIAS_RELU>(p, stream);
+    return launch_tail_kernel<T, A_KC, B_KC, EPI_RELU>(p, stream);
+  }
+  if (p.bias) return launch_tail_kernel<T, A_KC, B_KC, EPI_BIAS>(p, stream);
+  return launch_tail_kernel<T, A_KC, B_KC, EPI_PLAIN>(p, stream);
 }
 
 template <typename T, bool A_KC, bool B_KC>
