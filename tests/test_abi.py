@@ -298,6 +298,52 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 8, 65664, 32768, tb=True) == "skinny/pieces"
 
 
+def test_kernel_selection_answers_for_any_problem():
+    """Random shapes, types, layouts, pitches, batches and alignments (zero extents included): the selection logic
+    answers every one with success and a known plan name.  (Run against the host-sanitizer build of the library, this is
+    also the fuzz of its arithmetic: `make -C swiftrt_amd/csrc SANITIZE=1`, SWIFTRT_HIP_LIBRARY.)"""
+    L = native.lib()
+    g = np.random.default_rng(123)
+    buf = ctypes.create_string_buffer(64)
+    known = {"empty", "generic", "skinny", "f32_mfma", "mfma_256x256", "mfma_128x128", "mfma_64x64", "mfma_256x256_k64",
+             "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128_any", "mfma_64x64_any",
+             "mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail"}
+
+    def logu(lo, hi):
+        return int(np.exp(g.uniform(np.log(lo), np.log(hi))))
+
+    seen = set()
+    for _ in range(4000):
+        dt = [native.REAL16BF, native.REAL16F, native.REAL32F][int(g.integers(0, 3))]
+        batch = 1 if g.random() < 0.7 else logu(1, 300)
+        M, N, K = logu(1, 20000), logu(1, 40000), logu(1, 40000)
+        if g.random() < 0.6:
+            M, N, K = max(8, M // 8 * 8), max(8, N // 8 * 8), max(8, K // 8 * 8)
+        if g.random() < 0.02:
+            M = 0
+        if g.random() < 0.02:
+            K = 0
+        ta, tb = int(g.integers(0, 2)), int(g.integers(0, 2))
+        pa, pb, pc = [int(g.integers(0, 3)) * 8 if g.random() < 0.2 else 0 for _ in range(3)]
+        ash = (K, M) if ta else (M, K)
+        bsh = (N, K) if tb else (K, N)
+        if batch > 1:
+            ad = native.make_descriptor(dt, (batch,) + ash, (ash[0] * (ash[1] + pa), ash[1] + pa, 1), native.ORDER_ROW)
+            bd = native.make_descriptor(dt, (batch,) + bsh, (bsh[0] * (bsh[1] + pb), bsh[1] + pb, 1), native.ORDER_ROW)
+            od = native.make_descriptor(dt, (batch, M, N), (M * (N + pc), N + pc, 1), native.ORDER_ROW)
+        else:
+            ad = native.make_descriptor(dt, ash, (ash[1] + pa, 1), native.ORDER_ROW)
+            bd = native.make_descriptor(dt, bsh, (bsh[1] + pb, 1), native.ORDER_ROW)
+            od = native.make_descriptor(dt, (M, N), (N + pc, 1), native.ORDER_ROW)
+        p = ctypes.c_void_p(256 if g.random() < 0.9 else int(g.integers(1, 16)) * 2)
+        st = L.srtMatmulQueryKernel(ctypes.byref(ad[0]), ta, ctypes.byref(bd[0]), tb, ctypes.byref(od[0]), p, p, p, buf, 64)
+        assert st == 0, (dt, batch, M, N, K, ta, tb)
+        name = buf.value.decode()
+        assert name.split("/")[0] in known and name.split("/")[-1] in known | {"pieces"}, name
+        seen.add(name.split("/")[0])
+    assert {"skinny", "mfma_64x64", "mfma_256x256_m16", "mfma_128x256_m16", "f32_mfma"} <= seen
+
+
 def test_tensor_layout_and_views():
     t = srt.Tensor(np.arange(12, dtype=np.float32).reshape(3, 4))
     assert t.shape == (3, 4) and t.strides == (4, 1)
