@@ -195,9 +195,12 @@ srtStatus srtMemsetAsync(void* dst, int32_t value, size_t byteCount, srtStream s
  * (Sources/SwiftRTCore/platform/cpu/functions/CpuMath.swift:1141-1161, :1164-1186).
  * Elements: srtReal32F, srtReal16F, srtReal16BF, all three tensors the same type.  Products
  * are accumulated in fp32 and rounded once (nearest even) to the element type.
- * Operands may be any strided view; `out` may have any strides, but the span of storage it covers
- * (first to last element) must not overlap the span of `a`, `b` or the bias: srtErrorInvalidValue
- * otherwise (tiles are stored while other tiles are still being read).
+ * Operands may be any strided view; `out` may have any strides, but must share no element with `a`, `b`
+ * or the bias (tiles are stored while other tiles are still being read).  Views whose storage spans
+ * (first to last element) do not overlap are accepted, and so are overlapping spans that a common pitch
+ * proves apart: column slices of one wide row-major buffer, interleaved batches.  `out` starting on an
+ * input's first element, or overlapping an input as row blocks of one pitch, is srtErrorInvalidValue; spans that overlap in a way the check cannot resolve are
+ * srtErrorNotSupported (the caller's fallback runs).
  *
  * Returns srtErrorNotSupported (caller falls back to the CPU) for other element types,
  * orders other than row/col, or rank other than 2/3; srtErrorInvalidValue when extents do not
@@ -301,7 +304,11 @@ srtStatus srtActivationBackwardBias(const void* y, const srtTensorDescriptor* yD
  * nothing.  Limit: with a bias gradient, N <= 2 097 152 columns (one fp32 partial row must fit the 8 MiB);
  * srtErrorInvalidValue beyond that.  Every call on a GPU shares that GPU's array:
  * calls that overlap in time on one GPU (different streams, or different threads) race; serialise them.
- * The array needs no clearing between calls (every entry read is written first by the same call). */
+ * The array needs no clearing between calls (every entry read is written first by the same call).
+ * The array used is that of the device `stream` belongs to (the current device for the null stream).  Its
+ * address is looked up once per device: by srtStreamCreate for the device current at that time, otherwise by
+ * the first call on that device -- a lookup is a runtime query, not a launch, so with a stream made elsewhere
+ * make one call per device before capturing calls into a graph. */
 srtStatus srtActivationBackwardBiasNoAlloc(const void* y, const srtTensorDescriptor* yDesc,
                                            const void* dy, const srtTensorDescriptor* dyDesc,
                                            srtActivation activation, double coef,

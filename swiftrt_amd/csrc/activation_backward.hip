@@ -175,26 +175,45 @@ __global__ __launch_bounds__(64 * kFinishWaves) void bias_gradient_finish_kernel
 constexpr size_t kScratchBytes = 8u << 20;
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
 
-// The current device's address of `scratch` (cached per device), or null with *status set.
-float* scratch_of_current_device(srtStatus* status) {
-  static std::atomic<void*> cached[64];
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) {
+// Device `device`'s address of `scratch`, resolved once per device with that device current and cached.
+// srtStreamCreate resolves it for its stream's device (prepare_backward_scratch), so a call on a stream this
+// library created finds it cached; for a stream made elsewhere the first call per device resolves it here.
+std::atomic<void*> scratch_address[64];
+
+float* scratch_of_device(int device, srtStatus* status) {
+  if (device < 0 || device >= 64) {
     *status = srtErrorNoDevice;
     return nullptr;
   }
-  void* ptr = cached[device].load(std::memory_order_acquire);
+  void* ptr = scratch_address[device].load(std::memory_order_acquire);
   if (ptr == nullptr) {
-    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    int current = -1;
+    hipError_t e = hipGetDevice(&current);
+    const bool other = e == hipSuccess && current != device;
+    if (other) e = hipSetDevice(device);
+    if (e == hipSuccess) e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (other) (void)hipSetDevice(current);
     if (e != hipSuccess || ptr == nullptr) {
       (void)hipGetLastError();
       *status = e == hipSuccess ? srtErrorUnknown : from_hip(e);
       return nullptr;
     }
-    cached[device].store(ptr, std::memory_order_release);
+    scratch_address[device].store(ptr, std::memory_order_release);
   }
   *status = srtSuccess;
   return static_cast<float*>(ptr);
+}
+
+// The array of the device `stream` belongs to (the null stream: the current device).
+float* scratch_of_stream(hipStream_t stream, srtStatus* status) {
+  int device = -1;
+  const hipError_t e = stream ? hipStreamGetDevice(stream, &device) : hipGetDevice(&device);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *status = from_hip(e);
+    return nullptr;
+  }
+  return scratch_of_device(device, status);
 }
 
 // fixed_workspace: false -- the partial rows come from the library's stream-ordered allocator;
@@ -229,7 +248,7 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
   if (dbias && fixed_workspace) {
     if ((size_t)chunks * p.N * sizeof(float) > kScratchBytes) return srtErrorInvalidValue;
     srtStatus s;
-    workspace = scratch_of_current_device(&s);
+    workspace = scratch_of_stream(stream, &s);
     if (!workspace) return s;
     // every entry the second kernel reads is written by the first (all chunks, all N columns), so the
     // previous call's contents need no clearing
@@ -254,6 +273,15 @@ srtStatus run(BackwardProblem p, void* dbias, long long dbias_stride, hipStream_
 }
 
 }  // namespace
+
+// Set-up hook of the runtime (srtStreamCreate): resolves the current device's scratch address ahead of the first
+// srtActivationBackwardBiasNoAlloc, whose calls then touch no runtime state beyond their launches.
+void prepare_backward_scratch() {
+  int device = -1;
+  srtStatus ignored;
+  if (hipGetDevice(&device) == hipSuccess) (void)scratch_of_device(device, &ignored);
+  else (void)hipGetLastError();
+}
 }  // namespace srt
 
 static srtStatus activation_backward_bias(const void* y, const srtTensorDescriptor* yDesc, const void* dy,

@@ -625,8 +625,11 @@ int mfma_config(const GemmProblem& p, int tile) {
 int mfma_select(const GemmProblem& p) {
   const int layout = mfma_layout(p);
   auto tiles = [&](int t) { return (long long)((p.M + t - 1) / t) * ((p.N + t - 1) / t) * p.batch; };
+  // the device's compute units and half of them: "a device's worth" and "half a device's worth" of tiles below (the
+  // other tile counts in the rules are measured cross-over points on a 256-unit device)
+  const long long cus = compute_units(), half_cus = cus / 2;
   // operands that miss the alignment rules: unaligned or element-wise staging, 128 x 128 tiles once they fill the device
-  if (layout < 0) return mfma_config(p, tiles(128) >= 256 ? 7 : 8);
+  if (layout < 0) return mfma_config(p, tiles(128) >= cus ? 7 : 8);
   // Tile choice, from measurements over mid-size problems (1024^3 .. 4096 x 14336 x 4096):
   //  * the 256 x 256 kernels are so much more efficient per tile (deep prefetch, 4x the arithmetic
   //    intensity) that they win long before they can fill the device: from 24 tiles up (48 when K < 1024) for the
@@ -663,7 +666,6 @@ int mfma_select(const GemmProblem& p) {
   //    when it fits in one round (1536 x 11008 x 4096 NT: 190 us against 168 us whole), and the
   //    64 x 64 kernel is as good up to about 96 half tiles (1024 x 1024 x 2048: 20 us against 23 us).
   const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
-  const long long cus = 256;
   const long long rounds256 = (t256 + cus - 1) / cus, rounds_h = (th + cus - 1) / cus;
   //  * a problem of a handful of tiles is bound by the latency of its k stages, and the ring's
   //    deep prefetch beats the 64 x 64 kernel's load-wait-compute stages even on one or two
@@ -700,7 +702,7 @@ int mfma_select(const GemmProblem& p) {
   // (those two are of batches; a single matrix shares its operands between tiles and takes half tiles from 72: 397 x 7528 x
   // 1056, 120 of them, 15 us against 21; 664 x 3208 x 8544, 78, 87 against 97)
   const long long th_min = p.batch == 1 ? 72 : p.K >= 2048 ? 96 : (p.K >= 1024 && p.M < 512) ? 128 : 72;
-  const bool one_round = th >= th_min && rounds_h == 1 && half_fill_ok && (p.batch == 1 || t256 < 128);
+  const bool one_round = th >= th_min && rounds_h == 1 && half_fill_ok && (p.batch == 1 || t256 < half_cus);
   const bool small_rows = p.M <= 128 && p.K <= 512 && th >= 72;
   const bool half_nt = p.M > 64 && (one_round || small_rows);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
@@ -723,7 +725,7 @@ int mfma_select(const GemmProblem& p) {
   const bool whole_ok = big_ok && ((p.M > 128 && p.N > 128) || p.K >= 4096 ||
                                    ((layout & 2) == 0 && p.K >= (p.batch > 1 ? 512 : 1024) && p.M >= 64 && p.N >= 64) ||
                                    (layout == 0 && p.K >= 512) ||   // (8 x 88 x 2576, one tile: 51 us against 63; 16 x 2560 x 960: 22 against 25)
-                                   (t256 >= 128 && (layout == 0 || p.K >= 2048 || (p.M >= 72 && p.N >= 72))));
+                                   (t256 >= half_cus && (layout == 0 || p.K >= 2048 || (p.M >= 72 && p.N >= 72))));
   // (a device's worth of tiles that are two thirds padding still beats 64 x 64 tiles: 41 x 1480 x 72 x 1248 x . W^T 37 us
   // against 68, 21 x 1840 x 88 x 152 11 against 17; not with a handful of rows: 35 x 8 x 2024 x 1144 52 against 38)
   // (with neither operand k-contiguous the 64 x 64 kernel transposes both in registers: whole tiles from 12 up,
@@ -751,22 +753,22 @@ int mfma_select(const GemmProblem& p) {
   // two k-contiguous operands and a last row of tiles that is half padding or more: the 32x32x16 64-deep kernel loses
   // less to the padding (64 x 384 x 384 x 4096: 130 us against 155 for the 16x16x32 one, K = 256: 14.9 against 16.9)
   const int m_rest = p.M % 256;
-  const bool padded_nt = layout == 3 && m_rest >= 1 && m_rest <= 128 && p.M < 1024 && t256 >= 128;
+  const bool padded_nt = layout == 3 && m_rest >= 1 && m_rest <= 128 && p.M < 1024 && t256 >= half_cus;
   int tile;
   if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
   else if (whole_ok && padded_nt) tile = 4;
   else if (small_tt) tile = 3;
-  else if (whole_ok && deep_ok && (t256 >= 128 || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
+  else if (whole_ok && deep_ok && (t256 >= half_cus || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
   // (two k-contiguous operands and a k extent that is not a whole number of 32-deep stages: the 16x16x32 ring loses its
   // prefetch across tiles there, 4826 x 12408 x 7056: 833 us against 703 for the 32x32x16 64-deep kernel)
-  else if (whole_ok && layout == 3 && t256 >= 128 && p.K % 32 != 0) tile = 4;
-  else if (whole_ok && t256 >= 128 && (layout != 3 || p.K >= 2048)) tile = 5;
-  else if (whole_ok && layout == 3 && t256 >= 128) tile = 4;   // (1480 x 7920 x 128, 186 tiles: 11.8 us against 14.2 for the ring)
+  else if (whole_ok && layout == 3 && t256 >= half_cus && p.K % 32 != 0) tile = 4;
+  else if (whole_ok && t256 >= half_cus && (layout != 3 || p.K >= 2048)) tile = 5;
+  else if (whole_ok && layout == 3 && t256 >= half_cus) tile = 4;   // (1480 x 7920 x 128, 186 tiles: 11.8 us against 14.2 for the ring)
   // (k loops too short for the 64-deep kernel, A not k-contiguous: the 16x16x32 ring, 4 x 1024 x 1024 x 64: 9.1 us against 10.1)
   else if (whole_ok && !deep_ok && (layout & 2) == 0 && t256 >= ring_from && mfma_config(p, 5) != 0) tile = 5;
   // (a handful of rows against a k-contiguous B: the 64 x 64 tiles, 4 x 8 x 104 x 7264 103 us against 116)
   else if (whole_ok && (t256 >= ring_from || (p.K >= 4096 && (layout == 0 || (layout == 1 && p.M > 64))))) tile = 1;
-  else if (!big_ok && tiles(128) >= 256) tile = 2;
+  else if (!big_ok && tiles(128) >= cus) tile = 2;
   else tile = 3;
   return (tile << 2) | layout;
 }
@@ -832,7 +834,7 @@ int mfma_splitk_parts(const GemmProblem& p) {
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256);   // also the count of half tiles then
   int parts = 0;
   for (int s = 2; s <= 16; s *= 2) {
-    if (t256 * s > 256) break;
+    if (t256 * s > compute_units()) break;
     if (p.K % (s * 32) != 0 || p.K / s < 512) break;
     parts = s;
   }

@@ -63,16 +63,6 @@ constexpr int EPI_PARTIAL = 6;   // fp32 accumulators as they are, for a split-K
 
 #define SRT_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-// Measurement builds only (the probe ablate_m16.hip; the library is built without it): parts of the main
-// loop can be taken out to see what each costs in time and, under the power limit, in clock.  The MFMA
-// stream stays as it is; results are wrong by construction.
-//   1  no workgroup barrier at the stage sync            2  operand requests aimed out of range (no memory traffic)
-//   4  fragments are read from LDS in a tile's first stage only and stay in registers after it
-//   8  every workgroup requests the operands of tile 0 (all requests after the first hit in L2)
-#ifndef SRT_ABLATE
-#define SRT_ABLATE 0
-#endif
-
 // acc += b x a (operands are 16 x 32 fragments, the accumulator a 16 x 16 fp32 tile in AGPRs)
 template <typename T>
 __device__ __forceinline__ void mfma16(f32x4_t& acc, const u32x4_t& b, const u32x4_t& a);
@@ -304,9 +294,6 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
       for (int j = 0; j < 8; ++j) {
         const f32x4_t& tile = FLIP ? acc[j][i] : acc[i][j];
         float a0 = tile[0], a1 = tile[1], a2 = tile[2], a3 = tile[3];
-#ifdef SRT_EPILOGUE_PIN   // measurement builds: pinning the copies costs three register moves per tile
-        asm volatile("" : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3));
-#endif
         if (HAS_BIAS) {
           const float br = T::to_float((S)(b[i].x & 0xffffu));
           a0 += per_row ? br : T::to_float((S)(b[j].x & 0xffffu));
@@ -492,7 +479,6 @@ __device__ __forceinline__ TileRef locate_tile(const GemmProblem& p, int v, int 
   const long long ldb = B_KC ? p.sbn : p.sbk;
   t.offa = (uint32_t)(((long long)bz * p.sab + (A_KC ? (long long)t.m0 * lda : (long long)t.m0)) * 2);
   t.offb = (uint32_t)(((long long)bz * p.sbb + (B_KC ? (long long)t.n0 * ldb : (long long)t.n0)) * 2);
-  if (SRT_ABLATE & 8) t.offa = t.offb = 0;
   return t;
 }
 
@@ -529,11 +515,7 @@ template <int TM> constexpr int phase1_scalar(int u) {      // scalar events 0..
 // k-contiguous A only), for problems that leave compute units idle with the large tile.
 template <typename T, bool A_KC, bool B_KC, int EPI, int NS, int TM = 8>
 __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
-#ifdef SRT_M16_ANY_RING_DEPTH   // measurement builds: shallower rings, to see what the prefetch distance is worth
-  static_assert(NS >= 3 && NS <= 5, "ring depth");
-#else
-  static_assert(NS == 5, "ring depth");   // the library's: five stages of 32 KiB are the whole LDS
-#endif
+  static_assert(NS == 5, "ring depth");   // five stages of 32 KiB are the whole LDS
   static_assert(TM == 8 || (TM == 4 && A_KC), "the 128-row A region is k-contiguous");
   constexpr int TILE_M = 32 * TM;                 // 256 or 128
   constexpr int LPW_A = TM / 2;                   // A loads per wave and stage
@@ -561,8 +543,8 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
   const long long ldb = B_KC ? p.sbn : p.sbk;
   const long long a_view = A_KC ? (long long)(p.M - 1) * lda + p.K : (long long)(p.K - 1) * lda + p.M;
   const long long b_view = B_KC ? (long long)(p.N - 1) * ldb + p.K : (long long)(p.K - 1) * ldb + p.N;
-  const u32x4_t ra = ring::make_rsrc(p.A, (SRT_ABLATE & 2) ? 0u : (uint32_t)(((long long)(p.batch - 1) * p.sab + a_view) * 2));
-  const u32x4_t rb = ring::make_rsrc(p.B, (SRT_ABLATE & 2) ? 0u : (uint32_t)(((long long)(p.batch - 1) * p.sbb + b_view) * 2));
+  const u32x4_t ra = ring::make_rsrc(p.A, (uint32_t)(((long long)(p.batch - 1) * p.sab + a_view) * 2));
+  const u32x4_t rb = ring::make_rsrc(p.B, (uint32_t)(((long long)(p.batch - 1) * p.sbb + b_view) * 2));
   const uint32_t kstep_a = A_KC ? (uint32_t)(BK * 2) : (uint32_t)(BK * lda * 2);   // bytes per k stage
   const uint32_t kstep_b = B_KC ? (uint32_t)(BK * 2) : (uint32_t)(BK * ldb * 2);
   const int KT = (p.K + BK - 1) / BK;
@@ -696,10 +678,8 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
           }
           // the rest of stage kt: B tiles 4-7 (first used half way through the phase), the A tiles of phase 1
           const int rb_ = phase0_b_read<TM>(u), ra_ = phase0_a_read<TM>(u);
-          if (!(SRT_ABLATE & 4) || FIRST) {
-            if (rb_ >= 0) bf[4 + rb_] = fb.read(cur + REGION_A, 4 + rb_);
-            if (ra_ >= 0) af[HALF + ra_] = fa.read(cur, HALF + ra_);
-          }
+          if (rb_ >= 0) bf[4 + rb_] = fb.read(cur + REGION_A, 4 + rb_);
+          if (ra_ >= 0) af[HALF + ra_] = fa.read(cur, HALF + ra_);
           // request r = ka: its A part goes out in phase 1, its B part in phase 0 of the next stage
           const int ev = phase0_scalar<TM>(u);
           if (ev == 0) nxt = cur + STAGE_B;
@@ -713,8 +693,7 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
         }
       }
       // ---- sync: all of stage kt is in registers, stage kt+1 has landed ----
-      if (SRT_ABLATE & 1) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "i"(LOADS * (NS - 2)) : "memory");
-      else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(LOADS * (NS - 2)) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(LOADS * (NS - 2)) : "memory");
       SRT_FENCE();
       // ---- phase 1: the second half of the A tiles; reads of stage kt+1; A loads of stage kt+NS ----
 #pragma unroll
@@ -735,10 +714,8 @@ __global__ __launch_bounds__(NT) void gemm_m16_kernel(GemmProblem p) {
           }
           // stage kt+1: the A tiles of phase 0 (idle since then) and B tiles 0-3, each as it falls free
           const int ra_ = phase1_a_read<TM>(u), rb_ = phase1_b_read<TM>(u);
-          if (!(SRT_ABLATE & 4) || FIRST) {
-            if (ra_ >= 0) af[ra_] = fa.read(nxt, ra_);
-            if (rb_ >= 0) bf[rb_] = fb.read(nxt + REGION_A, rb_);
-          }
+          if (ra_ >= 0) af[ra_] = fa.read(nxt, ra_);
+          if (rb_ >= 0) bf[rb_] = fb.read(nxt + REGION_A, rb_);
           // the stage of request r = ka + 1, and where its B part will land
           const int ev = phase1_scalar<TM>(u);
           if (ev == 0) {

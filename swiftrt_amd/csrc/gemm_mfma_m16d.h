@@ -37,6 +37,9 @@
 // compute units without work in the last round: the tiles left over after the whole rounds are cut along k
 // and all workgroups share them; see gemm_m16d_body.
 #pragma once
+#include <chrono>
+#include <random>
+
 #include "gemm_mfma_m16.h"
 
 namespace srt {
@@ -309,14 +312,11 @@ __device__ __forceinline__ void store_tile_tail(const GemmProblem& p, const f32x
   }
 }
 
-#ifdef SRT_TAIL_TRACE   // measurement builds: times (100 MHz) of piece boundaries, 16 per workgroup
-static __device__ unsigned long long tail_trace[256 * 16];
-#endif
-
 // What the tail-sharing form of the kernel needs beyond the problem (see gemm_m16d_body, SK).
 struct TailShare {
   float* partial;                // [left-over tile][part][wave][64 accumulator tiles][64 lanes][4] floats
   unsigned long long* flags;     // [left-over tile][part]: `epoch` once that piece's partial is complete
+  unsigned int* stored;          // checking builds: [left-over tile] times the tile was stored (else unused)
   unsigned long long epoch;      // a value no earlier use of the memory has left there
   int parts;                     // pieces per left-over tile, 2 or 3
   int cut1, cut2;                // part k covers quads [cut(k), cut(k+1)): 0, cut1, cut2, quads per tile (cut2 = that for 2 parts)
@@ -378,11 +378,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   const int S_full = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least four)
 
   // per-XCD start of the k walk for an A stored k x m (see gemm_ring_kernel)
-#ifndef SRT_M16D_ROTATE   // measurement builds: 0 never, 1 always
   constexpr bool rotate = !A_KC;
-#else
-  constexpr bool rotate = SRT_M16D_ROTATE != 0;
-#endif
   const int rot = rotate && !SK ? (int)(((unsigned)(blockIdx.x & 7) * (unsigned)S_full) / 8u) : 0;
   auto stage_of = [&](int r) {   // r = 0, 1, 2 only; a piece has at least four super-stages
     if constexpr (SK) return r;
@@ -486,17 +482,6 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
 
   uint32_t x = lds;   // slot of A_s; B_s follows it, then A_{s+1}, B_{s+1}, A_{s+2} (B_{s+2} goes where A_s is)
 
-#ifdef SRT_TAIL_TRACE   // measurement builds: times (100 MHz) of piece boundaries, 16 per workgroup
-  int trace_at = 0;
-  auto stamp = [&]() {
-    if (threadIdx.x == 0 && trace_at < 16) tail_trace[blockIdx.x * 16 + trace_at] = (unsigned long long)wall_clock64();
-    ++trace_at;
-  };
-#define SRT_STAMP() stamp()
-#else
-#define SRT_STAMP()
-#endif
-  SRT_STAMP();
   bool first_tile = true;
   for (;;) {
     // per-lane addressing state, derived per tile and scoped to it (see gemm_ring_kernel)
@@ -622,14 +607,12 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
             if (LOADS == 3) ring::load_to_lds_at_m0(rb, lb.voff[Loader<B_KC>::vindex(ld)], so);
             else ring::load_to_lds_at_m0(ra, la.voff[Loader<A_KC>::vindex(ld)], so);
           }
-          if (!(SRT_ABLATE & 4) || FIRST) {   // (measurement builds can keep the first super-stage's fragments)
-            if (OWN) {
-              if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
-              if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.template read<H>(ua, 4 + ((u - 8) >> 1));
-            } else {
-              if (u < 16 && (u & 3) == 1) af[u >> 2] = fa.template read<H>(ua, u >> 2);
-              if (u < 16 && (u & 3) == 3) bf[u >> 2] = fb.template read<H>(ub, u >> 2);
-            }
+          if (OWN) {
+            if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
+            if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.template read<H>(ua, 4 + ((u - 8) >> 1));
+          } else {
+            if (u < 16 && (u & 3) == 1) af[u >> 2] = fa.template read<H>(ua, u >> 2);
+            if (u < 16 && (u & 3) == 3) bf[u >> 2] = fb.template read<H>(ub, u >> 2);
           }
           ev(u);
           SRT_FENCE();
@@ -675,8 +658,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
         if (u == 25) tb = x + Loader<B_KC>::wave_share(wave);
       });
       // ---- sync: all of super-stage s is in registers, A_{s+1} and B_{s+1} have landed ----
-      if (SRT_ABLATE & 1) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       SRT_FENCE();
       // ---- phase 3: k half 1, A tiles 4-7; the loads of B_{s+2}; reads of super-stage s + 1 ----
       phase(C1{}, std::false_type{}, std::false_type{}, C0{}, C3{}, xa1, xb1, tb, so_b0, so_b1, so_b2, so_b3, [&](int u) __attribute__((always_inline)) {
@@ -701,7 +683,6 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     // Every load in flight must have landed, in every wave, before the slots vacated last become the
     // staging area.  The s_nops are the wait states between the last MFMAs and the first reads of their
     // accumulators by other instructions.
-    SRT_STAMP();   // the piece's main loop is done
     // (flipped: the result's rows are this problem's columns)
     const int em0 = FLIP ? cur_tile.n0 + wn0 : cur_tile.m0 + wm0, en0 = FLIP ? cur_tile.m0 + wm0 : cur_tile.n0 + wn0;
     const int bz = cur_tile.bz;
@@ -731,7 +712,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
       // flag before the second look.  (Agent-scope fences would write back and invalidate whole L2s, once
       // per workgroup: measured at 100 us per launch.)
       const bool part_of_tile = cur_piece.tile >= 0;
-      const int place0 = cur_piece.tile * TAIL_MAX_PARTS, mine = cur_piece.part;
+      const int place0 = part_of_tile ? cur_piece.tile * ts.parts : 0, mine = cur_piece.part;
       auto others_done = [&]() {
         bool ok = true;
         for (int k = 0; k < ts.parts; ++k)
@@ -748,8 +729,8 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
         __syncthreads();
         return v != 0;
       };
-      auto partial_of = [&](int part) {
-        float* base = ts.partial + ((size_t)((place0 + part) * 4 + wave) * 64) * 256;
+      auto partial_of = [&](int part) {   // (a whole tile has no partials: an empty descriptor on the workspace's start)
+        float* base = ts.partial + (part_of_tile ? ((size_t)((place0 + part) * 4 + wave) * 64) * 256 : 0);
         return __builtin_amdgcn_make_buffer_rsrc(base, 0, part_of_tile ? 65536 : 0, 0x00020000);
       };
       TailStore how;
@@ -773,6 +754,10 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
           }
           m16::pin_all<TM>(acc);   // (nothing read from the accumulators moves out of the loop)
           store_tile_tail<T, HAS_BIAS, CLAMP, FLIP>(pe, acc, em0, en0, bz, lane_id(), stage, bias_regs, how);
+#ifdef SRT_DEBUG_LAUNCH
+          // checking builds count the stores of every shared tile; the host reads the counts after the launch
+          if (part_of_tile && threadIdx.x == 0) atomicAdd(ts.stored + cur_piece.tile, 1u);
+#endif
           break;
         }
         publish_accumulators(acc, ring::make_rsrc(ts.partial + ((size_t)((place0 + mine) * 4 + wave) * 64) * 256, 65536), lane_id());
@@ -797,7 +782,6 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
       else if (EPI == EPI_CLIPPED) m16::store_tile<T, TM, true, 2, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
       else m16::store_tile<T, TM, false, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
     }
-    SRT_STAMP();   // and its epilogue
     if (!has_next) break;
 
     // every wave has finished reading its staging area before any wave's loads overwrite it
@@ -846,7 +830,8 @@ inline GemmProblem flipped(const GemmProblem& p) {
 
 // ---- the tail-sharing form ----------------------------------------------------------------------------
 constexpr size_t TAIL_PARTIAL_BYTES = 256 * 256 * sizeof(float);   // per piece
-constexpr size_t TAIL_FLAG_BYTES = 8192;                           // 255 x 3 flags, ahead of the partials
+constexpr size_t TAIL_FLAG_BYTES = 8192;                           // 255 x 3 flags (6120 bytes), ahead of the partials
+constexpr size_t TAIL_STORED_OFFSET = 6144;                        // checking builds: 256 store counts behind the flags
 
 // How the tail-sharing form would cut the left-over tiles of `p`; parts = 0: it does not apply.
 struct TailPlan {
@@ -900,13 +885,21 @@ inline TailPlan tail_plan(const GemmProblem& p) {
 }
 inline bool tail_fits(const GemmProblem& p) { return tail_plan(p).parts != 0; }
 
-// Flag values: a process-wide launch counter under a fixed 32-bit tag.  The flags live in memory that
-// other kernels have written before (the allocator recycles blocks), so what they hold at launch is
-// arbitrary; a launch waits for its own value, which no earlier launch has written and which arbitrary
-// data matches with probability 2^-64 per flag.
+// Flag values: a 64-bit launch counter that starts at a value drawn once per process.  The flags live in
+// memory that other kernels have written before (the allocator recycles blocks), so what they hold at launch
+// is arbitrary -- most likely the flags of an earlier launch of this kernel.  Those hold earlier values of the
+// counter, which this launch's value differs from by construction (2^64 launches apart at the earliest);
+// anything else -- other kernels' data, another process's flags in memory the driver handed over -- matches
+// with probability 2^-64 per flag.
 inline unsigned long long next_tail_epoch() {
+  static const unsigned long long start = [] {
+    std::random_device rd;
+    unsigned long long v = ((unsigned long long)rd() << 32) ^ (unsigned long long)rd();
+    v ^= (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9e3779b97f4a7c15ull;
+    return v;
+  }();
   static std::atomic<unsigned long long> counter{0};
-  return 0x5ca1ab1e00000000ull | (++counter & 0xffffffffull);
+  return start + ++counter;
 }
 
 template <typename T, bool A_KC, bool B_KC, int EPI, bool FLIP = false>
@@ -919,7 +912,8 @@ hipError_t launch_tail_kernel(const GemmProblem& p, hipStream_t stream) {
   if (plan.parts == 0) return hipErrorInvalidValue;
   const int grid = compute_units();
   void* workspace = nullptr;
-  const size_t bytes = TAIL_FLAG_BYTES + (size_t)plan.left * TAIL_MAX_PARTS * TAIL_PARTIAL_BYTES;
+  // flags (and, in checking builds, the store counts behind them), then a partial per piece
+  const size_t bytes = TAIL_FLAG_BYTES + (size_t)plan.left * plan.parts * TAIL_PARTIAL_BYTES;
   if (srtDeviceAllocate(&workspace, bytes, reinterpret_cast<srtStream>(stream)) != srtSuccess) return hipErrorOutOfMemory;
   TailShare ts;
   ts.parts = plan.parts;
@@ -928,10 +922,29 @@ hipError_t launch_tail_kernel(const GemmProblem& p, hipStream_t stream) {
   ts.groups = plan.groups;
   ts.per_group = plan.per_group;
   ts.flags = reinterpret_cast<unsigned long long*>(workspace);
+  ts.stored = reinterpret_cast<unsigned int*>(static_cast<unsigned char*>(workspace) + TAIL_STORED_OFFSET);
   ts.partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + TAIL_FLAG_BYTES);
   ts.epoch = next_tail_epoch();
+#ifdef SRT_DEBUG_LAUNCH
+  if (srtMemsetAsync(ts.stored, 0, 256 * sizeof(unsigned int), reinterpret_cast<srtStream>(stream)) != srtSuccess) {
+    (void)srtDeviceFree(workspace);
+    return hipErrorUnknown;
+  }
+#endif
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p, ts);
-  const hipError_t e = launch_status(stream);
+  hipError_t e = launch_status(stream);
+#ifdef SRT_DEBUG_LAUNCH
+  // (launch_status has waited for the kernel.)  No piece ever waits for another; what guarantees that some piece
+  // of every shared tile adds up and stores is the order "publish, raise the flag, look at the others' flags" in
+  // every piece.  Here that is checked: every left-over tile must have been stored at least once.
+  if (e == hipSuccess) {
+    unsigned int counts[256];
+    e = hipMemcpyAsync(counts, ts.stored, sizeof(counts), hipMemcpyDeviceToHost, stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    for (int i = 0; e == hipSuccess && i < plan.left; ++i)
+      if (counts[i] == 0) e = hipErrorLaunchFailure;
+  }
+#endif
   (void)srtDeviceFree(workspace);   // stream-ordered: reused only by work queued after the kernel
   return e;
 }

@@ -105,18 +105,8 @@ template <int IMM>
 __device__ __forceinline__ void set_lds_target(uint32_t lds_base) {
   asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_base), "n"(IMM) : "scc");
 }
-// measurement builds: cache-policy bits of the main loop's operand loads (SRT_LOAD_POLICY_ID 1: nt, 2: sc1, 3: sc0)
-#if !defined(SRT_LOAD_POLICY_ID)
-#define SRT_LOAD_POLICY ""
-#elif SRT_LOAD_POLICY_ID == 1
-#define SRT_LOAD_POLICY " nt"
-#elif SRT_LOAD_POLICY_ID == 2
-#define SRT_LOAD_POLICY " sc1"
-#else
-#define SRT_LOAD_POLICY " sc0"
-#endif
 __device__ __forceinline__ void load_to_lds_at_m0(u32x4_t rsrc, uint32_t voff, uint32_t soff) {
-  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen" SRT_LOAD_POLICY " lds" : : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 // ---- global -> LDS ---------------------------------------------------------------------------
@@ -235,11 +225,7 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
     const int xcd = wg % XCDS, local = wg / XCDS;
     logical = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
   }
-#ifdef SRT_GROUP_M   // measurement builds: another patch shape
-  constexpr int GROUP_M = SRT_GROUP_M;
-#else
   constexpr int GROUP_M = 8;
-#endif
   const int per_group = GROUP_M * tiles_n;
   const int group = logical / per_group;
   const int first_m = group * GROUP_M;

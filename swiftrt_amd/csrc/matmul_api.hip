@@ -8,6 +8,7 @@
 
 #include "gemm_common.h"
 #include "status.h"
+#include "views.h"
 
 namespace {
 
@@ -68,26 +69,27 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
   if (M == 0 || N == 0 || batch == 0) { *empty = true; return srtSuccess; }
   if (!a || !b || !out) return srtErrorInvalidValue;
 
-  // The kernels read operand tiles while other workgroups already store results: a result whose
-  // storage span overlaps the span of an input is refused (the Swift side always hands in a freshly
-  // allocated dense result, operators/Matmul.swift:38-39).
+  // The kernels read operand tiles while other workgroups already store results, so the result must share no
+  // element with an input (the Swift side always hands in a freshly allocated dense result,
+  // operators/Matmul.swift:38-39).  Storage spans that do not overlap settle it.  Views whose spans do overlap
+  // are accepted when a common pitch proves them apart (column slices of one wide buffer, interleaved
+  // batches: see views_disjoint); a result that provably shares an element with an input (the same first element, or overlapping row blocks
+  // of one pitch) is an error; anything else
+  // is answered "not supported", so that the caller's fallback runs instead of a wrong guess either way.
   if (check_alias) {   // (the kernel query takes placeholder pointers and launches nothing)
     const size_t es = od->type == srtReal32F ? 4 : 2;
-    auto span = [&](const void* base, long long e0, long long s0, long long e1, long long s1, long long e2, long long s2,
-                    uintptr_t* lo, uintptr_t* hi) {
-      const long long last = (e0 - 1) * s0 + (e1 - 1) * s1 + (e2 - 1) * s2;   // strides are non-negative (size_t)
-      *lo = reinterpret_cast<uintptr_t>(base);
-      *hi = *lo + (uintptr_t)(last + 1) * es;
+    const srt::StridedView vo = srt::make_view(out, es, p->M, p->scm, p->N, p->scn, p->batch, p->scb);
+    auto verdict = [&](const srt::StridedView& v) {
+      if (!srt::spans_overlap(vo, v)) return srtSuccess;
+      if (srt::views_alias(vo, v)) return srtErrorInvalidValue;
+      return srt::views_disjoint(vo, v) ? srtSuccess : srtErrorNotSupported;
     };
-    uintptr_t olo, ohi, lo, hi;
-    span(out, p->M, p->scm, p->N, p->scn, p->batch, p->scb, &olo, &ohi);
-    span(a, p->M, p->sam, p->K, p->sak, p->batch, p->sab, &lo, &hi);
-    if (p->K > 0 && lo < ohi && olo < hi) return srtErrorInvalidValue;
-    span(b, p->K, p->sbk, p->N, p->sbn, p->batch, p->sbb, &lo, &hi);
-    if (p->K > 0 && lo < ohi && olo < hi) return srtErrorInvalidValue;
+    if (p->K > 0) {
+      if (srtStatus s = verdict(srt::make_view(a, es, p->M, p->sam, p->K, p->sak, p->batch, p->sab)); s != srtSuccess) return s;
+      if (srtStatus s = verdict(srt::make_view(b, es, p->K, p->sbk, p->N, p->sbn, p->batch, p->sbb)); s != srtSuccess) return s;
+    }
     if (bias) {
-      span(bias, p->N, p->sbias, 1, 0, 1, 0, &lo, &hi);
-      if (lo < ohi && olo < hi) return srtErrorInvalidValue;
+      if (srtStatus s = verdict(srt::make_view(bias, es, p->N, p->sbias, 1, 0, 1, 0)); s != srtSuccess) return s;
     }
   }
 

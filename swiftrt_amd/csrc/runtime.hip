@@ -219,6 +219,7 @@ __global__ void delay_kernel(unsigned long long ticks) {
 }  // namespace
 
 namespace srt {
+void prepare_backward_scratch();   // activation_backward.hip
 srtStatus from_hip(hipError_t e) {
   switch (e) {
     case hipSuccess: return srtSuccess;
@@ -300,6 +301,8 @@ srtStatus srtStreamCreate(srtStream* stream) {
   hipStream_t s = nullptr;
   hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);  // default priority
   *stream = reinterpret_cast<srtStream>(s);
+  // once per device: the address of the fixed workspace of srtActivationBackwardBiasNoAlloc
+  if (e == hipSuccess) srt::prepare_backward_scratch();
   return from_hip(e);
 }
 

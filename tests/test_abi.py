@@ -83,6 +83,36 @@ def test_descriptor_validation_without_gpu():
         == native.ERROR_INVALID_VALUE
 
 
+def test_result_alias_rules_without_gpu():
+    # The alias check runs on addresses and strides alone, before any device work: the refusals are observable
+    # on a CPU-only host (the accepted cases go on to a launch and are tested on the GPU).
+    L = native.lib()
+    base = 1 << 20
+
+    def call(a_off, a_shape, a_strides, o_off, o_shape, o_strides, b_shape=None):
+        ad, k1 = native.make_descriptor(native.REAL32F, a_shape, a_strides, native.ORDER_ROW)
+        kk = a_shape[-1]
+        bs = b_shape or ((kk, o_shape[-1]) if len(a_shape) == 2 else (a_shape[0], kk, o_shape[-1]))
+        bst = (bs[-1], 1) if len(bs) == 2 else (bs[-2] * bs[-1], bs[-1], 1)
+        bd, k2 = native.make_descriptor(native.REAL32F, bs, bst, native.ORDER_ROW)
+        od, k3 = native.make_descriptor(native.REAL32F, o_shape, o_strides, native.ORDER_ROW)
+        return L.srtMatmul(ctypes.c_void_p(base + 4 * a_off), ctypes.byref(ad), 0, ctypes.c_void_p(1 << 30), ctypes.byref(bd), 0,
+                           ctypes.c_void_p(base + 4 * o_off), ctypes.byref(od), None)
+
+    # the same first element: provably aliased
+    assert call(0, (32, 32), (64, 1), 0, (32, 32), (64, 1)) == native.ERROR_INVALID_VALUE
+    # overlapping row blocks of one 64-wide buffer, same columns: provably aliased
+    assert call(0, (32, 32), (64, 1), 16 * 64, (32, 32), (64, 1)) == native.ERROR_INVALID_VALUE
+    # row blocks that overlap with column ranges that meet in part: provably aliased too
+    assert call(0, (32, 32), (64, 1), 16 * 64 + 16, (32, 32), (64, 1)) == native.ERROR_INVALID_VALUE
+    # spans overlap, pitches differ: the check cannot tell -> the caller's fallback
+    assert call(0, (32, 32), (64, 1), 40, (32, 32), (48, 1)) == native.ERROR_NOT_SUPPORTED
+    # a transposed view covers the same elements as the block it transposes: provably aliased with a result 8 columns along
+    assert call(0, (32, 32), (1, 64), 8, (32, 32), (64, 1)) == native.ERROR_INVALID_VALUE
+    # rows of 32 under a pitch of 96 against rows under a pitch of 64, 8 elements in: apart or not, no pitch shows it
+    assert call(0, (32, 32), (96, 1), 8, (32, 32), (64, 1)) == native.ERROR_NOT_SUPPORTED
+
+
 def test_elementwise_and_backward_validation_without_gpu():
     L = native.lib()
     dummy = ctypes.c_void_p(256)

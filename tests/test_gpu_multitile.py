@@ -463,3 +463,34 @@ def test_result_overlapping_an_operand_is_refused():
     lo, hi = buf[0:32, :], buf[32:64, :]
     w = srt.Tensor(np.eye(64, dtype=np.float32))
     q.matmul(lo, False, w, False, hi)
+
+
+def test_column_slices_and_interleaved_batches_of_one_buffer_are_accepted():
+    # storage spans overlap, yet a common pitch proves the views apart: operand, bias and result as column
+    # slices of one wide row-major buffer, and operand and result as alternate batches of one buffer
+    q = srt.current_queue()
+    r = H.rng(91)
+    wide = r.integers(-3, 4, (48, 96)).astype(np.float32)
+    buf = srt.Tensor(wide.copy())
+    w = r.integers(-3, 4, (32, 32)).astype(np.float32)
+    a, out = buf[:, 0:32], buf[:, 64:96]
+    bias = srt.Tensor(shape=[32], order=buf.order, _storage=buf.storage, _offset=buf.offset + 32, _strides=[1])
+    q.matmul(a, False, srt.Tensor(w), False, out, bias=bias)
+    got = buf.array()
+    assert np.array_equal(got[:, 64:96], wide[:, 0:32] @ w + wide[0, 32:64])
+    assert np.array_equal(got[:, 0:64], wide[:, 0:64])            # the rest of the buffer is untouched
+    both = r.integers(-3, 4, (6, 16, 24)).astype(np.float32)
+    buf3 = srt.Tensor(both.copy())
+    w3 = r.integers(-3, 4, (3, 24, 24)).astype(np.float32)
+    q.matmul(buf3[0::2], False, srt.Tensor(w3), False, buf3[1::2])
+    got = buf3.array()
+    assert np.array_equal(got[1::2], both[0::2] @ w3)
+    assert np.array_equal(got[0::2], both[0::2])
+    # even against odd columns of one buffer (the element pitch of 2 proves them apart)
+    eo = r.integers(-3, 4, (16, 64)).astype(np.float32)
+    buf2 = srt.Tensor(eo.copy())
+    w2 = r.integers(-3, 4, (32, 32)).astype(np.float32)
+    q.matmul(buf2[:, 0::2], False, srt.Tensor(w2), False, buf2[:, 1::2])
+    got = buf2.array()
+    assert np.array_equal(got[:, 1::2], eo[:, 0::2] @ w2)
+    assert np.array_equal(got[:, 0::2], eo[:, 0::2])
