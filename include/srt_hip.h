@@ -253,6 +253,7 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
  * (sums are fp32; their order differs between plans).
  * chosen (optional): receives the plan's name ("mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail" (the same kernel
  * with the tiles left over after its whole rounds cut along k; its result does not depend on timing either),
+ * "mfma_256x256_m16_k64_split" (the same kernel with its last round in 192-wide tiles: only ever a tuned or loaded plan),
  * "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
  * "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any" (16-bit
  * operands of any stride and alignment), "skinny", "f32_mfma_64x64", "f32_mfma_splitk", "generic").

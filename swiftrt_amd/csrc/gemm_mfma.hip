@@ -84,6 +84,15 @@ SRT_M16DP_DECL(BF16)
 SRT_M16DP_DECL(F16)
 #undef SRT_M16DP_DECL
 bool m16d_tail_fits_BF16_xx(const GemmProblem&);   // (the answer does not depend on the element type)
+#define SRT_M16DS_DECL(T)                                                       \
+  hipError_t launch_m16d_split_##T##_00(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_split_##T##_01(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_split_##T##_10(const GemmProblem&, hipStream_t);       \
+  hipError_t launch_m16d_split_##T##_11(const GemmProblem&, hipStream_t);
+SRT_M16DS_DECL(BF16)
+SRT_M16DS_DECL(F16)
+#undef SRT_M16DS_DECL
+bool m16d_split_fits_BF16_xx(const GemmProblem&);
 hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_F16_10(const GemmProblem&, hipStream_t);
@@ -547,6 +556,20 @@ hipError_t launch_m16d_tail(const GemmProblem& p, bool a_kc, bool b_kc, hipStrea
   if (b_kc) return launch_m16d_tail_F16_01(p, stream);
   return launch_m16d_tail_F16_00(p, stream);
 }
+// the split form of the 64-deep kernel: whole rounds of whole tiles, then one round of 192-wide ones
+template <typename T>
+hipError_t launch_m16d_split(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) {
+    if (a_kc && b_kc) return launch_m16d_split_BF16_11(p, stream);
+    if (a_kc) return launch_m16d_split_BF16_10(p, stream);
+    if (b_kc) return launch_m16d_split_BF16_01(p, stream);
+    return launch_m16d_split_BF16_00(p, stream);
+  }
+  if (a_kc && b_kc) return launch_m16d_split_F16_11(p, stream);
+  if (a_kc) return launch_m16d_split_F16_10(p, stream);
+  if (b_kc) return launch_m16d_split_F16_01(p, stream);
+  return launch_m16d_split_F16_00(p, stream);
+}
 template <typename T>
 hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16h_BF16_11(p, stream) : launch_m16h_BF16_10(p, stream);
@@ -564,6 +587,7 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 6: return launch_m16h<T>(p, b_kc, stream);
     case 9: return launch_m16d<T>(p, a_kc, b_kc, stream);
     case 10: return launch_m16d_tail<T>(p, a_kc, b_kc, stream);
+    case 11: return launch_m16d_split<T>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     case 7: return launch_any_layout<T, 128, 128>(p, stream);
     case 8: return launch_any_layout<T, 64, 64>(p, stream);
@@ -602,7 +626,7 @@ static int mfma_layout(const GemmProblem& p) {
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
 // 128 x 256 form for a k-contiguous A, 9: the 16x16x32 kernel with 64-deep staging units), or 0 when the
-// problem does not qualify for it.  10: tile 9's tail-sharing form.
+// problem does not qualify for it.  10: tile 9's tail-sharing form.  11: its split form (a last round of 192-wide tiles).
 int mfma_config(const GemmProblem& p, int tile) {
   if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
     if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
@@ -610,13 +634,15 @@ int mfma_config(const GemmProblem& p, int tile) {
     return tile << 2;
   }
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || (tile > 6 && tile != 9 && tile != 10)) return 0;
+  if (layout < 0 || tile < 1 || (tile > 6 && tile != 9 && tile != 10 && tile != 11)) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
   if (tile == 9 && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
   if (tile == 10) {   // left-over tiles to share, k in whole quads, no transcendental activation
     const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
     if (trans || !m16d_tail_fits_BF16_xx(p)) return 0;
   }
+  // whole rounds of whole tiles and a last round that 192-wide tiles fill, no transcendental activation (pinned or tuned plans only)
+  if (tile == 11 && !m16d_split_fits_BF16_xx(p)) return 0;
   if (tile == 6 && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
@@ -999,6 +1025,7 @@ const char* mfma_name(int config) {
     case 6: return "mfma_128x256_m16";
     case 9: return "mfma_256x256_m16_k64";
     case 10: return "mfma_256x256_m16_k64_tail";
+    case 11: return "mfma_256x256_m16_k64_split";
     case 2: return "mfma_128x128";
     case 7: return "mfma_128x128_any";
     case 8: return "mfma_64x64_any";

@@ -90,12 +90,12 @@ __device__ __forceinline__ void mfma16_first<F16>(f32x4_t& acc, const u32x4_t& b
 
 // An empty statement that "rewrites" every accumulator tile: reads of the accumulators that follow it in
 // the source cannot be scheduled ahead of it (see ring::pin).
-template <int TM>
-__device__ __forceinline__ void pin_all(f32x4_t (&acc)[TM][8]) {
+template <int TM, int TN = 8>
+__device__ __forceinline__ void pin_all(f32x4_t (&acc)[TM][TN]) {
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+    for (int j = 0; j < TN; ++j) asm volatile("" : "+a"(acc[i][j]));
 }
 
 // ---- global -> LDS --------------------------------------------------------------------------------
@@ -258,10 +258,13 @@ __device__ __forceinline__ void load_bias(const GemmProblem& p, int wave_m0, int
 // FLIP: the accumulator of the tile in row group i, column group j of the result is acc[j][i] (the kernel computed
 // the transposed product with the operands' roles exchanged; each 16 x 16 tile lies in the registers as it does
 // otherwise).
-template <typename T, int TM, bool HAS_BIAS, int CLAMP, bool FLIP = false>
-__device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[TM][8], int wave_m0, int wave_n0,
-                                           int bz, int lane, uint32_t stage, const u32x2_t (&b)[8]) {
-  static_assert(!FLIP || TM == 8, "a square block of accumulator tiles");
+// TN: column tiles per wave (8; 6 for the 192-wide workgroup tile, whose wave covers 96 columns).  n_end: columns at
+// or beyond it belong to another tile and are not stored (a workgroup tile narrower than its MFMA footprint).
+template <typename T, int TM, bool HAS_BIAS, int CLAMP, bool FLIP = false, int TN = 8>
+__device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (&acc)[TM][TN], int wave_m0, int wave_n0,
+                                           int bz, int lane, uint32_t stage, const u32x2_t (&b)[8], int n_end = 0x7fffffff) {
+  static_assert(!FLIP || (TM == 8 && TN == 8), "a square block of accumulator tiles");
+  static_assert(TN <= 8, "the staging rows hold 16 chunks");
   constexpr int ROWS = TM == 8 ? 64 : 32;
   using S = typename T::storage;
   const bool per_row = p.bias_per_row != 0;
@@ -274,13 +277,14 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
   const int jn = lane & 15, g = lane >> 4;
   const int rd_chunk = lane & 15, rd_row = lane >> 4;   // read side: chunk of rows rd_row + 4 it
   const int n_rd = wave_n0 + 8 * rd_chunk;
-  const bool n_rd_ok = n_rd < p.N;   // N is a multiple of 8 (checked on the host): the chunk is whole
+  // N is a multiple of 8 (checked on the host): the chunk is whole
+  const bool n_rd_ok = n_rd < p.N && (TN == 8 || (rd_chunk < 2 * TN && n_rd < n_end));
 
   // staging address of accumulator tile (ii, j): row 16 ii + jn, chunk (2 j + g / 2) ^ jn -- the lane's part of
   // it is the same for every ii (a row group is 4096 bytes further: an immediate offset of the write)
-  uint32_t wr[8];
+  uint32_t wr[TN];
 #pragma unroll
-  for (int j = 0; j < 8; ++j)
+  for (int j = 0; j < TN; ++j)
     wr[j] = stage + (uint32_t)jn * 256u + (uint32_t)(g & 1) * 8u + (uint32_t)(((2 * j + (g >> 1)) ^ jn) << 4);
 
 #pragma unroll
@@ -291,9 +295,10 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
       const int i = (ROWS / 16) * half + ii;
       SRT_FENCE();
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const f32x4_t& tile = FLIP ? acc[j][i] : acc[i][j];
-        float a0 = tile[0], a1 = tile[1], a2 = tile[2], a3 = tile[3];
+      for (int j = 0; j < TN; ++j) {
+        float a0, a1, a2, a3;
+        if constexpr (FLIP) { a0 = acc[j][i][0]; a1 = acc[j][i][1]; a2 = acc[j][i][2]; a3 = acc[j][i][3]; }
+        else { a0 = acc[i][j][0]; a1 = acc[i][j][1]; a2 = acc[i][j][2]; a3 = acc[i][j][3]; }
         if (HAS_BIAS) {
           const float br = T::to_float((S)(b[i].x & 0xffffu));
           a0 += per_row ? br : T::to_float((S)(b[j].x & 0xffffu));

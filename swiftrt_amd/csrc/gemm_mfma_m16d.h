@@ -143,6 +143,25 @@ struct FragReader<false> {
   }
 };
 
+// ---- the schedule's slots for a wave tile of TN column tiles (a phase is 4 TN MFMAs, u = 4 j + i) -----------------
+// TN = 8 is the schedule as described above.  TN = 6 (the 192-wide workgroup tile: 24 MFMAs per phase) keeps the order
+// of events and moves them to earlier slots: the A loads ride on MFMAs 8, 12, 16, 20 of phases 0 and 1, the eight B
+// loads on every third MFMA of phase 3, and the scalar bookkeeping goes where the table below says.
+template <int TN> constexpr int a_load_at(int u) {   // index 0..3 of the A load riding on MFMA u (phases 0, 1), or -1
+  return (u >= 4 * TN - 16 && (u & 3) == 0) ? (u - (4 * TN - 16)) >> 2 : -1;
+}
+template <int TN> constexpr int b_load_at(int u) {   // index 0..7 of the B load riding on MFMA u (phase 3), or -1
+  return TN == 8 ? ((u & 3) == 0 ? u >> 2 : -1) : ((u % 3 == 0 && u < 24) ? u / 3 : -1);
+}
+// The slot of the TN = 8 schedule whose scalar bookkeeping happens behind MFMA u of phase PH (-1: none)
+template <int TN, int PH> constexpr int event_at(int u) {
+  if (TN == 8) return u;
+  if (PH == 0) return u < 7 ? 2 * u + 1 : -1;                      // 1, 3, .. 13 -> 0 .. 6 (ahead of the loads from 8 on)
+  if (PH == 1) return u;                                           // 2, 6, 10, 14
+  if (PH == 2) return (u >= 15 && (u & 1) == 1) ? u + 2 : -1;      // 17 .. 25 -> 15 .. 23
+  return u == 13 ? 18 : u == 17 ? 22 : u == 22 ? 26 : -1;          // 18, 22, 26 -> 13, 17, 22 (clear of the loads)
+}
+
 // The epilogue of the tail-sharing form: m16::store_tile (TM = 8) with switches that are uniform at run time,
 // so that the kernel holds one copy of it and one place where the accumulators are read.  (With a copy per
 // case the compiler moves all 256 accumulators out of their registers once, ahead of the branches, spilling
@@ -345,9 +364,14 @@ constexpr int TAIL_MAX_PARTS = 3;
 // addresses the tile block transposed.  For a k-contiguous A against an n-contiguous B this makes the operand
 // with the transposing LDS reads the one whose fragments are read four tiles per phase (1512 -> 1540 TFLOP/s at
 // 8192^3: the kernel runs 2 % faster whenever its B is k-contiguous, whatever A is).
-template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false>
+// TN: column tiles per wave.  8: the 256 x 256 tile.  6: a workgroup tile of 256 x 192 MFMA footprint (waves of 128 x 96)
+// whose valid width p.tile_n <= 192 is a multiple of 8 -- tiles lie p.tile_n columns apart and columns beyond that
+// width are computed and not stored.  It fills a last round of the persistent grid that whole tiles would leave three
+// quarters full or less (see gemm_m16d_split_kernel).  B is staged as for the wide tile (a 256-wide unit).
+template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false, int TN = 8>
 __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailShare& ts) {
   static_assert(!FLIP || (EPI != EPI_PARTIAL && EPI != EPI_TRANS), "flipped: the store_tile epilogues only");
+  static_assert(TN == 8 || (TN == 6 && !SK && !FLIP && EPI != EPI_PARTIAL && EPI != EPI_TRANS), "the narrow tile: plain form, store_tile epilogues");
   constexpr int TM = 8;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
@@ -359,9 +383,10 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     asm volatile("" : "+s"(zero));   // opaque: keeps the two instructions where they are written
     return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
   };
-  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * (16 * TN);
 
-  const int tiles_m = (p.M + 255) / 256, tiles_n = (p.N + BN - 1) / BN;
+  const int tile_w = TN == 8 ? BN : p.tile_n;   // columns between neighbouring tiles
+  const int tiles_m = (p.M + 255) / 256, tiles_n = (p.N + tile_w - 1) / tile_w;
   const int total = tiles_m * tiles_n * p.batch;
   const int grid = (int)gridDim.x;
   int v = (int)blockIdx.x;
@@ -372,6 +397,15 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   const long long b_view = B_KC ? (long long)(p.N - 1) * ldb + p.K : (long long)(p.K - 1) * ldb + p.N;
   const u32x4_t ra = ring::make_rsrc(p.A, (uint32_t)(((long long)(p.batch - 1) * p.sab + a_view) * 2));
   const u32x4_t rb = ring::make_rsrc(p.B, (uint32_t)(((long long)(p.batch - 1) * p.sbb + b_view) * 2));
+  // tile number -> position and operand offsets (the narrow tile's columns lie tile_w apart)
+  auto locate = [&](int tile) {
+    TileRef t = m16::locate_tile<A_KC, B_KC, 256>(p, tile, tiles_m, tiles_n);
+    if constexpr (TN != 8) {
+      t.n0 = (t.n0 / BN) * tile_w;
+      t.offb = (uint32_t)(((long long)t.bz * p.sbb + (B_KC ? (long long)t.n0 * ldb : (long long)t.n0)) * 2);
+    }
+    return t;
+  };
   const uint32_t kstep_a = A_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * lda * 2);   // bytes per super-stage
   const uint32_t kstep_b = B_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * ldb * 2);
   const uint32_t lstep_a = Loader<A_KC>::step(lda), lstep_b = Loader<B_KC>::step(ldb);
@@ -463,7 +497,8 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     uniform(cur_piece);
     cur_tile = cur_piece.t;
   } else {
-    cur_tile = m16::locate_tile<A_KC, B_KC, 256>(p, v, tiles_m, tiles_n);
+    if (v >= total) return;   // (a walk with fewer tiles than workgroups: the split kernel's)
+    cur_tile = locate(v);
   }
 
   // the eight loads of one unit, outside the main loop (first fill, and B_1 after an epilogue)
@@ -520,8 +555,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     } else {
       vn = v + grid;
       has_next = vn < total;
-      next_tile =
-          m16::locate_tile<A_KC, B_KC, 256>(p, (int)select_lt(vn, total, (uint32_t)vn, (uint32_t)v), tiles_m, tiles_n);
+      next_tile = locate((int)select_lt(vn, total, (uint32_t)vn, (uint32_t)v));
     }
     const int vn_bound = SK ? 1 : total;
     // A requests below limit_a are real (A'_0 and A'_1 of the next tile); of B only B'_0: B'_1 would land in
@@ -529,8 +563,8 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     const int limit_a = (int)select_lt(vn, vn_bound, (uint32_t)(S + 2), (uint32_t)S);
     const int limit_b = (int)select_lt(vn, vn_bound, (uint32_t)(S + 1), (uint32_t)S);
 
-    f32x4_t acc[TM][8];   // defined by the MFMAs of the tile's first super-stage
-    u32x4_t af[TM], bf[8];
+    f32x4_t acc[TM][TN];   // defined by the MFMAs of the tile's first super-stage
+    u32x4_t af[TM], bf[TN];
 #pragma unroll
     for (int t = 0; t < 4; ++t) bf[t] = fb.template read<0>(xb, t);
 #pragma unroll
@@ -556,14 +590,15 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
       constexpr bool OWN = decltype(own_tag)::value;
       constexpr int H = decltype(h_tag)::value;
       constexpr int LOADS = decltype(loads_tag)::value;
+      constexpr int PH = LOADS == 1 ? 0 : LOADS == 2 ? 1 : LOADS == 0 ? 2 : 3;   // the phase's number
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < TN; ++j) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int u = 4 * j + i;
           // which load, if any, rides on this MFMA
-          const int ld = LOADS == 3 ? ((u & 3) == 0 ? u >> 2 : -1)
-                       : (LOADS == 1 || LOADS == 2) ? ((u >= 16 && (u & 3) == 0) ? ((u - 16) >> 2) + (LOADS == 2 ? 4 : 0) : -1)
+          const int ld = LOADS == 3 ? b_load_at<TN>(u)
+                       : (LOADS == 1 || LOADS == 2) ? (a_load_at<TN>(u) >= 0 ? a_load_at<TN>(u) + (LOADS == 2 ? 4 : 0) : -1)
                        : -1;
           if (ld >= 0) {
             if (LOADS == 3) {
@@ -608,13 +643,13 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
             else ring::load_to_lds_at_m0(ra, la.voff[Loader<A_KC>::vindex(ld)], so);
           }
           if (OWN) {
-            if (u < 8 && (u & 1) == 0) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
+            if (u < 8 && (u & 1) == 0 && 4 + (u >> 1) < TN) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
             if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.template read<H>(ua, 4 + ((u - 8) >> 1));
           } else {
             if (u < 16 && (u & 3) == 1) af[u >> 2] = fa.template read<H>(ua, u >> 2);
             if (u < 16 && (u & 3) == 3) bf[u >> 2] = fb.template read<H>(ub, u >> 2);
           }
-          ev(u);
+          ev(event_at<TN, PH>(u));
           SRT_FENCE();
         }
       }
@@ -694,6 +729,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     if (LINEAR_BIAS) m16::load_bias<T, TM>(pe, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
     if (LINEAR_BIAS || SK) m16::pin_all<TM>(acc);
+    const int n_end = cur_tile.n0 + tile_w;   // (the narrow tile: its valid columns end here)
     // staging: the slots of A_{S-1} (waves 0, 1) and B_{S-1} (waves 2, 3), half a slot each; x is A_S's by now
     uint32_t sa = x < lds + 2 * UNIT ? x + 3 * UNIT : x - 2 * UNIT;
     uint32_t sb = x < lds + UNIT ? x + 4 * UNIT : x - UNIT;
@@ -770,17 +806,17 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
         });
         if (!finish) break;
       }
-    } else if (EPI == EPI_PARTIAL) {
+    } else if constexpr (EPI == EPI_PARTIAL) {
       m16::store_tile_partial<TM>(p, acc, em0, en0, bz, le, stage);
-    } else if (EPI == EPI_TRANS) {
+    } else if constexpr (EPI == EPI_TRANS) {
       m16::load_bias<T, TM>(p, em0, en0, le, bias_regs);
       m16::store_tile_transcendental<T, TM>(p, acc, em0, en0, bz, le, stage, bias_regs);
     } else {
-      if (EPI == EPI_BIAS) m16::store_tile<T, TM, true, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
-      else if (EPI == EPI_RELU) m16::store_tile<T, TM, false, 1, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
-      else if (EPI == EPI_BIAS_RELU) m16::store_tile<T, TM, true, 1, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
-      else if (EPI == EPI_CLIPPED) m16::store_tile<T, TM, true, 2, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
-      else m16::store_tile<T, TM, false, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs);
+      if (EPI == EPI_BIAS) m16::store_tile<T, TM, true, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else if (EPI == EPI_RELU) m16::store_tile<T, TM, false, 1, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else if (EPI == EPI_BIAS_RELU) m16::store_tile<T, TM, true, 1, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else if (EPI == EPI_CLIPPED) m16::store_tile<T, TM, true, 2, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else m16::store_tile<T, TM, false, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
     }
     if (!has_next) break;
 
@@ -800,6 +836,22 @@ __global__ __launch_bounds__(NT) void gemm_m16d_kernel(GemmProblem p) {
 template <typename T, bool A_KC, bool B_KC, int EPI, bool FLIP = false>
 __global__ __launch_bounds__(NT) void gemm_m16d_tail_kernel(GemmProblem p, TailShare ts) {
   gemm_m16d_body<T, A_KC, B_KC, EPI, true, FLIP>(p, ts);
+}
+
+// Two tile walks in one launch, for a tile count that leaves the last round of the persistent grid between half
+// and three quarters full (688 tiles on 256 units: 2.69 rounds, 3 paid).  The columns are cut in two: `wide` covers
+// the first columns in whole 256 x 256 tiles that fill whole rounds (it is the problem as the plain kernel would get
+// it, flipped where that one flips), `narrow` the remaining columns in one round of tiles of 192-wide footprint (TN =
+// 6), which cost about three quarters of a whole tile each.  Every workgroup runs its share of the first walk and then
+// of the second: no launch boundary and no waiting between them.  (`narrow` is never flipped: its columns are the
+// caller's.)
+template <typename T, bool A_KC, bool B_KC, int EPI>
+__global__ __launch_bounds__(NT) void gemm_m16d_split_kernel(GemmProblem wide, GemmProblem narrow) {
+  constexpr bool FLIP = A_KC && !B_KC;
+  gemm_m16d_body<T, FLIP ? false : A_KC, FLIP ? true : B_KC, EPI, false, FLIP>(wide, TailShare{});
+  // the second walk starts from scratch in LDS: every wave is done with the first walk's staging area
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  gemm_m16d_body<T, A_KC, B_KC, EPI, false, false, 6>(narrow, TailShare{});
 }
 
 #undef SRT_FENCE
@@ -998,6 +1050,72 @@ hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   }
   if (p.bias) return launch_kernel<T, KA, KB, EPI_BIAS, FLIP>(q, stream);
   return launch_kernel<T, KA, KB, EPI_PLAIN, FLIP>(q, stream);
+}
+
+// ---- the split form: whole rounds of whole tiles, then one round of narrow tiles (gemm_m16d_split_kernel) ----------
+// wide_cols = 0: the form does not apply.
+struct SplitPlan {
+  int wide_cols;   // columns of the first walk: whole 256-wide tiles that fill whole rounds of the grid
+  int narrow_w;    // valid width of the second walk's tiles (a multiple of 8 in (128, 192])
+  int grid;
+};
+inline SplitPlan split_plan(const GemmProblem& p) {
+  SplitPlan s{0, 0, 0};
+  const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
+  if (!deep_fits(p) || p.batch != 1 || trans) return s;
+  const int grid = compute_units() & ~7;
+  if (grid <= 0) return s;
+  const long long tiles_m = (p.M + 255) / 256, cols = (p.N + 255) / 256;
+  const long long rounds = tiles_m * cols / grid;        // whole rounds of whole tiles
+  if (rounds < 1 || tiles_m * cols == rounds * grid || tiles_m > grid) return s;
+  const long long c1 = rounds * grid / tiles_m;          // column tiles of the first walk (at most `rounds` rounds)
+  const long long c2 = grid / tiles_m;                   // narrow tiles per row of tiles: one round holds them all
+  const long long rest = p.N - 256 * c1;                 // columns left for the second walk
+  if (c1 < 1 || rest <= 0) return s;
+  const long long w = ((rest + c2 - 1) / c2 + 7) & ~7LL;
+  // wider than 192: whole tiles lose nothing to speak of; up to 128: a tile half as wide would be the one (not built)
+  if (w > 192 || w <= 128) return s;
+  s.wide_cols = (int)(256 * c1);
+  s.narrow_w = (int)w;
+  s.grid = grid;
+  return s;
+}
+inline bool split_fits(const GemmProblem& p) { return split_plan(p).wide_cols != 0; }
+
+template <typename T, bool A_KC, bool B_KC, int EPI>
+hipError_t launch_split_kernel(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_m16d_split_kernel<T, A_KC, B_KC, EPI>;
+  constexpr int lds_bytes = UNITS * UNIT;
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
+  const SplitPlan plan = split_plan(p);
+  if (plan.wide_cols == 0) return hipErrorInvalidValue;
+  auto at = [](const void* base, long long elements) {
+    return static_cast<const void*>(static_cast<const char*>(base) + elements * 2);   // 16-bit elements
+  };
+  GemmProblem wide = p, narrow = p;
+  wide.N = plan.wide_cols;
+  narrow.N = p.N - plan.wide_cols;
+  narrow.tile_n = plan.narrow_w;
+  narrow.B = at(p.B, (long long)plan.wide_cols * p.sbn);
+  narrow.C = const_cast<void*>(at(p.C, (long long)plan.wide_cols * p.scn));
+  if (p.bias && !p.bias_per_row) narrow.bias = at(p.bias, (long long)plan.wide_cols * p.sbias);
+  constexpr bool FLIP = A_KC && !B_KC;
+  const GemmProblem first = FLIP ? flipped(wide) : wide;
+  hipLaunchKernelGGL(kernel, dim3(plan.grid), dim3(NT), lds_bytes, stream, first, narrow);
+  return launch_status(stream);
+}
+
+// (the transcendental activations have no split form)
+template <typename T, bool A_KC, bool B_KC>
+hipError_t launch_split(const GemmProblem& p, hipStream_t stream) {
+  if (p.activation == srtActivationClippedRelu) return launch_split_kernel<T, A_KC, B_KC, EPI_CLIPPED>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_split_kernel<T, A_KC, B_KC, EPI_BIAS_RELU>(p, stream);
+    return launch_split_kernel<T, A_KC, B_KC, EPI_RELU>(p, stream);
+  }
+  if (p.bias) return launch_split_kernel<T, A_KC, B_KC, EPI_BIAS>(p, stream);
+  return launch_split_kernel<T, A_KC, B_KC, EPI_PLAIN>(p, stream);
 }
 
 // The split-K pass: fp32 accumulators to a workspace, no epilogue arithmetic.

@@ -114,13 +114,13 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
 // (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
 // and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
 enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK,
-            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanCount };
+            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanM16DSplit, kPlanCount };
 
 const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
                                             "f32_mfma_64x64", "f32_mfma_splitk", "mfma_256x256_k64",
                                             "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16",
                                             "mfma_128x128_any", "mfma_64x64_any", "mfma_256x256_m16_k64",
-                                            "mfma_256x256_m16_k64_tail"};
+                                            "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split"};
 
 bool plan_supported(const GemmProblem& p, Plan plan) {
   switch (plan) {
@@ -136,6 +136,7 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
     case kPlanAny64: return srt::mfma_config(p, 8) != 0;
     case kPlanM16D: return srt::mfma_config(p, 9) != 0;
     case kPlanM16DTail: return srt::mfma_config(p, 10) != 0;
+    case kPlanM16DSplit: return srt::mfma_config(p, 11) != 0;
     case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
     case kPlanF32SplitK: return srt::f32_mfma_supported(p);
     default: return srt::generic_supported(p);
@@ -154,6 +155,10 @@ Plan heuristic_plan(const GemmProblem& p) {
   if (streams && few_parts && p.M <= 32) return kPlanSkinny;
   // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units
   if (srt::mfma_prefers_tail(p)) return kPlanM16DTail;
+  // (The split form -- whole rounds of whole tiles, then one round of 192-wide ones -- is never the heuristic's choice:
+  // on this power-limited device the compute units that idle through a ragged last round lend their power to the busy
+  // ones, and the form measures the same as whole tiles or worse.  4096 x 11008 x 4096, 2.69 rounds, same run: 249-257 us
+  // whole, 254-258 split; 2048 x 13000 x 4096, 1.59 rounds: 158-162 against 168-170.  srtMatmulTune still times it.)
   if (streams && few_parts) return kPlanSkinny;
   // few 256 x 256 tiles and a long k loop: K split over the idle compute units
   if (srt::mfma_prefers_splitk(p)) return kPlanSplitK;
@@ -191,6 +196,7 @@ hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
     case kPlanAny64: return srt::launch_mfma(p, srt::mfma_config(p, 8), stream);
     case kPlanM16D: return srt::launch_mfma(p, srt::mfma_config(p, 9), stream);
     case kPlanM16DTail: return srt::launch_mfma(p, srt::mfma_config(p, 10), stream);
+    case kPlanM16DSplit: return srt::launch_mfma(p, srt::mfma_config(p, 11), stream);
     case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
     case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
     default: return srt::launch_generic(p, stream);

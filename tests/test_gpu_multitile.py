@@ -448,6 +448,36 @@ def test_reference_kat_batched_and_right_batched(kats, dt):
     assert np.array_equal(got.view(np.uint8), H.encode(np.array(kr["c"], np.float32), dt).view(np.uint8))
 
 
+# ---- the split form: whole rounds of 256 x 256 tiles, then one round of 192-wide tiles ----------------------------
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+@pytest.mark.parametrize("ta,tb", LAYOUTS)
+def test_split_form_integer_bit_exact(dt, ta, tb, tmp_path):
+    """4096 x 11008 (16 x 43 tiles = 2.69 rounds of 256 workgroups: 8192 columns in whole tiles, 2816 in 16 narrow tiles
+    of 176 per row of tiles) with bias + relu, K = 512; 2000 x 13000 x 256 (8 x 51 tiles = 1.59 rounds: 32 narrow tiles of
+    152 per row, ragged last row of tiles); 4104 x 10480 x 320 (17 rows of tiles, 15 narrow tiles of 192 per row: 255 of the 256
+    workgroups take one)."""
+    check_plan(tmp_path, "mfma_256x256_m16_k64_split", dt, 4096, 11008, 512, ta, tb, with_bias_relu=True)
+    check_plan(tmp_path, "mfma_256x256_m16_k64_split", dt, 2000, 13000, 256, ta, tb)
+    check_plan(tmp_path, "mfma_256x256_m16_k64_split", dt, 4104, 10480, 320, ta, tb, with_bias_relu=True)
+
+
+def test_split_form_is_offered_for_the_dense_shape_and_refused_where_it_does_not_apply(tmp_path):
+    a = srt.Tensor(shape=[4096, 4096], dtype=np.uint16)
+    b = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+    out = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_m16_k64"      # the heuristic never takes it (a wash)
+    pin(tmp_path, "mfma_256x256_m16_k64_split", H.BF16, 4096, 11008, 4096, False, False)
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_m16_k64_split"
+    # 8192^3 has no ragged round; 4096 x 10240 leaves exactly half a round (a 128-wide tile's case); a batch has no split form
+    for (M, N, K, batch) in [(8192, 8192, 8192, 1), (4096, 10240, 4096, 1), (1024, 2752, 256, 4)]:
+        lead = [batch] if batch > 1 else []
+        a = srt.Tensor(shape=lead + [M, K], dtype=np.uint16)
+        b = srt.Tensor(shape=lead + [K, N], dtype=np.uint16)
+        out = srt.Tensor(shape=lead + [M, N], dtype=np.uint16)
+        pin(tmp_path, "mfma_256x256_m16_k64_split", H.BF16, M, N, K, False, False, batch=batch)
+        assert query_kernel(a, False, b, False, out) != "mfma_256x256_m16_k64_split", (M, N, K, batch)
+
+
 # ---- operands that alias the result -------------------------------------------------------------------
 def test_result_overlapping_an_operand_is_refused():
     q = srt.current_queue()
