@@ -224,7 +224,7 @@ def main():
 class Bench:
     """The configurations, each as one prepared foreign call per step."""
 
-    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1", "few_tiles",
+    SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg4_dense_backward", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1", "few_tiles",
                  "fp16_4096", "fp32_4096")
 
     def __init__(self, srt, native, q):
@@ -299,6 +299,33 @@ class Bench:
             return {"name": "cfg4 Dense bf16 4096x4096x11008 +bias +relu", "call": call, "kernel": kernel,
                     "flops": 2.0 * 4096 * 4096 * 11008, "bytes": (4096 * 4096 + 4096 * 11008 * 2 + 11008) * 2,
                     "bound": "mfma", "dtype": "bf16", "steps": 100}
+        if name == "cfg4_dense_backward":
+            # the whole pullback of config 4 (MathDerivatives.swift:460-482, :520-554): dz = dy * relu'(y) and dbias in one
+            # pass, then dx = dz . W^T and dW = x^T . dz -- three entry-point calls on one stream, timed end to end
+            g = rng(8)
+            x = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))
+            w = srt.Tensor(bf16_encode(g.standard_normal((4096, 11008), dtype=np.float32) / np.float32(64)))
+            y = srt.Tensor(bf16_encode(np.maximum(g.standard_normal((4096, 11008), dtype=np.float32), 0)))
+            dy = srt.Tensor(bf16_encode(g.standard_normal((4096, 11008), dtype=np.float32) / np.float32(64)))
+            dz = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+            db = srt.Tensor(shape=[11008], dtype=np.uint16)
+            dx = srt.Tensor(shape=[4096, 4096], dtype=np.uint16)
+            dw = srt.Tensor(shape=[4096, 11008], dtype=np.uint16)
+            for t in (y, dy, dz, db):
+                t.device_read(q)
+            dx_call, dx_kernel = self.prepared(dz, False, w, True, dx)
+            dw_call, dw_kernel = self.prepared(x, True, dz, False, dw)
+            relu = srt.ActivationType.relu
+
+            def call(i):
+                q.activation_backward(y, dy, relu, 0.0, dz, db)
+                dx_call(i)
+                dw_call(i)
+            e = 4096 * 11008 * 2
+            return {"name": "cfg4 Dense backward bf16, end to end: dz + dbias, dx = dz.W^T, dW = x^T.dz", "call": call,
+                    "kernel": f"activation_backward + {dx_kernel} + {dw_kernel}", "flops": 2 * 2.0 * 4096 * 4096 * 11008,
+                    "bytes": 3 * e + (e + e + 4096 * 4096 * 2) + (4096 * 4096 * 2 + e + e), "bound": "mfma", "dtype": "bf16",
+                    "steps": 40, "keep": (x, w, y, dy, dz, db, dx, dw)}
         if name.startswith("cfg5_m"):
             m = int(name[6:])
             g = rng(4)

@@ -40,8 +40,8 @@ struct SigmoidFast {
   static __device__ __forceinline__ float apply(float a, float) { return __fdividef(1.0f, 1.0f + __expf(-a)); }
 };
 struct TanhFast {
-  // 1 - 2 / (exp(2|a|) + 1) away from 0, a short series below 0.125 where that form cancels
-  // (at a = 1e-6 it is 6 % off, 15 rounding steps of a bfloat16)
+  // a quotient of two short polynomials, exact to a fraction of a 16-bit rounding step and uniformly so down to
+  // the smallest arguments (see activation16_ct)
   static __device__ __forceinline__ float apply(float a, float) { return srt::activation16_ct<srtActivationTanh>(0.0f, a); }
 };
 struct Copy { static __device__ __forceinline__ float apply(float a, float) { return a; } };
