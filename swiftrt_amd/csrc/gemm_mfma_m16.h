@@ -60,6 +60,8 @@ using ring::EPI_BIAS_RELU;
 using ring::EPI_CLIPPED;
 using ring::EPI_TRANS;
 constexpr int EPI_PARTIAL = 6;   // fp32 accumulators as they are, for a split-K pass (C is a float workspace)
+// bias, then sigmoid / tanh / elu applied in registers on the way to the staging area (store_tile; the 64-deep kernel):
+constexpr int EPI_SIGMOID = 7, EPI_TANH = 8, EPI_ELU = 9;
 
 #define SRT_FENCE() __builtin_amdgcn_sched_barrier(0)
 
@@ -253,8 +255,12 @@ __device__ __forceinline__ void load_bias(const GemmProblem& p, int wave_m0, int
 // sides: a write instruction covers 16 rows x 32 B, a read 4 whole rows).
 // NaN handling as in ring::store_tile: the hardware converter rounds everything, and when any
 // lane of the wave saw a NaN the staged patterns are rewritten to 0x7FFF on the way out.
-// Bias and the clamps (CLAMP 1: relu, 2: clipped relu) are applied to the copy that leaves the
-// accumulator registers, so the accumulators themselves are only read.
+// Bias and the activation (CLAMP 1: relu, 2: clipped relu, 3: sigmoid, 4: tanh, 5: elu) are applied to the copy that
+// leaves the accumulator registers, so the accumulators themselves are only read.  The transcendental ones are
+// straight-line code per value (activation16_ct: selects, no branches) -- 256 copies of a dozen instructions per
+// lane, fetched once per tile.  Against staging fp32 values and applying the activation in a rolled loop
+// (store_tile_transcendental) that saves the second trip through LDS, the scalar encoder and the 8-byte stores:
+// 4096 x 8192 x 4096 + bias + tanh 213-220 us that way, 181 plain.
 // FLIP: the accumulator of the tile in row group i, column group j of the result is acc[j][i] (the kernel computed
 // the transposed product with the operands' roles exchanged; each 16 x 16 tile lies in the registers as it does
 // otherwise).
@@ -306,13 +312,18 @@ __device__ __forceinline__ void store_tile(const GemmProblem& p, const f32x4_t (
           a2 += per_row ? br : T::to_float((S)(b[j].y & 0xffffu));
           a3 += per_row ? br : T::to_float((S)(b[j].y >> 16));
         }
-        if (CLAMP >= 1) {
+        if (CLAMP == 1 || CLAMP == 2) {
           a0 = __builtin_fmaxf(a0, 0.0f); a1 = __builtin_fmaxf(a1, 0.0f);
           a2 = __builtin_fmaxf(a2, 0.0f); a3 = __builtin_fmaxf(a3, 0.0f);
         }
         if (CLAMP == 2) {
           a0 = __builtin_fminf(a0, ceiling); a1 = __builtin_fminf(a1, ceiling);
           a2 = __builtin_fminf(a2, ceiling); a3 = __builtin_fminf(a3, ceiling);
+        }
+        if (CLAMP >= 3) {
+          constexpr int ACT = CLAMP == 3 ? srtActivationSigmoid : CLAMP == 4 ? srtActivationTanh : srtActivationElu;
+          a0 = activation16_ct<ACT>(ceiling, a0); a1 = activation16_ct<ACT>(ceiling, a1);
+          a2 = activation16_ct<ACT>(ceiling, a2); a3 = activation16_ct<ACT>(ceiling, a3);
         }
         if (FIXUP) nan |= __builtin_isunordered(a0, a1) | __builtin_isunordered(a2, a3);
         const u32x2_t w = {T::template pack2<false>(a0, a1), T::template pack2<false>(a2, a3)};

@@ -52,6 +52,9 @@ using m16::EPI_PARTIAL;
 using m16::EPI_PLAIN;
 using m16::EPI_RELU;
 using m16::EPI_TRANS;
+using m16::EPI_SIGMOID;
+using m16::EPI_TANH;
+using m16::EPI_ELU;
 using m16::mfma16;
 using m16::mfma16_first;
 using ring::BN;
@@ -370,8 +373,9 @@ constexpr int TAIL_MAX_PARTS = 3;
 // quarters full or less (see gemm_m16d_split_kernel).  B is staged as for the wide tile (a 256-wide unit).
 template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false, int TN = 8>
 __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailShare& ts) {
-  static_assert(!FLIP || (EPI != EPI_PARTIAL && EPI != EPI_TRANS), "flipped: the store_tile epilogues only");
-  static_assert(TN == 8 || (TN == 6 && !SK && !FLIP && EPI != EPI_PARTIAL && EPI != EPI_TRANS), "the narrow tile: plain form, store_tile epilogues");
+  static_assert(EPI != EPI_TRANS, "sigmoid / tanh / elu have epilogue kinds of their own here");
+  static_assert(!FLIP || EPI != EPI_PARTIAL, "flipped: the store_tile epilogues only");
+  static_assert(TN == 8 || (TN == 6 && !SK && !FLIP && EPI != EPI_PARTIAL), "the narrow tile: plain form, store_tile epilogues");
   constexpr int TM = 8;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
@@ -724,7 +728,8 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     GemmProblem pe = p;   // the problem as the epilogue sees it
     if (FLIP) { pe.M = p.N; pe.N = p.M; }
     const int le = lane_id();
-    constexpr bool LINEAR_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED;
+    constexpr bool LINEAR_BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU || EPI == EPI_CLIPPED || EPI == EPI_SIGMOID ||
+                                 EPI == EPI_TANH || EPI == EPI_ELU;
     u32x2_t bias_regs[8];
     if (LINEAR_BIAS) m16::load_bias<T, TM>(pe, em0, en0, le, bias_regs);   // lands during the wait below
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 7\n\ts_nop 7" ::: "memory");
@@ -808,14 +813,14 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
       }
     } else if constexpr (EPI == EPI_PARTIAL) {
       m16::store_tile_partial<TM>(p, acc, em0, en0, bz, le, stage);
-    } else if constexpr (EPI == EPI_TRANS) {
-      m16::load_bias<T, TM>(p, em0, en0, le, bias_regs);
-      m16::store_tile_transcendental<T, TM>(p, acc, em0, en0, bz, le, stage, bias_regs);
     } else {
       if (EPI == EPI_BIAS) m16::store_tile<T, TM, true, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
       else if (EPI == EPI_RELU) m16::store_tile<T, TM, false, 1, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
       else if (EPI == EPI_BIAS_RELU) m16::store_tile<T, TM, true, 1, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
       else if (EPI == EPI_CLIPPED) m16::store_tile<T, TM, true, 2, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else if (EPI == EPI_SIGMOID) m16::store_tile<T, TM, true, 3, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else if (EPI == EPI_TANH) m16::store_tile<T, TM, true, 4, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
+      else if (EPI == EPI_ELU) m16::store_tile<T, TM, true, 5, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
       else m16::store_tile<T, TM, false, 0, FLIP>(pe, acc, em0, en0, bz, le, stage, bias_regs, n_end);
     }
     if (!has_next) break;
@@ -1034,15 +1039,15 @@ hipError_t launch_tail(const GemmProblem& p, hipStream_t stream) {
 
 template <typename T, bool A_KC, bool B_KC>
 hipError_t launch(const GemmProblem& p, hipStream_t stream) {
-  const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh ||
-                     p.activation == srtActivationElu;
-  if (trans) return launch_kernel<T, A_KC, B_KC, EPI_TRANS>(p, stream);
   // x . W runs as (W^T . x^T)^T: the flipped problem has an m-contiguous A and a k-contiguous B.  Whatever qualifies
   // this way round qualifies flipped: the operands' reaches and alignments exchange places, an n-contiguous B's N is a
   // multiple of 8 as an m-contiguous A's M must be, and the result is addressed as before.
   constexpr bool FLIP = A_KC && !B_KC;
   constexpr bool KA = FLIP ? false : A_KC, KB = FLIP ? true : B_KC;
   const GemmProblem q = FLIP ? flipped(p) : p;
+  if (p.activation == srtActivationSigmoid) return launch_kernel<T, KA, KB, EPI_SIGMOID, FLIP>(q, stream);
+  if (p.activation == srtActivationTanh) return launch_kernel<T, KA, KB, EPI_TANH, FLIP>(q, stream);
+  if (p.activation == srtActivationElu) return launch_kernel<T, KA, KB, EPI_ELU, FLIP>(q, stream);
   if (p.activation == srtActivationClippedRelu) return launch_kernel<T, KA, KB, EPI_CLIPPED, FLIP>(q, stream);
   if (p.activation == srtActivationRelu) {
     if (p.bias) return launch_kernel<T, KA, KB, EPI_BIAS_RELU, FLIP>(q, stream);
