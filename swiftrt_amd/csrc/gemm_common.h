@@ -5,6 +5,8 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <chrono>
+#include <random>
 
 #include "../../include/srt_hip.h"
 #include "status.h"
@@ -227,6 +229,24 @@ inline int compute_units() {
     cached[device & 31].store(n, std::memory_order_relaxed);
   }
   return n;
+}
+
+// Flag values of kernels whose workgroups tell each other "my part is in memory" (the tail-sharing matmul): a 64-bit
+// launch counter that starts at a value drawn once per process.  The flags live in
+// memory that other kernels have written before (the allocator recycles blocks), so what they hold at launch
+// is arbitrary -- most likely the flags of an earlier launch of this kernel.  Those hold earlier values of the
+// counter, which this launch's value differs from by construction (2^64 launches apart at the earliest);
+// anything else -- other kernels' data, another process's flags in memory the driver handed over -- matches
+// with probability 2^-64 per flag.
+inline unsigned long long next_launch_epoch() {
+  static const unsigned long long start = [] {
+    std::random_device rd;
+    unsigned long long v = ((unsigned long long)rd() << 32) ^ (unsigned long long)rd();
+    v ^= (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9e3779b97f4a7c15ull;
+    return v;
+  }();
+  static std::atomic<unsigned long long> counter{0};
+  return start + ++counter;
 }
 
 // ---- launchers (one per kernel family), defined in the .hip files ------------------------

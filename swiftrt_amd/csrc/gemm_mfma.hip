@@ -93,6 +93,10 @@ SRT_M16DS_DECL(BF16)
 SRT_M16DS_DECL(F16)
 #undef SRT_M16DS_DECL
 bool m16d_split_fits_BF16_xx(const GemmProblem&);
+hipError_t launch_m16dh_BF16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dh_BF16_11(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dh_F16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dh_F16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_F16_10(const GemmProblem&, hipStream_t);
@@ -570,6 +574,12 @@ hipError_t launch_m16d_split(const GemmProblem& p, bool a_kc, bool b_kc, hipStre
   if (b_kc) return launch_m16d_split_F16_01(p, stream);
   return launch_m16d_split_F16_00(p, stream);
 }
+// the 128 x 256 half tile of the 64-deep kernel (k-contiguous A)
+template <typename T>
+hipError_t launch_m16dh(const GemmProblem& p, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) return b_kc ? launch_m16dh_BF16_11(p, stream) : launch_m16dh_BF16_10(p, stream);
+  return b_kc ? launch_m16dh_F16_11(p, stream) : launch_m16dh_F16_10(p, stream);
+}
 template <typename T>
 hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16h_BF16_11(p, stream) : launch_m16h_BF16_10(p, stream);
@@ -588,6 +598,7 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 9: return launch_m16d<T>(p, a_kc, b_kc, stream);
     case 10: return launch_m16d_tail<T>(p, a_kc, b_kc, stream);
     case 11: return launch_m16d_split<T>(p, a_kc, b_kc, stream);
+    case 12: return launch_m16dh<T>(p, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     case 7: return launch_any_layout<T, 128, 128>(p, stream);
     case 8: return launch_any_layout<T, 64, 64>(p, stream);
@@ -626,7 +637,7 @@ static int mfma_layout(const GemmProblem& p) {
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
 // 128 x 256 form for a k-contiguous A, 9: the 16x16x32 kernel with 64-deep staging units), or 0 when the
-// problem does not qualify for it.  10: tile 9's tail-sharing form.  11: its split form (a last round of 192-wide tiles).
+// problem does not qualify for it.  10: tile 9's tail-sharing form.  11: its split form (a last round of 192-wide tiles).  12: its 128 x 256 half tile (k-contiguous A).
 int mfma_config(const GemmProblem& p, int tile) {
   if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
     if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
@@ -634,16 +645,16 @@ int mfma_config(const GemmProblem& p, int tile) {
     return tile << 2;
   }
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || (tile > 6 && tile != 9 && tile != 10 && tile != 11)) return 0;
+  if (layout < 0 || tile < 1 || (tile > 6 && (tile < 9 || tile > 12))) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
-  if (tile == 9 && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
+  if ((tile == 9 || tile == 12) && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
   if (tile == 10) {   // left-over tiles to share, k in whole quads, no transcendental activation
     const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
     if (trans || !m16d_tail_fits_BF16_xx(p)) return 0;
   }
   // whole rounds of whole tiles and a last round that 192-wide tiles fill, no transcendental activation (pinned or tuned plans only)
   if (tile == 11 && !m16d_split_fits_BF16_xx(p)) return 0;
-  if (tile == 6 && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
+  if ((tile == 6 || tile == 12) && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
 }
@@ -730,7 +741,12 @@ int mfma_select(const GemmProblem& p) {
   const long long th_min = p.batch == 1 ? 72 : p.K >= 2048 ? 96 : (p.K >= 1024 && p.M < 512) ? 128 : 72;
   const bool one_round = th >= th_min && rounds_h == 1 && half_fill_ok && (p.batch == 1 || t256 < half_cus);
   const bool small_rows = p.M <= 128 && p.K <= 512 && th >= 72;
-  const bool half_nt = p.M > 64 && (one_round || small_rows);
+  // (x . W^T with a short k loop and whole tiles that leave a second or later round at most half full: twice the
+  // workgroups fill it better -- 3072 x 6144 x 512, 288 tiles: 25.4 us against 27.3 whole; 3072 x 6144 x 256: 18.7 against
+  // 20.7; 3072 x 6144 x 1024: 39.7 against 42.8.  Whole rounds stay whole: 4096 x 4096 x 512 19.8 us against 21.4)
+  const bool short_nt = p.K <= 1024 && p.K % 64 == 0 && p.K >= 256 && t256 > cus && t256 % cus != 0 && 2 * (t256 % cus) <= cus &&
+                        p.batch == 1 && half_fill_ok;
+  const bool half_nt = p.M > 64 && (one_round || small_rows || short_nt);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
@@ -759,7 +775,9 @@ int mfma_select(const GemmProblem& p) {
   // (x^T . W^T at K = 1024: a single matrix of 16-32 tiles is 6-10 % faster in 64 x 64 tiles -- 1024 x 2048 x 1024 20.9 us
   // against 22.8 --, a batch, whose tiles share no operand, in whole ones from 16: 16 x 256 x 256 x 1024 21.9 against 24.3)
   const long long ring_from = layout == 3 ? 96
-                            : layout == 0 ? (p.K >= 1024 ? 1 : p.K >= 512 ? 8 : 64)   // (312 x 6136 x 80, 48 tiles: 9.9 us against 8.7)
+                            // (312 x 6136 x 80, 48 tiles: 9.9 us against 8.7; at K = 256 the 64-deep kernel is ahead from 36 tiles:
+                            // 1536 x 1536 x 256 11.3 us against 12.1, 1024 x 3072 x 256 11.5 against 12.6)
+                            : layout == 0 ? (p.K >= 1024 ? 1 : p.K >= 512 ? 8 : p.K >= 256 ? 32 : 64)
                             : p.K < 1024 ? 32 : layout == 1 ? (p.batch > 1 ? 16 : 40) : 24;
   //  * the 64-deep form of the 16x16x32 kernel (whole-line loads of k-contiguous operands, one barrier per 128
   //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
@@ -781,7 +799,9 @@ int mfma_select(const GemmProblem& p) {
   const int m_rest = p.M % 256;
   const bool padded_nt = layout == 3 && m_rest >= 1 && m_rest <= 128 && p.M < 1024 && t256 >= half_cus;
   int tile;
-  if (big_ok && (layout & 2) != 0 && half_ok) tile = 6;
+  // (half tiles in their 64-deep form whenever K allows: never behind the 32-deep one, 2-5 % ahead for x . W -- 2048^3 26.1 ->
+  // 24.9 us -- and 10-17 % for x . W^T, whose loads then move whole lines: 2048 x 4096 x 2048 34.1 -> 28.2 us)
+  if (big_ok && (layout & 2) != 0 && half_ok) tile = deep_ok ? 12 : 6;
   else if (whole_ok && padded_nt) tile = 4;
   else if (small_tt) tile = 3;
   else if (whole_ok && deep_ok && (t256 >= half_cus || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
@@ -968,6 +988,11 @@ bool mfma_prefers_tail(const GemmProblem& p) {
   if (left < 64 && (p.M < 512 || (p.K > 4096 && p.batch == 1))) return false;
   // x . W has half tiles to fall back on: while they fit one round they are as good or better below K = 8192 from 72 tiles
   // up (1536 x 3072 x 4096: 46-53 us in half tiles, 53 shared; 2048 x 3072 x 4096: 48-52 against 51-55)
+  // so has x . W^T since its half tiles are 64 deep (whole-line loads): one round of them beats the shared tiles below
+  // K = 8192 (1024 x 8192 x 4096: 52.6 us against 57.6; 1536 x 4096 x 4096: 44.9 against 48.5; 2048 x 3072 x 4096: 44.0
+  // against 48.7)
+  // (from five eighths of a round of them: at half a round the shared tiles are as good or better -- 512 x 8192 x 4096 41.5 us)
+  if (layout == 3 && 8 * th >= 5 * cus && th <= cus && p.K < 8192) return false;
   if (left <= (layout == 2 ? 64 : 96)) return true;
   return layout == 3 || (layout & 2) == 0 || p.K >= 8192 || th > cus;
 }
@@ -1026,6 +1051,7 @@ const char* mfma_name(int config) {
     case 9: return "mfma_256x256_m16_k64";
     case 10: return "mfma_256x256_m16_k64_tail";
     case 11: return "mfma_256x256_m16_k64_split";
+    case 12: return "mfma_128x256_m16_k64";
     case 2: return "mfma_128x128";
     case 7: return "mfma_128x128_any";
     case 8: return "mfma_64x64_any";

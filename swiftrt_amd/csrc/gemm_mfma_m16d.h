@@ -37,9 +37,6 @@
 // compute units without work in the last round: the tiles left over after the whole rounds are cut along k
 // and all workgroups share them; see gemm_m16d_body.
 #pragma once
-#include <chrono>
-#include <random>
-
 #include "gemm_mfma_m16.h"
 
 namespace srt {
@@ -85,25 +82,27 @@ __device__ __forceinline__ uint32_t select_lt(int a, int b, uint32_t t, uint32_t
 // A request is described by up to four scalar offsets so[j] (the unit's first byte in the operand plus
 // j steps, or OOB); load i takes lane offset voff[vindex(i)], scalar offset so[sindex(i)] and lands
 // landing(i) bytes into the wave's share of the slot.
-template <bool KC>
+// NL: loads per wave and unit -- 8 for a 256-wide unit, 4 for the 128-row k-contiguous A unit of the half tile.
+template <bool KC, int NL = 8>
 struct Loader {
+  static_assert(NL == 8 || (KC && NL == 4), "an mn-contiguous unit is 256 wide");
   uint32_t voff[KC ? 2 : 4];
-  static constexpr int SOFFS = KC ? 4 : 2;
+  static constexpr int SOFFS = KC ? NL / 2 : 2;
   static constexpr int vindex(int i) { return KC ? (i & 1) : (i & 3); }
   static constexpr int sindex(int i) { return KC ? (i >> 1) : (i >> 2); }
   static constexpr uint32_t landing(int i) { return KC ? (uint32_t)i * 1024u : (uint32_t)(i >> 2) * 16384u + (uint32_t)(i & 3) * 1024u; }
-  static __device__ __forceinline__ uint32_t wave_share(int wave) { return (uint32_t)wave * (KC ? 8192u : 4096u); }
+  static __device__ __forceinline__ uint32_t wave_share(int wave) { return (uint32_t)wave * (KC ? NL * 1024u : 4096u); }
   // bytes between so[j] and so[j + 1]: 16 rows (KC) or 32 k rows (MN)
   static __device__ __forceinline__ uint32_t step(long long ld) { return (uint32_t)((KC ? 16 : 32) * ld * 2); }
 
   // ld: elements between rows (KC) or between k (MN)
   __device__ __forceinline__ void init(int wave, int lane, long long ld) {
     if constexpr (KC) {
-      // load i covers rows (8 wave + i) 8 .. + 7, 8 lanes per 128-byte row; (row >> 1) & 7 depends on the
+      // load i covers rows (NL wave + i) 8 .. + 7, 8 lanes per 128-byte row; (row >> 1) & 7 depends on the
       // lane and the parity of i only, so loads i and i + 2 differ by 16 rows in the scalar offset
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const int row = (wave * 8 + i) * 8 + (lane >> 3);
+        const int row = (wave * NL + i) * 8 + (lane >> 3);
         const int chunk = (lane & 7) ^ ((row >> 1) & 7);
         voff[i] = (uint32_t)(((long long)row * ld + chunk * 8) * 2);
       }
@@ -146,18 +145,45 @@ struct FragReader<false> {
   }
 };
 
-// ---- the schedule's slots for a wave tile of TN column tiles (a phase is 4 TN MFMAs, u = 4 j + i) -----------------
-// TN = 8 is the schedule as described above.  TN = 6 (the 192-wide workgroup tile: 24 MFMAs per phase) keeps the order
-// of events and moves them to earlier slots: the A loads ride on MFMAs 8, 12, 16, 20 of phases 0 and 1, the eight B
-// loads on every third MFMA of phase 3, and the scalar bookkeeping goes where the table below says.
-template <int TN> constexpr int a_load_at(int u) {   // index 0..3 of the A load riding on MFMA u (phases 0, 1), or -1
+// ---- the schedule's slots for a wave tile of TM x TN MFMA tiles (a phase is TM / 2 x TN MFMAs, u = TM / 2 j + i) ---------
+// (TM, TN) = (8, 8) is the schedule as described above.  (8, 6) -- the 192-wide workgroup tile, 24 MFMAs per phase -- and
+// (4, 8) -- the 128 x 256 half tile, 16 MFMAs per phase, two A loads per phase -- keep the order of events and move them to
+// earlier slots.  Every function gives, for MFMA u of a phase, the index of the thing that rides behind it, or -1.
+template <int TM, int TN> constexpr int a_load_at(int u) {   // A load of the phase's share (phases 0, 1)
+  if (TM == 4) return u == 12 ? 0 : u == 14 ? 1 : -1;
   return (u >= 4 * TN - 16 && (u & 3) == 0) ? (u - (4 * TN - 16)) >> 2 : -1;
 }
-template <int TN> constexpr int b_load_at(int u) {   // index 0..7 of the B load riding on MFMA u (phase 3), or -1
+template <int TM, int TN> constexpr int b_load_at(int u) {   // B load 0..7 (phase 3)
+  if (TM == 4) return (u & 1) == 0 ? u >> 1 : -1;
   return TN == 8 ? ((u & 3) == 0 ? u >> 2 : -1) : ((u % 3 == 0 && u < 24) ? u / 3 : -1);
 }
-// The slot of the TN = 8 schedule whose scalar bookkeeping happens behind MFMA u of phase PH (-1: none)
-template <int TN, int PH> constexpr int event_at(int u) {
+// fragment reads of a phase that multiplies the first half of the A tiles (the rest of its own k half) ...
+template <int TM, int TN> constexpr int own_b_read_at(int u) {   // B tiles 4 .. TN - 1
+  if (TM == 4) return u < 4 ? 4 + u : -1;
+  return (u < 8 && (u & 1) == 0 && 4 + (u >> 1) < TN) ? 4 + (u >> 1) : -1;
+}
+template <int TM> constexpr int own_a_read_at(int u) {           // A tiles TM / 2 .. TM - 1
+  if (TM == 4) return (u == 4 || u == 5) ? 2 + (u - 4) : -1;
+  return (u >= 8 && u < 16 && (u & 1) == 0) ? 4 + ((u - 8) >> 1) : -1;
+}
+// ... and of one that multiplies the second half (tiles of the next k half: A 0 .. TM / 2 - 1, idle by now, and B 0-3,
+// each right behind its last MFMA)
+template <int TM> constexpr int next_a_read_at(int u) {
+  if (TM == 4) return (u == 0 || u == 2) ? u >> 1 : -1;
+  return (u < 16 && (u & 3) == 1) ? u >> 2 : -1;
+}
+template <int TM> constexpr int next_b_read_at(int u) {
+  if (TM == 4) return (u < 8 && (u & 1) == 1) ? u >> 1 : -1;
+  return (u < 16 && (u & 3) == 3) ? u >> 2 : -1;
+}
+// The slot of the (8, 8) schedule whose scalar bookkeeping happens behind MFMA u of phase PH
+template <int TM, int TN, int PH> constexpr int event_at(int u) {
+  if (TM == 4) {
+    if (PH == 0) return (u >= 5 && u <= 11) ? 2 * (u - 5) + 1 : -1;             // 1, 3, .. 13 -> 5 .. 11 (loads at 12, 14)
+    if (PH == 1) return u == 8 ? 10 : u == 10 ? 14 : -1;                         // 10, 14 -> 8, 10 (2 and 6: no third and fourth offset)
+    if (PH == 2) return (u >= 7 && (u & 1) == 1) ? 17 + (u - 7) : -1;            // 17 .. 25 -> 7 .. 15
+    return u == 9 ? 18 : u == 11 ? 22 : u == 13 ? 26 : -1;                       // 18, 22, 26 -> 9, 11, 13
+  }
   if (TN == 8) return u;
   if (PH == 0) return u < 7 ? 2 * u + 1 : -1;                      // 1, 3, .. 13 -> 0 .. 6 (ahead of the loads from 8 on)
   if (PH == 1) return u;                                           // 2, 6, 10, 14
@@ -371,12 +397,18 @@ constexpr int TAIL_MAX_PARTS = 3;
 // whose valid width p.tile_n <= 192 is a multiple of 8 -- tiles lie p.tile_n columns apart and columns beyond that
 // width are computed and not stored.  It fills a last round of the persistent grid that whole tiles would leave three
 // quarters full or less (see gemm_m16d_split_kernel).  B is staged as for the wide tile (a 256-wide unit).
-template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false, int TN = 8>
+// TM: row tiles per wave.  8: 256 rows per workgroup tile.  4: the 128 x 256 half tile (waves of 64 x 128) for problems that
+// leave compute units idle with whole tiles; its A unit is 128 rows of a k-contiguous A (in a slot of the same size).
+template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false, int TN = 8, int TM = 8>
 __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailShare& ts) {
   static_assert(EPI != EPI_TRANS, "sigmoid / tanh / elu have epilogue kinds of their own here");
   static_assert(!FLIP || EPI != EPI_PARTIAL, "flipped: the store_tile epilogues only");
   static_assert(TN == 8 || (TN == 6 && !SK && !FLIP && EPI != EPI_PARTIAL), "the narrow tile: plain form, store_tile epilogues");
-  constexpr int TM = 8;
+  static_assert(TM == 8 || (TM == 4 && TN == 8 && A_KC && !SK && !FLIP && EPI != EPI_PARTIAL), "the half tile: k-contiguous A, plain form");
+  constexpr int HALF = TM / 2;        // A tiles per phase
+  constexpr int TILE_M = 32 * TM;     // rows of a workgroup tile
+  constexpr int NLA = TM;             // A loads per wave and unit
+  using LoaderA = Loader<A_KC, NLA>;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
   const uint32_t lds = (uint32_t)(uintptr_t)(SRT_LDS unsigned char*)lds_raw;
   const uint32_t lds_end = lds + UNITS * UNIT;
@@ -387,10 +419,10 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
     asm volatile("" : "+s"(zero));   // opaque: keeps the two instructions where they are written
     return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
   };
-  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * (16 * TN);
+  const int wm0 = (wave >> 1) * (16 * TM), wn0 = (wave & 1) * (16 * TN);
 
   const int tile_w = TN == 8 ? BN : p.tile_n;   // columns between neighbouring tiles
-  const int tiles_m = (p.M + 255) / 256, tiles_n = (p.N + tile_w - 1) / tile_w;
+  const int tiles_m = (p.M + TILE_M - 1) / TILE_M, tiles_n = (p.N + tile_w - 1) / tile_w;
   const int total = tiles_m * tiles_n * p.batch;
   const int grid = (int)gridDim.x;
   int v = (int)blockIdx.x;
@@ -403,7 +435,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   const u32x4_t rb = ring::make_rsrc(p.B, (uint32_t)(((long long)(p.batch - 1) * p.sbb + b_view) * 2));
   // tile number -> position and operand offsets (the narrow tile's columns lie tile_w apart)
   auto locate = [&](int tile) {
-    TileRef t = m16::locate_tile<A_KC, B_KC, 256>(p, tile, tiles_m, tiles_n);
+    TileRef t = m16::locate_tile<A_KC, B_KC, TILE_M>(p, tile, tiles_m, tiles_n);
     if constexpr (TN != 8) {
       t.n0 = (t.n0 / BN) * tile_w;
       t.offb = (uint32_t)(((long long)t.bz * p.sbb + (B_KC ? (long long)t.n0 * ldb : (long long)t.n0)) * 2);
@@ -412,7 +444,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   };
   const uint32_t kstep_a = A_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * lda * 2);   // bytes per super-stage
   const uint32_t kstep_b = B_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * ldb * 2);
-  const uint32_t lstep_a = Loader<A_KC>::step(lda), lstep_b = Loader<B_KC>::step(ldb);
+  const uint32_t lstep_a = LoaderA::step(lda), lstep_b = Loader<B_KC>::step(ldb);
   const int S_full = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least four)
 
   // per-XCD start of the k walk for an A stored k x m (see gemm_ring_kernel)
@@ -506,11 +538,11 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   }
 
   // the eight loads of one unit, outside the main loop (first fill, and B_1 after an epilogue)
-  auto issue_a = [&](const Loader<A_KC>& l, uint32_t slot, uint32_t base) {
+  auto issue_a = [&](const LoaderA& l, uint32_t slot, uint32_t base) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      ring::load_to_lds(ra, slot + Loader<A_KC>::wave_share(wave) + Loader<A_KC>::landing(i),
-                        l.voff[Loader<A_KC>::vindex(i)], base + (uint32_t)Loader<A_KC>::sindex(i) * lstep_a);
+    for (int i = 0; i < NLA; ++i)
+      ring::load_to_lds(ra, slot + LoaderA::wave_share(wave) + LoaderA::landing(i),
+                        l.voff[LoaderA::vindex(i)], base + (uint32_t)LoaderA::sindex(i) * lstep_a);
   };
   auto issue_b = [&](const Loader<B_KC>& l, uint32_t slot, uint32_t base) {
 #pragma unroll
@@ -524,7 +556,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   bool first_tile = true;
   for (;;) {
     // per-lane addressing state, derived per tile and scoped to it (see gemm_ring_kernel)
-    Loader<A_KC> la;
+    LoaderA la;
     Loader<B_KC> lb;
     FragReader<A_KC> fa;
     FragReader<B_KC> fb;
@@ -539,7 +571,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
       issue_b(lb, xb, cur_tile.offb + (uint32_t)stage_of(0) * kstep_b);
       issue_a(la, xa1, cur_tile.offa + (uint32_t)stage_of(1) * kstep_a);
       issue_b(lb, xb1, cur_tile.offb + (uint32_t)stage_of(1) * kstep_b);
-      asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "i"(NLA + 8) : "memory");
     } else {
       issue_b(lb, xb1, cur_tile.offb + (uint32_t)stage_of(1) * kstep_b);
     }
@@ -572,7 +604,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
 #pragma unroll
     for (int t = 0; t < 4; ++t) bf[t] = fb.template read<0>(xb, t);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) af[t] = fa.template read<0>(x, t);
+    for (int t = 0; t < HALF; ++t) af[t] = fa.template read<0>(x, t);
 
     int e_req = stage_of(2);   // k index of request s + 2
     uint32_t ea_off = (uint32_t)e_req * kstep_a, eb_off = (uint32_t)e_req * kstep_b;
@@ -598,11 +630,11 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int u = 4 * j + i;
+        for (int i = 0; i < HALF; ++i) {
+          const int u = HALF * j + i;
           // which load, if any, rides on this MFMA
-          const int ld = LOADS == 3 ? b_load_at<TN>(u)
-                       : (LOADS == 1 || LOADS == 2) ? (a_load_at<TN>(u) >= 0 ? a_load_at<TN>(u) + (LOADS == 2 ? 4 : 0) : -1)
+          const int ld = LOADS == 3 ? b_load_at<TM, TN>(u)
+                       : (LOADS == 1 || LOADS == 2) ? (a_load_at<TM, TN>(u) >= 0 ? a_load_at<TM, TN>(u) + (LOADS == 2 ? NLA / 2 : 0) : -1)
                        : -1;
           if (ld >= 0) {
             if (LOADS == 3) {
@@ -618,9 +650,9 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
               if (ld == 6) set_target(std::integral_constant<uint32_t, imm[6]>{}, target);
               if (ld == 7) set_target(std::integral_constant<uint32_t, imm[7]>{}, target);
             } else {
-              constexpr uint32_t imm[8] = {Loader<A_KC>::landing(0), Loader<A_KC>::landing(1), Loader<A_KC>::landing(2),
-                                           Loader<A_KC>::landing(3), Loader<A_KC>::landing(4), Loader<A_KC>::landing(5),
-                                           Loader<A_KC>::landing(6), Loader<A_KC>::landing(7)};
+              constexpr uint32_t imm[8] = {LoaderA::landing(0), LoaderA::landing(1), LoaderA::landing(2),
+                                           LoaderA::landing(3), LoaderA::landing(4), LoaderA::landing(5),
+                                           LoaderA::landing(6), LoaderA::landing(7)};
               if (ld == 0) set_target(std::integral_constant<uint32_t, imm[0]>{}, target);
               if (ld == 1) set_target(std::integral_constant<uint32_t, imm[1]>{}, target);
               if (ld == 2) set_target(std::integral_constant<uint32_t, imm[2]>{}, target);
@@ -633,27 +665,27 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
             SRT_FENCE();
           }
           if constexpr (FLIP) {   // A fragment first: the tile comes out as the transposed product's
-            if constexpr (FIRST) mfma16_first<T>(acc[4 * AH + i][j], af[4 * AH + i], bf[j]);
-            else mfma16<T>(acc[4 * AH + i][j], af[4 * AH + i], bf[j]);
+            if constexpr (FIRST) mfma16_first<T>(acc[HALF * AH + i][j], af[HALF * AH + i], bf[j]);
+            else mfma16<T>(acc[HALF * AH + i][j], af[HALF * AH + i], bf[j]);
           } else {
-            if constexpr (FIRST) mfma16_first<T>(acc[4 * AH + i][j], bf[j], af[4 * AH + i]);
-            else mfma16<T>(acc[4 * AH + i][j], bf[j], af[4 * AH + i]);
+            if constexpr (FIRST) mfma16_first<T>(acc[HALF * AH + i][j], bf[j], af[HALF * AH + i]);
+            else mfma16<T>(acc[HALF * AH + i][j], bf[j], af[HALF * AH + i]);
           }
           if (ld >= 0) {
             SRT_FENCE();
-            const int si = LOADS == 3 ? Loader<B_KC>::sindex(ld) : Loader<A_KC>::sindex(ld);
+            const int si = LOADS == 3 ? Loader<B_KC>::sindex(ld) : LoaderA::sindex(ld);
             const uint32_t so = si == 0 ? so0 : si == 1 ? so1 : si == 2 ? so2 : so3;
             if (LOADS == 3) ring::load_to_lds_at_m0(rb, lb.voff[Loader<B_KC>::vindex(ld)], so);
-            else ring::load_to_lds_at_m0(ra, la.voff[Loader<A_KC>::vindex(ld)], so);
+            else ring::load_to_lds_at_m0(ra, la.voff[LoaderA::vindex(ld)], so);
           }
           if (OWN) {
-            if (u < 8 && (u & 1) == 0 && 4 + (u >> 1) < TN) bf[4 + (u >> 1)] = fb.template read<H>(ub, 4 + (u >> 1));
-            if (u >= 8 && u < 16 && (u & 1) == 0) af[4 + ((u - 8) >> 1)] = fa.template read<H>(ua, 4 + ((u - 8) >> 1));
+            if (own_b_read_at<TM, TN>(u) >= 0) bf[own_b_read_at<TM, TN>(u)] = fb.template read<H>(ub, own_b_read_at<TM, TN>(u));
+            if (own_a_read_at<TM>(u) >= 0) af[own_a_read_at<TM>(u)] = fa.template read<H>(ua, own_a_read_at<TM>(u));
           } else {
-            if (u < 16 && (u & 3) == 1) af[u >> 2] = fa.template read<H>(ua, u >> 2);
-            if (u < 16 && (u & 3) == 3) bf[u >> 2] = fb.template read<H>(ub, u >> 2);
+            if (next_a_read_at<TM>(u) >= 0) af[next_a_read_at<TM>(u)] = fa.template read<H>(ua, next_a_read_at<TM>(u));
+            if (next_b_read_at<TM>(u) >= 0) bf[next_b_read_at<TM>(u)] = fb.template read<H>(ub, next_b_read_at<TM>(u));
           }
-          ev(event_at<TN, PH>(u));
+          ev(event_at<TM, TN, PH>(u));
           SRT_FENCE();
         }
       }
@@ -673,13 +705,13 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
         if (u == 3) xa2 = select_lt((int)xa2, (int)lds_end, xa2, xa2 - UNITS * UNIT);
         if (u == 5) sel = select_lt(r, S, cur_tile.offa, next_tile.offa);
         if (u == 7) soa = select_lt(r, limit_a, sel + ea_off, OOB);
-        if (u == 9) ta = xa2 + Loader<A_KC>::wave_share(wave);
+        if (u == 9) ta = xa2 + LoaderA::wave_share(wave);
         if (u == 11) so_a0 = soa;
         if (u == 13) so_a1 = select_lt(r, limit_a, soa + lstep_a, OOB);
       });
       // ---- phase 1: k half 0, A tiles 4-7; loads 4-7 of A_{s+2}; reads of k half 1 ----
       phase(C1{}, first_tag, std::false_type{}, C1{}, C2{}, x, xb, ta, so_a0, so_a1, so_a2, so_a3, [&](int u) __attribute__((always_inline)) {
-        if (Loader<A_KC>::SOFFS == 4) {
+        if (LoaderA::SOFFS == 4) {
           if (u == 2) so_a2 = select_lt(r, limit_a, soa + 2 * lstep_a, OOB);
           if (u == 6) so_a3 = select_lt(r, limit_a, soa + 3 * lstep_a, OOB);
         }
@@ -697,7 +729,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
         if (u == 25) tb = x + Loader<B_KC>::wave_share(wave);
       });
       // ---- sync: all of super-stage s is in registers, A_{s+1} and B_{s+1} have landed ----
-      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "i"(NLA) : "memory");
       SRT_FENCE();
       // ---- phase 3: k half 1, A tiles 4-7; the loads of B_{s+2}; reads of super-stage s + 1 ----
       phase(C1{}, std::false_type{}, std::false_type{}, C0{}, C3{}, xa1, xb1, tb, so_b0, so_b1, so_b2, so_b3, [&](int u) __attribute__((always_inline)) {
@@ -843,6 +875,12 @@ __global__ __launch_bounds__(NT) void gemm_m16d_tail_kernel(GemmProblem p, TailS
   gemm_m16d_body<T, A_KC, B_KC, EPI, true, FLIP>(p, ts);
 }
 
+// The 128 x 256 half tile (k-contiguous A), for problems that leave compute units idle with whole tiles.
+template <typename T, bool B_KC, int EPI>
+__global__ __launch_bounds__(NT) void gemm_m16d_half_kernel(GemmProblem p) {
+  gemm_m16d_body<T, true, B_KC, EPI, false, false, 8, 4>(p, TailShare{});
+}
+
 // Two tile walks in one launch, for a tile count that leaves the last round of the persistent grid between half
 // and three quarters full (688 tiles on 256 units: 2.69 rounds, 3 paid).  The columns are cut in two: `wide` covers
 // the first columns in whole 256 x 256 tiles that fill whole rounds (it is the problem as the plain kernel would get
@@ -942,23 +980,6 @@ inline TailPlan tail_plan(const GemmProblem& p) {
 }
 inline bool tail_fits(const GemmProblem& p) { return tail_plan(p).parts != 0; }
 
-// Flag values: a 64-bit launch counter that starts at a value drawn once per process.  The flags live in
-// memory that other kernels have written before (the allocator recycles blocks), so what they hold at launch
-// is arbitrary -- most likely the flags of an earlier launch of this kernel.  Those hold earlier values of the
-// counter, which this launch's value differs from by construction (2^64 launches apart at the earliest);
-// anything else -- other kernels' data, another process's flags in memory the driver handed over -- matches
-// with probability 2^-64 per flag.
-inline unsigned long long next_tail_epoch() {
-  static const unsigned long long start = [] {
-    std::random_device rd;
-    unsigned long long v = ((unsigned long long)rd() << 32) ^ (unsigned long long)rd();
-    v ^= (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9e3779b97f4a7c15ull;
-    return v;
-  }();
-  static std::atomic<unsigned long long> counter{0};
-  return start + ++counter;
-}
-
 template <typename T, bool A_KC, bool B_KC, int EPI, bool FLIP = false>
 hipError_t launch_tail_kernel(const GemmProblem& p, hipStream_t stream) {
   auto kernel = gemm_m16d_tail_kernel<T, A_KC, B_KC, EPI, FLIP>;
@@ -981,7 +1002,7 @@ hipError_t launch_tail_kernel(const GemmProblem& p, hipStream_t stream) {
   ts.flags = reinterpret_cast<unsigned long long*>(workspace);
   ts.stored = reinterpret_cast<unsigned int*>(static_cast<unsigned char*>(workspace) + TAIL_STORED_OFFSET);
   ts.partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + TAIL_FLAG_BYTES);
-  ts.epoch = next_tail_epoch();
+  ts.epoch = next_launch_epoch();
 #ifdef SRT_DEBUG_LAUNCH
   if (srtMemsetAsync(ts.stored, 0, 256 * sizeof(unsigned int), reinterpret_cast<srtStream>(stream)) != srtSuccess) {
     (void)srtDeviceFree(workspace);
@@ -1055,6 +1076,33 @@ hipError_t launch(const GemmProblem& p, hipStream_t stream) {
   }
   if (p.bias) return launch_kernel<T, KA, KB, EPI_BIAS, FLIP>(q, stream);
   return launch_kernel<T, KA, KB, EPI_PLAIN, FLIP>(q, stream);
+}
+
+// ---- the half tile ------------------------------------------------------------------------------------------------
+template <typename T, bool B_KC, int EPI>
+hipError_t launch_half_kernel(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_m16d_half_kernel<T, B_KC, EPI>;
+  constexpr int lds_bytes = UNITS * UNIT;
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
+  const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + BN - 1) / BN) * p.batch;
+  const int grid = ring::persistent_grid(tiles);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, p);
+  return launch_status(stream);
+}
+
+template <typename T, bool B_KC>
+hipError_t launch_half(const GemmProblem& p, hipStream_t stream) {
+  if (p.activation == srtActivationSigmoid) return launch_half_kernel<T, B_KC, EPI_SIGMOID>(p, stream);
+  if (p.activation == srtActivationTanh) return launch_half_kernel<T, B_KC, EPI_TANH>(p, stream);
+  if (p.activation == srtActivationElu) return launch_half_kernel<T, B_KC, EPI_ELU>(p, stream);
+  if (p.activation == srtActivationClippedRelu) return launch_half_kernel<T, B_KC, EPI_CLIPPED>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_half_kernel<T, B_KC, EPI_BIAS_RELU>(p, stream);
+    return launch_half_kernel<T, B_KC, EPI_RELU>(p, stream);
+  }
+  if (p.bias) return launch_half_kernel<T, B_KC, EPI_BIAS>(p, stream);
+  return launch_half_kernel<T, B_KC, EPI_PLAIN>(p, stream);
 }
 
 // ---- the split form: whole rounds of whole tiles, then one round of narrow tiles (gemm_m16d_split_kernel) ----------

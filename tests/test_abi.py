@@ -201,7 +201,7 @@ def test_plan_cache_file_round_trip_and_rejects_malformed_files(tmp_path):
     srt.PlanCache.clear()
     assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
                                   buf, 64) == 0
-    assert buf.value == b"mfma_128x256_m16"
+    assert buf.value == b"mfma_128x256_m16_k64"
     assert L.srtPlanCacheCount(None) == native.ERROR_INVALID_VALUE
     assert L.srtPlanCacheLoad(None) == native.ERROR_INVALID_VALUE
 
@@ -237,8 +237,8 @@ def test_kernel_selection_is_queryable_without_gpu():
     # 64 to 160 tiles: the tail-sharing form of the 64-deep kernel (every tile cut along k into two or three parts),
     # unless half-height tiles fill one round as well
     assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_256x256_m16_k64_tail"
-    assert query(native.REAL16BF, 2048, 4096, 4096, tb=True) == "mfma_256x256_m16_k64_tail"
-    assert query(native.REAL16BF, 2048, 4096, 4096) == "mfma_128x256_m16"
+    assert query(native.REAL16BF, 2048, 4096, 4096, tb=True) == "mfma_128x256_m16_k64"
+    assert query(native.REAL16BF, 2048, 4096, 4096) == "mfma_128x256_m16_k64"
     assert query(native.REAL16BF, 2048, 4096, 8192) == "mfma_256x256_m16_k64_tail"
     assert query(native.REAL16BF, 4096, 10240, 4096) == "mfma_256x256_m16_k64"        # after whole rounds it buys nothing
     assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_256x256_m16_k64_tail"    # 64 tiles again
@@ -253,9 +253,9 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16_k64"             # 144 tiles, long k loop
     assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256_m16_k64"             # and a short one
     # a k-contiguous A and at most one round of 128 x 256 tiles: the half-height form of the 16x16x32 kernel
-    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16"             # 128 half tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16"
-    assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16"             # 256 half tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16_k64"             # 128 half tiles
+    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16_k64"
+    assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16_k64"             # 256 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x256_m16_k64_tail"   # A not k-contiguous: whole tiles cut along k
     assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x256_m16_k64"
     # 258 whole tiles: a whole round, and the two left over cut along k in three parts each
@@ -263,10 +263,10 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16_k64_tail"
     assert query(native.REAL16BF, 1536, 11008, 2048) == "mfma_256x256_m16_k64"        # (not for a k loop this short)
     assert query(native.REAL16BF, 1536, 4096, 11008, tb=True) == "mfma_256x256_m16_k64_tail"   # 96 tiles, two parts each
-    assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16"              # 8 half tiles
+    assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16_k64"              # 8 half tiles
     assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
-    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16"              # K too short to split
-    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_128x256_m16"               # short k loops too (8.4 us against 10.0)
+    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16_k64"              # K too short to split
+    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_128x256_m16_k64"               # short k loops too (8.4 us against 10.0)
     assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"
@@ -281,7 +281,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 32, 4096, 2048) == "skinny"
     assert query(native.REAL16BF, 32, 4096, 4096) == "mfma_256x256_splitk"            # 64 workgroups, 17..32 rows
     assert query(native.REAL16BF, 8, 4096, 8192) == "mfma_256x256_splitk"             # long k loop
-    assert query(native.REAL16BF, 8, 28672, 1024) == "mfma_128x256_m16"               # 448 workgroups: not one round
+    assert query(native.REAL16BF, 8, 28672, 1024) == "mfma_128x256_m16_k64"               # 448 workgroups: not one round
     assert query(native.REAL16BF, 64, 14336, 4096) == "skinny"
     assert query(native.REAL16BF, 64, 11008, 4096) == "mfma_256x256_splitk"
     # what sweeps against every pinned plan found (the measured pairs stand next to the rules in csrc/gemm_mfma.hip)
@@ -307,7 +307,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query_batched(native.REAL16BF, 4, 256, 256, 4096, ta=True) == "mfma_256x256_m16_k64_tail"   # four tiles cut along k
     assert query_batched(native.REAL16BF, 16, 256, 256, 2048, ta=True, tb=True) == "mfma_256x256_m16_k64_tail"
     assert query_batched(native.REAL16BF, 4, 128, 128, 4096, tb=True) == "mfma_64x64"                  # mostly padding, both k-contiguous
-    assert query_batched(native.REAL16BF, 64, 256, 256, 1024, tb=True) == "mfma_128x256_m16"           # 128 half tiles in one round
+    assert query_batched(native.REAL16BF, 64, 256, 256, 1024, tb=True) == "mfma_128x256_m16_k64"           # 128 half tiles in one round
     assert query_batched(native.REAL16BF, 64, 256, 1024, 256, tb=True) == "mfma_256x256_m16_k64"       # 512 half tiles: whole tiles
     assert query_batched(native.REAL16BF, 64, 384, 384, 4096, tb=True) == "mfma_256x256_k64"           # a last row of tiles half padding
     assert query_batched(native.REAL16BF, 28, 8, 88, 7680) == "skinny"                                 # ahead of sharing padded tiles
@@ -337,7 +337,7 @@ def test_kernel_selection_answers_for_any_problem():
     buf = ctypes.create_string_buffer(64)
     known = {"empty", "generic", "skinny", "f32_mfma", "mfma_256x256", "mfma_128x128", "mfma_64x64", "mfma_256x256_k64",
              "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128_any", "mfma_64x64_any",
-             "mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split"}
+             "mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split", "mfma_128x256_m16_k64"}
 
     def logu(lo, hi):
         return int(np.exp(g.uniform(np.log(lo), np.log(hi))))

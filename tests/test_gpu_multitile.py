@@ -116,6 +116,7 @@ def plans_for(ta, tb):
         plans.append("mfma_256x256_k64")    # two k-contiguous operands
     if not ta:
         plans.append("mfma_128x256_m16")    # k-contiguous A
+        plans.append("mfma_128x256_m16_k64")
     return plans
 
 
