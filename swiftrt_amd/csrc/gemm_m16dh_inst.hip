@@ -12,4 +12,11 @@ hipError_t SRT_CAT(launch_m16dh, SRT_M16_TYPE, SRT_M16_BKC)(const GemmProblem& p
   return m16d::launch_half<SRT_M16_TYPE, SRT_M16_BKC != 0>(p, stream);
 }
 
+// launch_m16dh_partial_<type>_11: the split-K pass (used for a k-contiguous B only)
+#if SRT_M16_BKC
+hipError_t SRT_CAT(launch_m16dh_partial, SRT_M16_TYPE, SRT_M16_BKC)(const GemmProblem& p, hipStream_t stream) {
+  return m16d::launch_half_partial<SRT_M16_TYPE, true>(p, stream);
+}
+#endif
+
 }  // namespace srt

@@ -404,7 +404,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
   static_assert(EPI != EPI_TRANS, "sigmoid / tanh / elu have epilogue kinds of their own here");
   static_assert(!FLIP || EPI != EPI_PARTIAL, "flipped: the store_tile epilogues only");
   static_assert(TN == 8 || (TN == 6 && !SK && !FLIP && EPI != EPI_PARTIAL), "the narrow tile: plain form, store_tile epilogues");
-  static_assert(TM == 8 || (TM == 4 && TN == 8 && A_KC && !SK && !FLIP && EPI != EPI_PARTIAL), "the half tile: k-contiguous A, plain form");
+  static_assert(TM == 8 || (TM == 4 && TN == 8 && A_KC && !SK && !FLIP), "the half tile: k-contiguous A, plain form");
   constexpr int HALF = TM / 2;        // A tiles per phase
   constexpr int TILE_M = 32 * TM;     // rows of a workgroup tile
   constexpr int NLA = TM;             // A loads per wave and unit
@@ -1103,6 +1103,12 @@ hipError_t launch_half(const GemmProblem& p, hipStream_t stream) {
   }
   if (p.bias) return launch_half_kernel<T, B_KC, EPI_BIAS>(p, stream);
   return launch_half_kernel<T, B_KC, EPI_PLAIN>(p, stream);
+}
+
+// The split-K pass on half tiles (a k-contiguous A of at most 128 rows): fp32 accumulators to a workspace.
+template <typename T, bool B_KC>
+hipError_t launch_half_partial(const GemmProblem& p, hipStream_t stream) {
+  return launch_half_kernel<T, B_KC, EPI_PARTIAL>(p, stream);
 }
 
 // ---- the split form: whole rounds of whole tiles, then one round of narrow tiles (gemm_m16d_split_kernel) ----------
