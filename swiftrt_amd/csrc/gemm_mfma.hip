@@ -97,6 +97,10 @@ hipError_t launch_m16dh_BF16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_F16_10(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_F16_11(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dn_BF16_00(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dn_BF16_01(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dn_F16_00(const GemmProblem&, hipStream_t);
+hipError_t launch_m16dn_F16_01(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_partial_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_partial_F16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
@@ -582,6 +586,12 @@ hipError_t launch_m16dh(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16dh_BF16_11(p, stream) : launch_m16dh_BF16_10(p, stream);
   return b_kc ? launch_m16dh_F16_11(p, stream) : launch_m16dh_F16_10(p, stream);
 }
+// the 256 x 128 half tile of the 64-deep kernel (A not k-contiguous)
+template <typename T>
+hipError_t launch_m16dn(const GemmProblem& p, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) return b_kc ? launch_m16dn_BF16_01(p, stream) : launch_m16dn_BF16_00(p, stream);
+  return b_kc ? launch_m16dn_F16_01(p, stream) : launch_m16dn_F16_00(p, stream);
+}
 template <typename T>
 hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16h_BF16_11(p, stream) : launch_m16h_BF16_10(p, stream);
@@ -601,6 +611,7 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 10: return launch_m16d_tail<T>(p, a_kc, b_kc, stream);
     case 11: return launch_m16d_split<T>(p, a_kc, b_kc, stream);
     case 12: return launch_m16dh<T>(p, b_kc, stream);
+    case 13: return launch_m16dn<T>(p, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     case 7: return launch_any_layout<T, 128, 128>(p, stream);
     case 8: return launch_any_layout<T, 64, 64>(p, stream);
@@ -639,7 +650,7 @@ static int mfma_layout(const GemmProblem& p) {
 // Configuration for a given tile (1: 256 x 256 ring, 2: 128 x 128, 3: 64 x 64, 4: 256 x 256 with
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
 // 128 x 256 form for a k-contiguous A, 9: the 16x16x32 kernel with 64-deep staging units), or 0 when the
-// problem does not qualify for it.  10: tile 9's tail-sharing form.  11: its split form (a last round of 192-wide tiles).  12: its 128 x 256 half tile (k-contiguous A).
+// problem does not qualify for it.  10: tile 9's tail-sharing form.  11: its split form (a last round of 192-wide tiles).  12: its 128 x 256 half tile (k-contiguous A).  13: its 256 x 128 half tile (A not k-contiguous).
 int mfma_config(const GemmProblem& p, int tile) {
   if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
     if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
@@ -647,9 +658,9 @@ int mfma_config(const GemmProblem& p, int tile) {
     return tile << 2;
   }
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || (tile > 6 && (tile < 9 || tile > 12))) return 0;
+  if (layout < 0 || tile < 1 || (tile > 6 && (tile < 9 || tile > 13))) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
-  if ((tile == 9 || tile == 12) && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
+  if ((tile == 9 || tile == 12 || tile == 13) && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
   if (tile == 10) {   // left-over tiles to share, k in whole quads, no transcendental activation
     const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
     if (trans || !m16d_tail_fits_BF16_xx(p)) return 0;
@@ -657,8 +668,30 @@ int mfma_config(const GemmProblem& p, int tile) {
   // whole rounds of whole tiles and a last round that 192-wide tiles fill, no transcendental activation (pinned or tuned plans only)
   if (tile == 11 && !m16d_split_fits_BF16_xx(p)) return 0;
   if ((tile == 6 || tile == 12) && (layout & 2) == 0) return 0;   // the 128-row A region is k-contiguous
+  if (tile == 13 && (layout & 2) != 0) return 0;                  // the 256 x 128 half tile is for the other A layouts
   if (tile == 4 && layout != 3) return 0;   // the 64-deep kernel takes two k-contiguous operands only
   return (tile << 2) | layout;
+}
+
+int mfma_splitk_parts(const GemmProblem& p);
+
+// Whether the 256 x 128 half tile of an A that is not k-contiguous is the choice: when one round of them holds the problem
+// (whole tiles would leave half of those compute units idle) and the k loop is short enough that cutting it does not do better.
+//   K <= 1024       always: 512 x 512 x 512 x^T . W 10.7 us against 15.2 for 64 x 64 tiles, 512 x 2048 x 1024 15.9 against 22.6
+//                   whole, 512 x 512 x 1024 15.8 against 20.4 for split-K; x^T . W^T 1024 x 1024 x 1024 15.9 against 20.0 (64 x 64)
+//   K <= 2048       from 64 of them: 2048^3 26.5 us against 32.0 shared and 38.9 whole; 2048 x 4096 x 2048 32.5 against 39;
+//                   1024 x 2048 x 2048 26.0 against 27.8 for split-K
+//   K = 4096        x^T . W^T only (a k-contiguous B is staged without waste), from 96: 2048 x 2048 x 4096 45.0 us against
+//                   49.5 shared, 1536 x 4096 x 4096 47.2 against 51.2; x^T . W 1024 x 4096 x 4096: 46.0 against 42.9 shared
+static bool narrow_round(const GemmProblem& p, int layout) {
+  if (layout < 0 || (layout & 2) != 0 || mfma_config(p, 13) == 0 || p.M <= 128 || p.N <= 128) return false;
+  const long long tn = (long long)((p.M + 255) / 256) * ((p.N + 127) / 128) * p.batch;
+  if (tn > compute_units()) return false;
+  if (p.K <= 1024) return true;
+  if (p.K <= 2048) return tn >= 64;
+  // (with fewer rows four parts of the k loop do better when K can be cut in four: 384 x 6144 x 4096 36.0 us in parts against
+  // 43.4; 192 x 12568 x 3264, which only halves: 36.0 against 41.7)
+  return layout == 1 && p.K < 8192 && tn >= 96 && (p.M >= 1024 || mfma_splitk_parts(p) < 4);
 }
 
 int mfma_select(const GemmProblem& p) {
@@ -803,7 +836,11 @@ int mfma_select(const GemmProblem& p) {
   int tile;
   // (half tiles in their 64-deep form whenever K allows: never behind the 32-deep one, 2-5 % ahead for x . W -- 2048^3 26.1 ->
   // 24.9 us -- and 10-17 % for x . W^T, whose loads then move whole lines: 2048 x 4096 x 2048 34.1 -> 28.2 us)
-  if (big_ok && (layout & 2) != 0 && half_ok) tile = deep_ok ? 12 : 6;
+  // (an A that is not k-contiguous has its half tile too, 256 x 128: taken when one round holds the problem, which whole
+  // tiles would leave half empty -- see narrow_round for the measured pairs; with K = 4096 or more the shared tiles and
+  // split-K, asked earlier, keep what they took: 1024 x 4096 x 4096 42.9 us shared against 46.0)
+  if (narrow_round(p, layout)) tile = 13;
+  else if (big_ok && (layout & 2) != 0 && half_ok) tile = deep_ok ? 12 : 6;
   else if (whole_ok && padded_nt) tile = 4;
   else if (small_tt) tile = 3;
   else if (whole_ok && deep_ok && (t256 >= half_cus || ((layout & 2) == 0 && t256 >= ring_from))) tile = 9;
@@ -908,6 +945,8 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   const int parts = mfma_splitk_parts(p);
   if (parts < 2) return false;
   const int layout = mfma_layout(p);
+  // an A that is not k-contiguous and one round of its 256 x 128 half tiles: those do better than the parts (narrow_round)
+  if (narrow_round(p, layout)) return false;
   // a handful of tiles: nothing else occupies the device (192 x 512 x 2048: 23 us against 32 us for
   // 64 x 64 tiles; 512 x 512 x 3072: 28 us against 35 us for half tiles; with both operands
   // k-contiguous the 64 x 64 kernel holds out longer -- 192 x 512 x 2048: 19 us against 22 us, but
@@ -955,6 +994,7 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
 bool mfma_prefers_tail(const GemmProblem& p) {
   if (p.K < 2048 || mfma_config(p, 10) == 0) return false;
   const int layout = mfma_layout(p);
+  if (narrow_round(p, layout)) return false;   // one round of 256 x 128 half tiles does better
   const long long cus = compute_units();
   const long long t256 = (long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   const long long th = (long long)((p.M + 127) / 128) * ((p.N + 255) / 256) * p.batch;
@@ -968,8 +1008,8 @@ bool mfma_prefers_tail(const GemmProblem& p) {
     return p.K >= from;
   }
   if (p.K < 4096) {
-    // an A that is not k-contiguous has no half tiles to fall back on: from K = 2048 (1024 x 4096 x 2048, 64 tiles:
-    // 32.5 us against 37.7 for split-K; 1536 x 4096 x 2048, 96 tiles: 34.4 against 40.1 whole)
+    // an A that is not k-contiguous (and more than one round of its 256 x 128 half tiles, see above): shared tiles from K =
+    // 2048 (1024 x 4096 x 2048, 64 tiles: 32.5 us against 37.7 for split-K; 1536 x 4096 x 2048, 96 tiles: 34.4 against 40.1 whole)
     return (layout & 2) == 0 && t256 >= (p.M >= 512 ? 48 : 64) && t256 <= 128;
   }
   // tiles that are mostly padding rows: 64 x 64 x 512 x 4096, 128 tiles, x . W^T 95 us against 77 for 64 x 64 tiles, with
@@ -1058,6 +1098,7 @@ const char* mfma_name(int config) {
     case 10: return "mfma_256x256_m16_k64_tail";
     case 11: return "mfma_256x256_m16_k64_split";
     case 12: return "mfma_128x256_m16_k64";
+    case 13: return "mfma_256x128_m16_k64";
     case 2: return "mfma_128x128";
     case 7: return "mfma_128x128_any";
     case 8: return "mfma_64x64_any";

@@ -146,15 +146,16 @@ struct FragReader<false> {
 };
 
 // ---- the schedule's slots for a wave tile of TM x TN MFMA tiles (a phase is TM / 2 x TN MFMAs, u = TM / 2 j + i) ---------
-// (TM, TN) = (8, 8) is the schedule as described above.  (8, 6) -- the 192-wide workgroup tile, 24 MFMAs per phase -- and
-// (4, 8) -- the 128 x 256 half tile, 16 MFMAs per phase, two A loads per phase -- keep the order of events and move them to
-// earlier slots.  Every function gives, for MFMA u of a phase, the index of the thing that rides behind it, or -1.
+// (TM, TN) = (8, 8) is the schedule as described above.  (8, 6) -- the 192-wide workgroup tile, 24 MFMAs per phase --,
+// (4, 8) -- the 128 x 256 half tile, 16 MFMAs per phase, two A loads per phase -- and (8, 4) -- the 256 x 128 half tile,
+// 16 MFMAs per phase -- keep the order of events and move them to earlier slots.  Every function gives, for MFMA u of a phase, the index of the thing that rides behind it, or -1.
 template <int TM, int TN> constexpr int a_load_at(int u) {   // A load of the phase's share (phases 0, 1)
   if (TM == 4) return u == 12 ? 0 : u == 14 ? 1 : -1;
+  if (TN == 4) return (u >= 8 && (u & 1) == 0) ? (u - 8) >> 1 : -1;
   return (u >= 4 * TN - 16 && (u & 3) == 0) ? (u - (4 * TN - 16)) >> 2 : -1;
 }
 template <int TM, int TN> constexpr int b_load_at(int u) {   // B load 0..7 (phase 3)
-  if (TM == 4) return (u & 1) == 0 ? u >> 1 : -1;
+  if (TM == 4 || TN == 4) return (u & 1) == 0 ? u >> 1 : -1;
   return TN == 8 ? ((u & 3) == 0 ? u >> 2 : -1) : ((u % 3 == 0 && u < 24) ? u / 3 : -1);
 }
 // fragment reads of a phase that multiplies the first half of the A tiles (the rest of its own k half) ...
@@ -162,8 +163,9 @@ template <int TM, int TN> constexpr int own_b_read_at(int u) {   // B tiles 4 ..
   if (TM == 4) return u < 4 ? 4 + u : -1;
   return (u < 8 && (u & 1) == 0 && 4 + (u >> 1) < TN) ? 4 + (u >> 1) : -1;
 }
-template <int TM> constexpr int own_a_read_at(int u) {           // A tiles TM / 2 .. TM - 1
+template <int TM, int TN> constexpr int own_a_read_at(int u) {   // A tiles TM / 2 .. TM - 1
   if (TM == 4) return (u == 4 || u == 5) ? 2 + (u - 4) : -1;
+  if (TN == 4) return (u < 8 && (u & 1) == 1) ? 4 + (u >> 1) : -1;
   return (u >= 8 && u < 16 && (u & 1) == 0) ? 4 + ((u - 8) >> 1) : -1;
 }
 // ... and of one that multiplies the second half (tiles of the next k half: A 0 .. TM / 2 - 1, idle by now, and B 0-3,
@@ -185,6 +187,12 @@ template <int TM, int TN, int PH> constexpr int event_at(int u) {
     return u == 9 ? 18 : u == 11 ? 22 : u == 13 ? 26 : -1;                       // 18, 22, 26 -> 9, 11, 13
   }
   if (TN == 8) return u;
+  if (TN == 4) {
+    if (PH == 0) return u < 7 ? 2 * u + 1 : -1;                                   // 1, 3, .. 13 -> 0 .. 6 (loads at 8, 10, 12, 14)
+    if (PH == 1) return u;                                                        // 2, 6, 10, 14
+    if (PH == 2) return (u >= 8 && u <= 12) ? 17 + 2 * (u - 8) : -1;              // 17 .. 25 -> 8 .. 12
+    return u == 8 ? 18 : u == 10 ? 22 : u == 12 ? 26 : -1;                        // 18, 22, 26 -> 8, 10, 12 (behind a load each)
+  }
   if (PH == 0) return u < 7 ? 2 * u + 1 : -1;                      // 1, 3, .. 13 -> 0 .. 6 (ahead of the loads from 8 on)
   if (PH == 1) return u;                                           // 2, 6, 10, 14
   if (PH == 2) return (u >= 15 && (u & 1) == 1) ? u + 2 : -1;      // 17 .. 25 -> 15 .. 23
@@ -397,13 +405,17 @@ constexpr int TAIL_MAX_PARTS = 3;
 // whose valid width p.tile_n <= 192 is a multiple of 8 -- tiles lie p.tile_n columns apart and columns beyond that
 // width are computed and not stored.  It fills a last round of the persistent grid that whole tiles would leave three
 // quarters full or less (see gemm_m16d_split_kernel).  B is staged as for the wide tile (a 256-wide unit).
+// 4: the 256 x 128 half tile (waves of 128 x 64; p.tile_n <= 128), which gives an A that is not k-contiguous -- and so has
+// no 128 x 256 half tile -- twice the workgroups on a partly filled device.  The B unit stays 256 wide in LDS; of a
+// k-contiguous B only the first 128 rows are requested (the loads of waves 2 and 3 aim out of range), an n-contiguous
+// B's k rows are fetched whole (the tile's neighbour's columns ride along).
 // TM: row tiles per wave.  8: 256 rows per workgroup tile.  4: the 128 x 256 half tile (waves of 64 x 128) for problems that
 // leave compute units idle with whole tiles; its A unit is 128 rows of a k-contiguous A (in a slot of the same size).
 template <typename T, bool A_KC, bool B_KC, int EPI, bool SK, bool FLIP = false, int TN = 8, int TM = 8>
 __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailShare& ts) {
   static_assert(EPI != EPI_TRANS, "sigmoid / tanh / elu have epilogue kinds of their own here");
   static_assert(!FLIP || EPI != EPI_PARTIAL, "flipped: the store_tile epilogues only");
-  static_assert(TN == 8 || (TN == 6 && !SK && !FLIP && EPI != EPI_PARTIAL), "the narrow tile: plain form, store_tile epilogues");
+  static_assert(TN == 8 || ((TN == 6 || TN == 4) && !SK && !FLIP && EPI != EPI_PARTIAL), "the narrow tiles: plain form, store_tile epilogues");
   static_assert(TM == 8 || (TM == 4 && TN == 8 && A_KC && !SK && !FLIP), "the half tile: k-contiguous A, plain form");
   constexpr int HALF = TM / 2;        // A tiles per phase
   constexpr int TILE_M = 32 * TM;     // rows of a workgroup tile
@@ -545,6 +557,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
                         l.voff[LoaderA::vindex(i)], base + (uint32_t)LoaderA::sindex(i) * lstep_a);
   };
   auto issue_b = [&](const Loader<B_KC>& l, uint32_t slot, uint32_t base) {
+    if constexpr (TN == 4 && B_KC) base = select_lt(wave, 2, base, OOB);   // rows 128-255 of the unit are not needed
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       ring::load_to_lds(rb, slot + Loader<B_KC>::wave_share(wave) + Loader<B_KC>::landing(i),
@@ -680,7 +693,7 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
           }
           if (OWN) {
             if (own_b_read_at<TM, TN>(u) >= 0) bf[own_b_read_at<TM, TN>(u)] = fb.template read<H>(ub, own_b_read_at<TM, TN>(u));
-            if (own_a_read_at<TM>(u) >= 0) af[own_a_read_at<TM>(u)] = fa.template read<H>(ua, own_a_read_at<TM>(u));
+            if (own_a_read_at<TM, TN>(u) >= 0) af[own_a_read_at<TM, TN>(u)] = fa.template read<H>(ua, own_a_read_at<TM, TN>(u));
           } else {
             if (next_a_read_at<TM>(u) >= 0) af[next_a_read_at<TM>(u)] = fa.template read<H>(ua, next_a_read_at<TM>(u));
             if (next_b_read_at<TM>(u) >= 0) bf[next_b_read_at<TM>(u)] = fb.template read<H>(ub, next_b_read_at<TM>(u));
@@ -716,7 +729,10 @@ __device__ __forceinline__ void gemm_m16d_body(const GemmProblem& p, const TailS
           if (u == 6) so_a3 = select_lt(r, limit_a, soa + 3 * lstep_a, OOB);
         }
         if (u == 10) sel = select_lt(r, S, cur_tile.offb, next_tile.offb);
-        if (u == 14) sob = select_lt(r, limit_b, sel + eb_off, OOB);
+        if (u == 14) {
+          sob = select_lt(r, limit_b, sel + eb_off, OOB);
+          if constexpr (TN == 4 && B_KC) sob = select_lt(wave, 2, sob, OOB);   // rows 128-255 of the unit are not needed
+        }
       });
       // ---- phase 2: k half 1, A tiles 0-3 ----
       phase(C0{}, std::false_type{}, std::true_type{}, C1{}, C0{}, x, xb, ta, so_a0, so_a1, so_a2, so_a3, [&](int u) __attribute__((always_inline)) {
@@ -879,6 +895,12 @@ __global__ __launch_bounds__(NT) void gemm_m16d_tail_kernel(GemmProblem p, TailS
 template <typename T, bool B_KC, int EPI>
 __global__ __launch_bounds__(NT) void gemm_m16d_half_kernel(GemmProblem p) {
   gemm_m16d_body<T, true, B_KC, EPI, false, false, 8, 4>(p, TailShare{});
+}
+
+// The 256 x 128 half tile, for an A that is not k-contiguous.
+template <typename T, bool B_KC, int EPI>
+__global__ __launch_bounds__(NT) void gemm_m16d_narrow_kernel(GemmProblem p) {
+  gemm_m16d_body<T, false, B_KC, EPI, false, false, 4, 8>(p, TailShare{});
 }
 
 // Two tile walks in one launch, for a tile count that leaves the last round of the persistent grid between half
@@ -1103,6 +1125,35 @@ hipError_t launch_half(const GemmProblem& p, hipStream_t stream) {
   }
   if (p.bias) return launch_half_kernel<T, B_KC, EPI_BIAS>(p, stream);
   return launch_half_kernel<T, B_KC, EPI_PLAIN>(p, stream);
+}
+
+// the 256 x 128 half tile (A not k-contiguous)
+template <typename T, bool B_KC, int EPI>
+hipError_t launch_narrow_kernel(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm_m16d_narrow_kernel<T, B_KC, EPI>;
+  constexpr int lds_bytes = UNITS * UNIT;
+  static std::atomic<uint32_t> configured{0};
+  if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
+  GemmProblem q = p;
+  q.tile_n = 128;
+  const long long tiles = (long long)((p.M + 255) / 256) * ((p.N + 127) / 128) * p.batch;
+  const int grid = ring::persistent_grid(tiles);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NT), lds_bytes, stream, q);
+  return launch_status(stream);
+}
+
+template <typename T, bool B_KC>
+hipError_t launch_narrow(const GemmProblem& p, hipStream_t stream) {
+  if (p.activation == srtActivationSigmoid) return launch_narrow_kernel<T, B_KC, EPI_SIGMOID>(p, stream);
+  if (p.activation == srtActivationTanh) return launch_narrow_kernel<T, B_KC, EPI_TANH>(p, stream);
+  if (p.activation == srtActivationElu) return launch_narrow_kernel<T, B_KC, EPI_ELU>(p, stream);
+  if (p.activation == srtActivationClippedRelu) return launch_narrow_kernel<T, B_KC, EPI_CLIPPED>(p, stream);
+  if (p.activation == srtActivationRelu) {
+    if (p.bias) return launch_narrow_kernel<T, B_KC, EPI_BIAS_RELU>(p, stream);
+    return launch_narrow_kernel<T, B_KC, EPI_RELU>(p, stream);
+  }
+  if (p.bias) return launch_narrow_kernel<T, B_KC, EPI_BIAS>(p, stream);
+  return launch_narrow_kernel<T, B_KC, EPI_PLAIN>(p, stream);
 }
 
 // The split-K pass on half tiles (a k-contiguous A of at most 128 rows): fp32 accumulators to a workspace.

@@ -117,6 +117,8 @@ def plans_for(ta, tb):
     if not ta:
         plans.append("mfma_128x256_m16")    # k-contiguous A
         plans.append("mfma_128x256_m16_k64")
+    else:
+        plans.append("mfma_256x128_m16_k64")    # the half tile of the other A layouts
     return plans
 
 
