@@ -1022,12 +1022,14 @@ bool mfma_prefers_tail(const GemmProblem& p) {
   if (t256 >= cus) {
     // a handful left over (see above), or one round and up to half of another with a k loop long enough to
     // carry the adding up (3072 x 8192 x 8192, 384 tiles: 275 us against 298)
-    return left > 0 && (8 * left <= cus || (t256 < 2 * cus && 2 * left <= cus && p.K >= 8192));
+    // (from K = 4096: 4096 x 6144 x 4096, 384 tiles, 149.8 us against 161.8 whole; 3072 x 8192 x 4096 152.1 against 163.0)
+    return left > 0 && (8 * left <= cus || (t256 < 2 * cus && 2 * left <= cus && p.K >= 4096));
   }
   if (left < 48 || left > 160) return false;
   // (the 48-tile figures are of 2-6 rows of tiles, one row stays with split-K; so does K = 8192, which four parts cut
   // deeper: 512 x 6144 x 8192 with A m-contiguous 58 us against 62)
-  if (left < 64 && (p.M < 512 || (p.K > 4096 && p.batch == 1))) return false;
+  // (with 1024 rows or more the shared tiles keep K = 8192 too: 1536 x 2048 x 8192 x^T . W^T 64.4 us against 72.5 in parts)
+  if (left < 64 && (p.M < 512 || (p.K > 4096 && p.batch == 1 && p.M < 1024))) return false;
   // x . W has half tiles to fall back on: while they fit one round they are as good or better below K = 8192 from 72 tiles
   // up (1536 x 3072 x 4096: 46-53 us in half tiles, 53 shared; 2048 x 3072 x 4096: 48-52 against 51-55)
   // so has x . W^T since its half tiles are 64 deep (whole-line loads): one round of them beats the shared tiles below

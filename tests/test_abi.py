@@ -244,10 +244,10 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_256x256_m16_k64_tail"    # 64 tiles again
     assert query(native.REAL16BF, 1024, 2048, 8192) == "mfma_256x256_splitk"          # 32 tiles: eight parts
     assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_256x256_splitk"
-    assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x128_m16_k64" # A not k-contiguous: from K = 2048
-    assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x128_m16_k64"    # 32 tiles: whole tiles from 24 up
-    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_256x128_m16_k64"    # 16 tiles, neither operand k-contiguous: whole tiles from 12 up
-    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x128_m16_k64"   # 128 tiles, K = 2048, no half tiles: cut in two
+    assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x128_m16_k64"    # A not k-contiguous: one round of its 256 x 128 half tiles
+    assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x128_m16_k64"    # (64 of them)
+    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_256x128_m16_k64"    # (32 of them, neither operand k-contiguous)
+    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x128_m16_k64"    # (256 of them: one round exactly)
     # mid-size problems: the 256 x 256 kernels from 24 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16_k64"             # 144 tiles, long k loop
@@ -256,7 +256,7 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16_k64"             # 128 half tiles
     assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16_k64"
     assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16_k64"             # 256 half tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x128_m16_k64"   # A not k-contiguous: whole tiles cut along k
+    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x128_m16_k64"    # A not k-contiguous: its half tile is 256 x 128
     assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x128_m16_k64"
     # 258 whole tiles: a whole round, and the two left over cut along k in three parts each
     assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_256x256_m16_k64_tail"
@@ -289,10 +289,10 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 8, 1288, 10432) == "skinny"                         # only two parts possible
     assert query(native.REAL16BF, 8, 88, 2576, ta=True) == "mfma_256x256_m16"           # one whole tile beats 64 x 64 tiles on an m-contiguous A
     assert query(native.REAL16BF, 4826, 12408, 7056, tb=True) == "mfma_256x256_k64"   # k extent not a whole number of 32-deep stages
-    assert query(native.REAL16BF, 192, 12568, 3264, ta=True, tb=True) == "mfma_256x128_m16_k64"   # two parts up to a quarter round
+    assert query(native.REAL16BF, 192, 12568, 3264, ta=True, tb=True) == "mfma_256x128_m16_k64"   # K only halves: one round of half tiles beats two parts
     assert query(native.REAL16BF, 664, 7536, 352, tb=True) == "mfma_128x256_m16"      # 13 % padding rows are fine for half tiles
     assert query(native.REAL16BF, 169, 9824, 504, tb=True) == "mfma_64x64"            # a second row of half tiles that is mostly padding is not
-    assert query(native.REAL16BF, 512, 512, 1024, ta=True) == "mfma_256x128_m16_k64"   # four tiles, neither operand k-contiguous
+    assert query(native.REAL16BF, 512, 512, 1024, ta=True) == "mfma_256x128_m16_k64"   # eight half tiles, neither operand k-contiguous: ahead of split-K
     # batches (no split-K pass)
     def query_batched(dt, B, M, N, K, ta=False, tb=False):
         ashape = (B, K, M) if ta else (B, M, K)
