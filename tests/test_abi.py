@@ -113,6 +113,57 @@ def test_result_alias_rules_without_gpu():
     assert call(0, (32, 32), (96, 1), 8, (32, 32), (64, 1)) == native.ERROR_NOT_SUPPORTED
 
 
+def test_result_alias_rule_never_accepts_views_that_share_an_element():
+    """Random small views (all strides, pitches and offsets inside one buffer), checked against the element sets written
+    out: whenever the result shares an element with an operand the call must be refused (either status); the proof of
+    disjointness may fail to find what is true, never claim what is false.  Accepted calls go on to a launch, so this runs
+    only where there is no device to launch on (placeholder pointers)."""
+    L = native.lib()
+    count = ctypes.c_int32(0)
+    if L.srtGetDeviceCount(ctypes.byref(count)) == 0 and count.value > 0:
+        pytest.skip("placeholder pointers: only on a host without a device")
+    g = np.random.Generator(np.random.Philox(1234))
+    base = 1 << 22
+
+    def view(rows, cols):
+        kind = int(g.integers(0, 4))
+        if kind == 0:       # dense rows under a pitch
+            pitch = cols + int(g.integers(0, 12))
+            st = (pitch, 1)
+        elif kind == 1:     # transposed: columns under a pitch
+            pitch = rows + int(g.integers(0, 12))
+            st = (1, pitch)
+        elif kind == 2:     # every other element of a row
+            pitch = 2 * cols + int(g.integers(0, 8))
+            st = (pitch, 2)
+        else:               # arbitrary
+            st = (int(g.integers(1, 40)), int(g.integers(1, 40)))
+        return int(g.integers(0, 64)), st
+
+    def elements(off, shape, st):
+        return {off + i * st[0] + j * st[1] for i in range(shape[0]) for j in range(shape[1])}
+
+    refused = accepted = overlapping = 0
+    for _ in range(3000):
+        M, N, K = int(g.integers(1, 7)), int(g.integers(1, 7)), int(g.integers(1, 7))
+        a_off, a_st = view(M, K)
+        o_off, o_st = view(M, N)
+        ad, k1 = native.make_descriptor(native.REAL32F, (M, K), a_st, native.ORDER_ROW)
+        bd, k2 = native.make_descriptor(native.REAL32F, (K, N), (N, 1), native.ORDER_ROW)
+        od, k3 = native.make_descriptor(native.REAL32F, (M, N), o_st, native.ORDER_ROW)
+        st = L.srtMatmul(ctypes.c_void_p(base + 4 * a_off), ctypes.byref(ad), 0, ctypes.c_void_p(1 << 30), ctypes.byref(bd), 0,
+                         ctypes.c_void_p(base + 4 * o_off), ctypes.byref(od), None)
+        shares = bool(elements(a_off, (M, K), a_st) & elements(o_off, (M, N), o_st))
+        overlapping += shares
+        if st in (native.ERROR_INVALID_VALUE, native.ERROR_NOT_SUPPORTED):
+            refused += 1
+        else:
+            accepted += 1
+            assert not shares, (M, N, K, a_off, a_st, o_off, o_st)
+    # the draw exercises both answers and both truths
+    assert overlapping > 300 and accepted > 300 and refused > 300, (overlapping, accepted, refused)
+
+
 def test_elementwise_and_backward_validation_without_gpu():
     L = native.lib()
     dummy = ctypes.c_void_p(256)
