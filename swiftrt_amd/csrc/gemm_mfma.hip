@@ -684,11 +684,20 @@ int mfma_splitk_parts(const GemmProblem& p);
 //   K = 4096        x^T . W^T only (a k-contiguous B is staged without waste), from 96: 2048 x 2048 x 4096 45.0 us against
 //                   49.5 shared, 1536 x 4096 x 4096 47.2 against 51.2; x^T . W 1024 x 4096 x 4096: 46.0 against 42.9 shared
 static bool narrow_round(const GemmProblem& p, int layout) {
-  if (layout < 0 || (layout & 2) != 0 || mfma_config(p, 13) == 0 || p.M <= 128 || p.N <= 128) return false;
+  // (from 64 rows and columns: a batch of 64 x 512 x 1024 problems runs 16.2 us in these tiles, three quarters padding,
+  // against 22.6 in whole tiles and 19.4 in 64 x 64 ones; 4 x 128 x 128 x 1024: 15.6 against 22.4)
+  if (layout < 0 || (layout & 2) != 0 || mfma_config(p, 13) == 0 || p.M < 64 || p.N < 64) return false;
   const long long tn = (long long)((p.M + 255) / 256) * ((p.N + 127) / 128) * p.batch;
   if (tn > compute_units()) return false;
+  // (tiles that are three quarters padding rows only while they leave half the device free: 64 x 64 x 512 x 1024, 256 of them,
+  // 27.1 us against 23.1 in 128 whole tiles)
+  if (p.M <= 64 && 2 * tn > compute_units()) return false;
   if (p.K <= 1024) return true;
   if (p.K <= 2048) return tn >= 64;
+  // (a batch at K = 4096: only tiles that are mostly padding rows -- 64 x 64 x 512 x 4096 x^T . W^T 68.4 us against 83.3 shared
+  // and 97.7 whole; 16 x 512 x 512 x 4096: 60.5 against 54.9 shared)
+  // (and only a device's worth of them: 16 x 64 x 512 x 4096, 64 tiles, 43.2 us against 39.3 shared)
+  if (p.batch > 1) return layout == 1 && p.K < 8192 && p.M <= 128 && 2 * tn > compute_units();
   // (with fewer rows four parts of the k loop do better when K can be cut in four: 384 x 6144 x 4096 36.0 us in parts against
   // 43.4; 192 x 12568 x 3264, which only halves: 36.0 against 41.7)
   return layout == 1 && p.K < 8192 && tn >= 96 && (p.M >= 1024 || mfma_splitk_parts(p) < 4);
@@ -773,15 +782,20 @@ int mfma_select(const GemmProblem& p) {
   // tiles, 38 us against 25 for 64 x 64 tiles)
   // (those two are of batches; a single matrix shares its operands between tiles and takes half tiles from 72: 397 x 7528 x
   // 1056, 120 of them, 15 us against 21; 664 x 3208 x 8544, 78, 87 against 97)
-  const long long th_min = p.batch == 1 ? 72 : p.K >= 2048 ? 96 : (p.K >= 1024 && p.M < 512) ? 128 : 72;
-  const bool one_round = th >= th_min && rounds_h == 1 && half_fill_ok && (p.batch == 1 || t256 < half_cus);
+  // (a batch in the 64-deep half tile, whose loads move whole lines of both operands, from 64 of them whatever K, and with
+  // rows that are half padding: 16 x 384 x 384 x 1024, 96 half tiles, 16.0 us against 19.7 for 64 x 64 tiles; 64 x 128 x 128 x
+  // 4096, 64 of them, 43.2 against 58.0; 64 x 64 x 512 x 1024, 128 of them half empty, 18.6 against 23.0)
+  const bool deep_batch = p.batch > 1 && p.K % 64 == 0 && p.K >= 256;
+  const long long th_min = deep_batch ? 64 : p.batch == 1 ? 72 : p.K >= 2048 ? 96 : (p.K >= 1024 && p.M < 512) ? 128 : 72;
+  const bool fill_ok = half_fill_ok || (deep_batch && 2 * (m_pad - p.M) <= m_pad);
+  const bool one_round = th >= th_min && rounds_h == 1 && fill_ok && (p.batch == 1 || t256 < half_cus || (deep_batch && t256 == half_cus));
   const bool small_rows = p.M <= 128 && p.K <= 512 && th >= 72;
   // (x . W^T with a short k loop and whole tiles that leave a second or later round at most half full: twice the
   // workgroups fill it better -- 3072 x 6144 x 512, 288 tiles: 25.4 us against 27.3 whole; 3072 x 6144 x 256: 18.7 against
   // 20.7; 3072 x 6144 x 1024: 39.7 against 42.8.  Whole rounds stay whole: 4096 x 4096 x 512 19.8 us against 21.4)
   const bool short_nt = p.K <= 1024 && p.K % 64 == 0 && p.K >= 256 && t256 > cus && t256 % cus != 0 && 2 * (t256 % cus) <= cus &&
                         p.batch == 1 && half_fill_ok;
-  const bool half_nt = p.M > 64 && (one_round || small_rows || short_nt);
+  const bool half_nt = (p.M > 64 || (deep_batch && p.M == 64)) && (one_round || small_rows || short_nt);
   // (a round of half tiles takes 0.6 of a round of whole ones on the 32-deep kernels, 0.7 against the 64-deep
   // one: 4096 x 10240 x 4096, five rounds of half tiles against three of whole ones, 265 us against 249 us)
   const bool deep = p.K % 64 == 0 && p.K >= 512;
