@@ -689,18 +689,20 @@ static bool narrow_round(const GemmProblem& p, int layout) {
   if (layout < 0 || (layout & 2) != 0 || mfma_config(p, 13) == 0 || p.M < 64 || p.N < 64) return false;
   const long long tn = (long long)((p.M + 255) / 256) * ((p.N + 127) / 128) * p.batch;
   if (tn > compute_units()) return false;
+  if (p.K > 2048) {
+    // (a batch at K = 4096: only tiles that are mostly padding rows, and only a device's worth of them -- 64 x 64 x 512 x 4096
+    // x^T . W^T 68.4 us against 83.3 shared and 97.7 whole; 16 x 512 x 512 x 4096: 60.5 against 54.9 shared; 16 x 64 x 512 x 4096,
+    // 64 tiles: 43.2 against 39.3 shared)
+    if (p.batch > 1) return layout == 1 && p.K < 8192 && p.M <= 128 && 2 * tn > compute_units();
+    // (with fewer rows four parts of the k loop do better when K can be cut in four: 384 x 6144 x 4096 36.0 us in parts against
+    // 43.4; 192 x 12568 x 3264, which only halves: 36.0 against 41.7)
+    return layout == 1 && p.K < 8192 && tn >= 96 && (p.M >= 1024 || mfma_splitk_parts(p) < 4);
+  }
   // (tiles that are three quarters padding rows only while they leave half the device free: 64 x 64 x 512 x 1024, 256 of them,
   // 27.1 us against 23.1 in 128 whole tiles)
   if (p.M <= 64 && 2 * tn > compute_units()) return false;
   if (p.K <= 1024) return true;
-  if (p.K <= 2048) return tn >= 64;
-  // (a batch at K = 4096: only tiles that are mostly padding rows -- 64 x 64 x 512 x 4096 x^T . W^T 68.4 us against 83.3 shared
-  // and 97.7 whole; 16 x 512 x 512 x 4096: 60.5 against 54.9 shared)
-  // (and only a device's worth of them: 16 x 64 x 512 x 4096, 64 tiles, 43.2 us against 39.3 shared)
-  if (p.batch > 1) return layout == 1 && p.K < 8192 && p.M <= 128 && 2 * tn > compute_units();
-  // (with fewer rows four parts of the k loop do better when K can be cut in four: 384 x 6144 x 4096 36.0 us in parts against
-  // 43.4; 192 x 12568 x 3264, which only halves: 36.0 against 41.7)
-  return layout == 1 && p.K < 8192 && tn >= 96 && (p.M >= 1024 || mfma_splitk_parts(p) < 4);
+  return tn >= 64;
 }
 
 int mfma_select(const GemmProblem& p) {
