@@ -787,7 +787,8 @@ int mfma_select(const GemmProblem& p) {
   // (a batch in the 64-deep half tile, whose loads move whole lines of both operands, from 64 of them whatever K, and with
   // rows that are half padding: 16 x 384 x 384 x 1024, 96 half tiles, 16.0 us against 19.7 for 64 x 64 tiles; 64 x 128 x 128 x
   // 4096, 64 of them, 43.2 against 58.0; 64 x 64 x 512 x 1024, 128 of them half empty, 18.6 against 23.0)
-  const bool deep_batch = p.batch > 1 && p.K % 64 == 0 && p.K >= 256;
+  // (not for short k loops: 32 x 256 x 256 x 256 7.7 us against 7.1 for 64 x 64 tiles, 64 x 128 x 128 x 256 7.7 against 6.9)
+  const bool deep_batch = p.batch > 1 && p.K % 64 == 0 && p.K >= 1024;
   const long long th_min = deep_batch ? 64 : p.batch == 1 ? 72 : p.K >= 2048 ? 96 : (p.K >= 1024 && p.M < 512) ? 128 : 72;
   const bool fill_ok = half_fill_ok || (deep_batch && 2 * (m_pad - p.M) <= m_pad);
   const bool one_round = th >= th_min && rounds_h == 1 && fill_ok && (p.batch == 1 || t256 < half_cus || (deep_batch && t256 == half_cus));

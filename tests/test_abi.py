@@ -355,6 +355,9 @@ def test_kernel_selection_is_queryable_without_gpu():
         p = ctypes.c_void_p(256)
         assert L.srtMatmulQueryKernel(ctypes.byref(ad), int(ta), ctypes.byref(bd), int(tb), ctypes.byref(od), p, p, p, buf, 64) == 0
         return buf.value.decode()
+    assert query_batched(native.REAL16F, 32, 256, 256, 256, tb=True) == "mfma_64x64"                   # benchmark config 2: launch-sized, every CU a workgroup
+    assert query_batched(native.REAL16BF, 16, 384, 384, 1024, tb=True) == "mfma_128x256_m16_k64"       # 96 half tiles of a batch, 64 deep
+    assert query_batched(native.REAL16BF, 16, 64, 512, 1024, ta=True) == "mfma_256x128_m16_k64"        # 64 tiles of 256 x 128, A not k-contiguous
     assert query_batched(native.REAL16BF, 4, 256, 256, 4096, ta=True) == "mfma_256x256_m16_k64_tail"   # four tiles cut along k
     assert query_batched(native.REAL16BF, 16, 256, 256, 2048, ta=True, tb=True) == "mfma_256x256_m16_k64_tail"
     assert query_batched(native.REAL16BF, 4, 128, 128, 4096, tb=True) == "mfma_64x64"                  # mostly padding, both k-contiguous
