@@ -1033,8 +1033,9 @@ def test_fp32_operand_beyond_4_gib_vs_exact():
 @pytest.mark.parametrize("plan,M,N", [(None, 64, 96), ("mfma_256x256_m16", 512, 512), ("mfma_256x256", 512, 512)])
 def test_fused_transcendentals_keep_their_digits_near_zero(act, dt, plan, M, N, tmp_path):
     """Pre-activations from 1e-7 to 0.4 in magnitude, both signs (K = 8 with a single non-zero term, so the
-    accumulator is exact): the fused epilogues use the hardware exponential, whose closed forms for tanh and
-    exp(x) - 1 cancel near 0; every result must be within two rounding steps of the stored type, relative."""
+    accumulator is exact): the fused epilogues work in fp32 with the hardware exponential (sigmoid, elu) or a
+    quotient of polynomials (tanh); a closed form that cancels near 0 -- (e^2x - 1) / (e^2x + 1), exp(x) - 1 --
+    would lose its digits here.  Every result must be within two rounding steps of the stored type, relative."""
     K = 8
     mags = np.logspace(-7, -0.4, N) * np.where(np.arange(N) % 2, -1.0, 1.0)
     x = np.zeros((M, K), np.float32)
