@@ -101,6 +101,14 @@ hipError_t launch_m16dn_BF16_00(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dn_BF16_01(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dn_F16_00(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dn_F16_01(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_BF16_00(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_BF16_01(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_BF16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_BF16_11(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_F16_00(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_F16_01(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_F16_10(const GemmProblem&, hipStream_t);
+hipError_t launch_m16q_F16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_partial_BF16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16dh_partial_F16_11(const GemmProblem&, hipStream_t);
 hipError_t launch_m16h_BF16_10(const GemmProblem&, hipStream_t);
@@ -592,6 +600,16 @@ hipError_t launch_m16dn(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16dn_BF16_01(p, stream) : launch_m16dn_BF16_00(p, stream);
   return b_kc ? launch_m16dn_F16_01(p, stream) : launch_m16dn_F16_00(p, stream);
 }
+// the 128 x 128 quarter tile of the 16x16x32 kernel (128-deep units), all four layouts
+template <typename T>
+hipError_t launch_m16q(const GemmProblem& p, bool a_kc, bool b_kc, hipStream_t stream) {
+  if (T::dtype == srtReal16BF) {
+    if (a_kc) return b_kc ? launch_m16q_BF16_11(p, stream) : launch_m16q_BF16_10(p, stream);
+    return b_kc ? launch_m16q_BF16_01(p, stream) : launch_m16q_BF16_00(p, stream);
+  }
+  if (a_kc) return b_kc ? launch_m16q_F16_11(p, stream) : launch_m16q_F16_10(p, stream);
+  return b_kc ? launch_m16q_F16_01(p, stream) : launch_m16q_F16_00(p, stream);
+}
 template <typename T>
 hipError_t launch_m16h(const GemmProblem& p, bool b_kc, hipStream_t stream) {
   if (T::dtype == srtReal16BF) return b_kc ? launch_m16h_BF16_11(p, stream) : launch_m16h_BF16_10(p, stream);
@@ -612,6 +630,7 @@ hipError_t launch_tile(const GemmProblem& p, int tile, bool a_kc, bool b_kc, hip
     case 11: return launch_m16d_split<T>(p, a_kc, b_kc, stream);
     case 12: return launch_m16dh<T>(p, b_kc, stream);
     case 13: return launch_m16dn<T>(p, b_kc, stream);
+    case 14: return launch_m16q<T>(p, a_kc, b_kc, stream);
     case 2: return launch_layout<T, 128, 128>(p, a_kc, b_kc, stream);
     case 7: return launch_any_layout<T, 128, 128>(p, stream);
     case 8: return launch_any_layout<T, 64, 64>(p, stream);
@@ -651,6 +670,7 @@ static int mfma_layout(const GemmProblem& p) {
 // 64-deep stages for two k-contiguous operands, 5: the 256 x 256 ring on 16x16x32 MFMAs, 6: its
 // 128 x 256 form for a k-contiguous A, 9: the 16x16x32 kernel with 64-deep staging units), or 0 when the
 // problem does not qualify for it.  10: tile 9's tail-sharing form.  11: its split form (a last round of 192-wide tiles).  12: its 128 x 256 half tile (k-contiguous A).  13: its 256 x 128 half tile (A not k-contiguous).
+// 14: the 128 x 128 quarter tile on 128-deep units (any layout).
 int mfma_config(const GemmProblem& p, int tile) {
   if (tile == 7 || tile == 8) {   // any strides and alignment (the loaders are chosen at launch)
     if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return 0;
@@ -658,9 +678,10 @@ int mfma_config(const GemmProblem& p, int tile) {
     return tile << 2;
   }
   const int layout = mfma_layout(p);
-  if (layout < 0 || tile < 1 || (tile > 6 && (tile < 9 || tile > 13))) return 0;
+  if (layout < 0 || tile < 1 || (tile > 6 && (tile < 9 || tile > 14))) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
   if ((tile == 9 || tile == 12 || tile == 13) && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
+  if (tile == 14 && !(p.K % 128 == 0 && p.K >= 512)) return 0;   // whole 128-deep units, at least four
   if (tile == 10) {   // left-over tiles to share, k in whole quads, no transcendental activation
     const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
     if (trans || !m16d_tail_fits_BF16_xx(p)) return 0;
@@ -1118,6 +1139,7 @@ const char* mfma_name(int config) {
     case 11: return "mfma_256x256_m16_k64_split";
     case 12: return "mfma_128x256_m16_k64";
     case 13: return "mfma_256x128_m16_k64";
+    case 14: return "mfma_128x128_m16_k128";
     case 2: return "mfma_128x128";
     case 7: return "mfma_128x128_any";
     case 8: return "mfma_64x64_any";

@@ -114,14 +114,14 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
 // (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
 // and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
 enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK,
-            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanM16DSplit, kPlanM16DH, kPlanM16DN, kPlanCount };
+            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanM16DSplit, kPlanM16DH, kPlanM16DN, kPlanM16Q, kPlanCount };
 
 const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
                                             "f32_mfma_64x64", "f32_mfma_splitk", "mfma_256x256_k64",
                                             "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16",
                                             "mfma_128x128_any", "mfma_64x64_any", "mfma_256x256_m16_k64",
                                             "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split",
-                                            "mfma_128x256_m16_k64", "mfma_256x128_m16_k64"};
+                                            "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128"};
 
 bool plan_supported(const GemmProblem& p, Plan plan) {
   switch (plan) {
@@ -140,6 +140,7 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
     case kPlanM16DSplit: return srt::mfma_config(p, 11) != 0;
     case kPlanM16DH: return srt::mfma_config(p, 12) != 0;
     case kPlanM16DN: return srt::mfma_config(p, 13) != 0;
+    case kPlanM16Q: return srt::mfma_config(p, 14) != 0;
     case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
     case kPlanF32SplitK: return srt::f32_mfma_supported(p);
     default: return srt::generic_supported(p);
@@ -180,6 +181,7 @@ Plan heuristic_plan(const GemmProblem& p) {
       case 10: return kPlanM16DTail;
       case 12: return kPlanM16DH;
       case 13: return kPlanM16DN;
+      case 14: return kPlanM16Q;
       default: return kPlanMfma64;
     }
   }
@@ -204,6 +206,7 @@ hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
     case kPlanM16DSplit: return srt::launch_mfma(p, srt::mfma_config(p, 11), stream);
     case kPlanM16DH: return srt::launch_mfma(p, srt::mfma_config(p, 12), stream);
     case kPlanM16DN: return srt::launch_mfma(p, srt::mfma_config(p, 13), stream);
+    case kPlanM16Q: return srt::launch_mfma(p, srt::mfma_config(p, 14), stream);
     case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
     case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
     default: return srt::launch_generic(p, stream);

@@ -391,7 +391,7 @@ def test_kernel_selection_answers_for_any_problem():
     buf = ctypes.create_string_buffer(64)
     known = {"empty", "generic", "skinny", "f32_mfma", "mfma_256x256", "mfma_128x128", "mfma_64x64", "mfma_256x256_k64",
              "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128_any", "mfma_64x64_any",
-             "mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64"}
+             "mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128"}
 
     def logu(lo, hi):
         return int(np.exp(g.uniform(np.log(lo), np.log(hi))))

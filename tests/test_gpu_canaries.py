@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 SENTINEL = {np.dtype(np.uint16): 0x7B5A, np.dtype(np.float16): 0x7B5A, np.dtype(np.float32): 0x7B5A7B5A}
 
 ALL_PLANS_16 = ("mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split", "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
-                "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128", "mfma_64x64", "mfma_128x128_any",
+                "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128", "mfma_128x128", "mfma_64x64", "mfma_128x128_any",
                 "mfma_64x64_any", "skinny", "generic")
 ALL_PLANS_32 = ("f32_mfma_64x64", "f32_mfma_splitk", "generic")
 
@@ -127,7 +127,7 @@ def test_every_16_bit_plan_keeps_inside_a_ragged_result_view(ta, tb, tmp_path):
     ran = run_matmul_case(tmp_path, H.BF16, 520, 776, 1024, 1, ta, tb, ALL_PLANS_16, 700 + 2 * ta + tb)
     print("plans exercised:", ran)
     for must in ("mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_splitk",
-                 "mfma_128x128", "mfma_64x64", "generic"):
+                 "mfma_128x128_m16_k128", "mfma_128x128", "mfma_64x64", "generic"):
         assert must in ran, must
     if not ta:
         assert "mfma_128x256_m16" in ran and "mfma_128x256_m16_k64" in ran

@@ -110,8 +110,10 @@ def check_plan(tmp_path, plan, dt, M, N, K, ta, tb, with_bias_relu=False):
     return got
 
 
-def plans_for(ta, tb):
+def plans_for(ta, tb, K):
     plans = ["mfma_256x256_m16_k64", "mfma_256x256_m16", "mfma_256x256"]
+    if K % 128 == 0 and K >= 512:
+        plans.append("mfma_128x128_m16_k128")    # the quarter tile: whole 128-deep units, at least four
     if not ta and tb:
         plans.append("mfma_256x256_k64")    # two k-contiguous operands
     if not ta:
@@ -126,7 +128,7 @@ def plans_for(ta, tb):
 @pytest.mark.parametrize("ta,tb", LAYOUTS)
 def test_headline_shape_integer_bit_exact(dt, ta, tb, tmp_path):
     """8192^3: 1024 tiles = 4 per workgroup, 256 whole stages, per-XCD k rotation with a transposed lhs."""
-    for plan in plans_for(ta, tb):
+    for plan in plans_for(ta, tb, 8192):
         check_plan(tmp_path, plan, dt, 8192, 8192, 8192, ta, tb)
 
 
@@ -135,9 +137,97 @@ def test_headline_shape_integer_bit_exact(dt, ta, tb, tmp_path):
 def test_ragged_round_integer_bit_exact(dt, ta, tb, tmp_path):
     """4608 x 4608 x 2048: 324 tiles on 256 workgroups (a second, ragged round; the grid is evened to 168),
     64 whole stages; and 4400 x 4360 x 320: edge tiles in M and N, ten whole stages = five 64-deep units."""
-    for plan in plans_for(ta, tb):
+    for plan in plans_for(ta, tb, 2048):
         check_plan(tmp_path, plan, dt, 4608, 4608, 2048, ta, tb)
+    for plan in plans_for(ta, tb, 320):
         check_plan(tmp_path, plan, dt, 4400, 4360, 320, ta, tb)
+
+
+# ---- the 128 x 128 quarter tile (128-deep units) on small pinned shapes ---------------------------------------
+QUARTER = "mfma_128x128_m16_k128"
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+@pytest.mark.parametrize("ta,tb", LAYOUTS)
+def test_quarter_tile_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
+    """Every staging layout; the shortest admissible k loop (four units), an odd number of units, ragged edges in M and
+    N (a last tile of 8 rows, of 8 columns), one tile and several per workgroup (1190 tiles), fewer tiles than workgroups;
+    then random operands against the fp64 product."""
+    r = H.rng(311)
+    for (M, N, K) in [(256, 384, 512), (1000, 520, 640), (2048, 2056, 896), (4400, 4360, 512), (136, 128, 1152)]:
+        pin(tmp_path, QUARTER, dt, M, N, K, ta, tb)
+        a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+        at, bt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(b, dt))
+        out = srt.Tensor(shape=[M, N], dtype=H.NP_STORAGE[dt])
+        assert query_kernel(at, ta, bt, tb, out) == QUARTER
+        srt.current_queue().matmul(at, ta, bt, tb, out)
+        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
+    M, N, K = 2040, 2056, 1024
+    pin(tmp_path, QUARTER, dt, M, N, K, ta, tb)
+    a_st = H.encode((r.standard_normal((K, M) if ta else (M, K)) / np.sqrt(K)).astype(np.float32), dt)
+    b_st = H.encode(r.standard_normal((N, K) if tb else (K, N)).astype(np.float32), dt)
+    out = srt.matmul(srt.Tensor(a_st), srt.Tensor(b_st), transposed_lhs=ta, transposed_rhs=tb).array()
+    a64, b64 = H.to64(a_st), H.to64(b_st)
+    c64 = (a64.T if ta else a64) @ (b64.T if tb else b64)
+    assert H.max_norm_rel(H.decode(out), c64) <= H.TOL[dt]
+    absprod = np.abs(a64.T if ta else a64) @ np.abs(b64.T if tb else b64)
+    assert H.elementwise_excess(H.decode(out), c64, absprod, dt, K) <= 1.0
+
+
+@pytest.mark.parametrize("dt", [H.BF16, H.F16])
+@pytest.mark.parametrize("act", list(srt.ActivationType))
+@pytest.mark.parametrize("tw", [False, True])
+def test_quarter_tile_epilogues_vs_oracle(act, dt, tw, tmp_path):
+    """y = act(x . W + b) and act(x . W^T + b): every activation through the fused epilogue, ragged M / N edges."""
+    from oracle import srt_oracle as ora
+    r = H.rng(29)
+    M, N, K = 1100, 1032, 512
+    x = H.encode(r.standard_normal((M, K)).astype(np.float32), dt)
+    w = H.encode((r.standard_normal((N, K) if tw else (K, N)) / 8).astype(np.float32), dt)
+    b = H.encode(r.uniform(-0.5, 0.5, N).astype(np.float32), dt)
+    coef = 0.75
+    pin(tmp_path, QUARTER, dt, M, N, K, False, tw, bias=True, act=act)
+    xt, wt, bt = srt.Tensor(x), srt.Tensor(w), srt.Tensor(b)
+    out = srt.Tensor(shape=[M, N], dtype=x.dtype)
+    assert query_kernel(xt, False, wt, tw, out) == QUARTER
+    srt.current_queue().matmul(xt, False, wt, tw, out, bias=bt, activation=act, coef=coef)
+    got = H.decode(out.array())
+    rows = np.concatenate([np.arange(0, M, 131), [M - 1]])
+    want = H.decode(ora.dense_forward(np.ascontiguousarray(x[rows]), w, b, int(act), coef=coef, transpose_w=tw,
+                                      acc=ora.ACC_F32, fused=True))
+    tol = {H.F16: 2.0 ** -10, H.BF16: 2.0 ** -7}[dt]
+    assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
+
+
+def test_quarter_tile_batched_and_nan(tmp_path):
+    """Strided batch (tiles of several batches per workgroup), and NaN / inf results encoded as the reference's codec does."""
+    r = H.rng(31)
+    B_, M, N, K = 5, 1024, 1032, 640
+    a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+    w = r.integers(-3, 4, (B_, K, N)).astype(np.float32)
+    pin(tmp_path, QUARTER, H.BF16, M, N, K, False, False, batch=B_)
+    at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+    out = srt.matmul(at, wt)
+    assert query_kernel(at, False, wt, False, out) == QUARTER
+    assert np.array_equal(out.array(), H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), H.BF16))
+    M = N = 768
+    K = 512
+    a = np.zeros((M, K), np.float32)
+    w = np.zeros((K, N), np.float32)
+    a[:, 0] = 1.0
+    w[0, :] = 2.0
+    a[5, 1] = np.nan
+    a[7, 1] = np.inf
+    w[1, :] = 1.0
+    pin(tmp_path, QUARTER, H.BF16, M, N, K, False, False)
+    at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
+    out = srt.matmul(at, wt)
+    assert query_kernel(at, False, wt, False, out) == QUARTER
+    got = out.array()
+    assert np.all(got[5] == 0x7FFF) and np.all(got[7] == 0x7F80)
+    assert np.all(got[6] == H.encode(np.array([2.0], np.float32), H.BF16)[0])
 
 
 # ---- the 64-deep form of the 16x16x32 kernel on small pinned shapes ------------------------------------------
