@@ -350,14 +350,14 @@ class Bench:
                     "flops": 2.0 * 32 * 256 ** 3, "bytes": 32 * 3 * 256 * 256 * 2, "bound": "mfma", "dtype": "f16",
                     "steps": 200}
         if name == "few_tiles":
-            # not one of the five benchmark configurations: a quarter-full device with a long k loop, the case of the
-            # tail-sharing form of the headline kernel (every tile cut along k into three parts)
+            # not one of the five benchmark configurations: a quarter of a device's worth of whole tiles with a long k
+            # loop, the case of the 128 x 128 quarter tile (256 of them, one per compute unit)
             g = rng(5)
             a = srt.Tensor(bf16_encode(g.standard_normal((1024, 4096), dtype=np.float32) / np.float32(64)))
             b = srt.Tensor(bf16_encode(g.standard_normal((4096, 4096), dtype=np.float32)))
             c = srt.Tensor(shape=[1024, 4096], dtype=np.uint16)
             call, kernel = self.prepared(a, False, b, False, c)
-            return {"name": "bf16 1024x4096x4096 (64 tiles of 256 x 256)", "call": call, "kernel": kernel,
+            return {"name": "bf16 1024x4096x4096 (64 tiles of 256 x 256 = 256 of 128 x 128)", "call": call, "kernel": kernel,
                     "flops": 2.0 * 1024 * 4096 * 4096, "bytes": (1024 * 4096 * 2 + 4096 * 4096) * 2, "bound": "mfma",
                     "dtype": "bf16", "steps": 200}
         if name == "fp16_4096":

@@ -265,6 +265,7 @@ hipError_t launch_mfma(const GemmProblem& p, int config, hipStream_t stream);
 int mfma_splitk_parts(const GemmProblem& p);
 bool mfma_prefers_splitk(const GemmProblem& p);
 bool mfma_prefers_tail(const GemmProblem& p);
+bool mfma_prefers_quarter(const GemmProblem& p);
 hipError_t launch_mfma_splitk(const GemmProblem& p, hipStream_t stream);
 
 bool skinny_supported(const GemmProblem& p);

@@ -1012,6 +1012,40 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
   return parts >= 8 || (parts >= 4 && (p.K >= 8192 || p.M <= 192 || th <= 96));
 }
 
+// Whether the 128 x 128 quarter tile is the choice: when one round of them holds the problem -- at most a quarter of
+// a device's worth of whole tiles -- and the k loop is not so long that cutting it over more units does better.  A
+// quarter tile's k loop runs 4.8 us per 1024 k on top of 5 us of launch, first fill and epilogue whatever the tile
+// count (one per unit), so its time does not depend on the tile count while that of split-K, shared tiles and half tiles
+// does.  Measured against what the other rules picked, all four layouts alike, us:
+//   K <= 2048       always: 2048^3 18.5 against 24.3-26.4 (half tiles), 1024 x 2048 x 2048 16.3 against 24.6, 512 x 512 x 1024
+//                   10.0 against 15.0, 128 x 512 x 512 (four tiles) 7.3 against 9.7
+//   K = 4096        from 48 tiles: 1024 x 4096 x 4096 (256) 31.8 against 42 (shared tiles), 512 x 4096 x 4096 (128) 25.5-26.9
+//                   against 38 (split-K), 256 x 4096 x 4096 (64) 25.5 against 28; 256 x 2048 x 4096 (32): 24.4 against 24-26 a tie,
+//                   128 x 2048 x 4096 (16): 25 against 18.5 (split-K in sixteen parts)
+//   K = 8192        from 112-128 tiles: 512 x 4096 x 8192 (128) 45-46 against 48-52 (split-K), 1024 x 4096 x 8192 (256) 59-60
+//                   against 63-66 (shared tiles); 65-96 tiles: 4-11 % behind
+//   two rounds (257-512 tiles): 3-20 % behind the half and whole tiles.
+// With 64 rows half of every tile is padding: against two k-contiguous operands the streaming kernel stays ahead (64 x 4096 x
+// 2048 x . W^T: 11.5 against 14.8), in the other layouts the tile still wins (x . W 14.8 against 16.7 streamed, x^T . W 14.9
+// against 21.1 in parts); with fewer rows it is not asked.
+bool mfma_prefers_quarter(const GemmProblem& p) {
+  const int config = mfma_config(p, 14);
+  if (config == 0 || p.M < 64 || p.N < 64 || (p.M == 64 && (config & 3) == 3)) return false;
+  const long long tq = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  if (tq > compute_units()) return false;
+  if (p.batch > 1) {
+    // A batch has no split-K pass, so few tiles and a long k loop are no exception (4 x 128 x 128 x 4096: 23.7 us against
+    // 40.3 shared; 16 x 128 x 128 x 4096 24.5 against 40.9; 4 x 384 x 384 x 4096 26 against 40).  But its problems share no
+    // operand: with more than half a device's worth of tiles from small problems the operand traffic, twice a half
+    // tile's, sets the pace (16 x 512 x 512 x 4096, 256 tiles: 66-75 us against 55-56 shared; 64 x 256 x 256 x 1024: 23.5
+    // against 18.7 in half tiles) -- unless a problem alone is 32 tiles or more (4 x 512 x 2048 x 4096: 34.5 against 47).
+    return 2 * tq <= compute_units() || tq / p.batch >= 32;
+  }
+  if (p.K <= 2048) return true;
+  if (p.K <= 4096) return tq >= 48;   // (512 x 1536 x 4096, 48 tiles: 25.3 against 28.4 in parts)
+  return tq * 73 >= p.K;              // 112 tiles at K = 8192
+}
+
 // Whether the heuristic takes the tail-sharing form of the 64-deep kernel (tile 10): the tiles left over
 // after the whole rounds are cut along k so that every compute unit works on them.  Adding up a tile's
 // parts costs about what three quads (768 k) of multiplying do, so it pays for long k loops only.  After

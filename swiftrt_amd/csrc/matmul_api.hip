@@ -148,6 +148,8 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
 }
 
 Plan heuristic_plan(const GemmProblem& p) {
+  // one round of 128 x 128 tiles holds the problem (64 rows or more) and its k loop is not worth cutting
+  if (srt::mfma_prefers_quarter(p)) return kPlanM16Q;
   if (srt::skinny_supported(p) && srt::skinny_preferred(p)) return kPlanSkinny;
   // Up to 64 rows against a long k loop, one round of the streaming kernel's workgroups: when split-K cannot cut the k
   // loop, or only in two (K / 4 not a whole number of stages; a batch has no split-K pass at all), the streaming kernel beats

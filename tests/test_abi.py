@@ -252,7 +252,7 @@ def test_plan_cache_file_round_trip_and_rejects_malformed_files(tmp_path):
     srt.PlanCache.clear()
     assert L.srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(ad), 0, ctypes.byref(ad), dummy, dummy, dummy,
                                   buf, 64) == 0
-    assert buf.value == b"mfma_128x256_m16_k64"
+    assert buf.value == b"mfma_128x128_m16_k128"
     assert L.srtPlanCacheCount(None) == native.ERROR_INVALID_VALUE
     assert L.srtPlanCacheLoad(None) == native.ERROR_INVALID_VALUE
 
@@ -283,40 +283,57 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_m16_k64"
     # few tiles and a long k loop: K split over the idle compute units -- when that buys more than the
     # half-height tiles a k-contiguous A allows
-    assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_256x256_splitk"           # eight parts
-    assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_256x256_splitk"
-    # 64 to 160 tiles: the tail-sharing form of the 64-deep kernel (every tile cut along k into two or three parts),
-    # unless half-height tiles fill one round as well
-    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_256x256_m16_k64_tail"
+    assert query(native.REAL16BF, 256, 2048, 4096) == "mfma_256x256_splitk"           # eight whole tiles in eight parts
+    assert query(native.REAL16BF, 256, 2048, 4096, tb=True) == "mfma_256x256_splitk"
+    # ... unless one round of 128 x 128 quarter tiles holds the problem and the k loop is short enough for them (K <= 2048: always;
+    # 4096: from 48 tiles; beyond: from K / 73 tiles)
+    assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_128x128_m16_k128"         # 128 quarter tiles (25.5 us against 38 in parts)
+    assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 512, 1536, 4096) == "mfma_128x128_m16_k128"         # 48
+    assert query(native.REAL16BF, 384, 1536, 4096) == "mfma_256x256_splitk"           # 36: parts
+    assert query(native.REAL16BF, 512, 2048, 8192) == "mfma_256x256_splitk"           # 64 at K = 8192: parts
+    assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_128x128_m16_k128"        # 256 quarter tiles (31.8 us against 42 shared)
+    # 64 to 160 whole tiles beyond one round of quarter tiles: the tail-sharing form of the 64-deep kernel (every tile cut
+    # along k into two or three parts), unless half-height tiles fill one round as well
     assert query(native.REAL16BF, 2048, 4096, 4096, tb=True) == "mfma_128x256_m16_k64"
     assert query(native.REAL16BF, 2048, 4096, 4096) == "mfma_128x256_m16_k64"
     assert query(native.REAL16BF, 2048, 4096, 8192) == "mfma_256x256_m16_k64_tail"
     assert query(native.REAL16BF, 4096, 10240, 4096) == "mfma_256x256_m16_k64"        # after whole rounds it buys nothing
-    assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_256x256_m16_k64_tail"    # 64 tiles again
-    assert query(native.REAL16BF, 1024, 2048, 8192) == "mfma_256x256_splitk"          # 32 tiles: eight parts
-    assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_256x256_splitk"
-    assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_256x128_m16_k64"    # A not k-contiguous: one round of its 256 x 128 half tiles
-    assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_256x128_m16_k64"    # (64 of them)
-    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_256x128_m16_k64"    # (32 of them, neither operand k-contiguous)
-    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x128_m16_k64"    # (256 of them: one round exactly)
+    assert query(native.REAL16BF, 2048, 2048, 8192) == "mfma_128x128_m16_k128"        # 256 quarter tiles, K = 8192 (59 us against 63-66 shared)
+    assert query(native.REAL16BF, 1024, 2048, 8192) == "mfma_128x128_m16_k128"        # 128 of them
+    assert query(native.REAL16BF, 256, 8192, 8192, ta=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 256, 4096, 8192, ta=True) == "mfma_256x256_splitk"      # 64: parts
+    assert query(native.REAL16BF, 1024, 2048, 2048, ta=True) == "mfma_128x128_m16_k128"   # any layout
+    assert query(native.REAL16BF, 1024, 2048, 1024, ta=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 1024, 1024, 1024, ta=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 1024, 8192, 2048, ta=True) == "mfma_256x128_m16_k64"    # 512 quarter tiles: A not k-contiguous, one round of its 256 x 128 half tiles
+    assert query(native.REAL16BF, 1024, 8192, 1920, ta=True) == "mfma_256x128_m16_k64"    # (so too where K is no whole number of 128-deep units)
+    assert query(native.REAL16BF, 1024, 2048, 1984, ta=True) == "mfma_256x128_m16_k64"
     # mid-size problems: the 256 x 256 kernels from 24 tiles up (96 when both operands are k-contiguous),
     # 64 x 64 tiles below, so that every CU gets a workgroup
     assert query(native.REAL16BF, 3072, 3072, 3072) == "mfma_256x256_m16_k64"             # 144 tiles, long k loop
     assert query(native.REAL16BF, 3072, 3072, 1024) == "mfma_256x256_m16_k64"             # and a short one
-    # a k-contiguous A and at most one round of 128 x 256 tiles: the half-height form of the 16x16x32 kernel
-    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x256_m16_k64"             # 128 half tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x256_m16_k64"
+    # a k-contiguous A and at most one round of 128 x 256 tiles: the half-height form of the 16x16x32 kernel -- beyond one
+    # round of quarter tiles, or where K is no whole number of their 128-deep units
+    assert query(native.REAL16BF, 2048, 2048, 2048) == "mfma_128x128_m16_k128"            # 256 quarter tiles (18.5 us against 24-26 in half tiles)
+    assert query(native.REAL16BF, 2048, 2048, 2048, tb=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 2048, 2048, 1984) == "mfma_128x256_m16_k64"             # 128 half tiles
+    assert query(native.REAL16BF, 2048, 2048, 1984, tb=True) == "mfma_128x256_m16_k64"
     assert query(native.REAL16BF, 2048, 4096, 2048) == "mfma_128x256_m16_k64"             # 256 half tiles
-    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_256x128_m16_k64"    # A not k-contiguous: its half tile is 256 x 128
-    assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_256x128_m16_k64"
+    assert query(native.REAL16BF, 2048, 2048, 2048, ta=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 2048, 2048, 1984, ta=True) == "mfma_256x128_m16_k64"    # A not k-contiguous: its half tile is 256 x 128
+    assert query(native.REAL16BF, 2048, 2048, 1024, ta=True) == "mfma_128x128_m16_k128"
     # 258 whole tiles: a whole round, and the two left over cut along k in three parts each
     assert query(native.REAL16BF, 1536, 11008, 4096) == "mfma_256x256_m16_k64_tail"
     assert query(native.REAL16BF, 1536, 11008, 4096, tb=True) == "mfma_256x256_m16_k64_tail"
     assert query(native.REAL16BF, 1536, 11008, 2048) == "mfma_256x256_m16_k64"        # (not for a k loop this short)
     assert query(native.REAL16BF, 1536, 4096, 11008, tb=True) == "mfma_256x256_m16_k64_tail"   # 96 tiles, two parts each
-    assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x256_m16_k64"              # 8 half tiles
-    assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
-    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x256_m16_k64"              # K too short to split
+    assert query(native.REAL16BF, 256, 1024, 1024) == "mfma_128x128_m16_k128"             # 16 quarter tiles
+    assert query(native.REAL16BF, 256, 1024, 960) == "mfma_128x256_m16_k64"               # 8 half tiles
+    assert query(native.REAL16BF, 1024, 1024, 2048, tb=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 1024, 1024, 1984, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
+    assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 512, 4096, 1984) == "mfma_128x256_m16_k64"              # K too short to split
     assert query(native.REAL16BF, 512, 4096, 256) == "mfma_128x256_m16_k64"               # short k loops too (8.4 us against 10.0)
     assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
@@ -326,15 +343,17 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 64, 4096, 4096, tb=True) == "skinny"                # 128 of 32, short enough k loop
     assert query(native.REAL16BF, 64, 4096, 14336, tb=True) == "mfma_256x256_splitk"  # few workgroups, long k loop
     assert query(native.REAL16BF, 64, 11008, 4096, tb=True) == "mfma_256x256_splitk"  # 344 workgroups: not one round
-    assert query(native.REAL16BF, 65, 14336, 4096, tb=True) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 65, 14336, 4096, tb=True) == "mfma_128x128_m16_k128"  # 112 quarter tiles, half padding
+    assert query(native.REAL16BF, 65, 14336, 4032, tb=True) == "mfma_256x256_splitk"
     # x . W with an n-contiguous W: the streaming kernel within one round of 64-column workgroups and a short k loop
     assert query(native.REAL16BF, 8, 14336, 4096) == "skinny"
     assert query(native.REAL16BF, 32, 4096, 2048) == "skinny"
     assert query(native.REAL16BF, 32, 4096, 4096) == "mfma_256x256_splitk"            # 64 workgroups, 17..32 rows
     assert query(native.REAL16BF, 8, 4096, 8192) == "mfma_256x256_splitk"             # long k loop
     assert query(native.REAL16BF, 8, 28672, 1024) == "mfma_128x256_m16_k64"               # 448 workgroups: not one round
-    assert query(native.REAL16BF, 64, 14336, 4096) == "skinny"
-    assert query(native.REAL16BF, 64, 11008, 4096) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 64, 14336, 4096) == "mfma_128x128_m16_k128"         # 64 rows against an n-contiguous W: quarter tiles from 48 up
+    assert query(native.REAL16BF, 64, 11008, 4096) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 64, 14336, 4032) == "skinny"
     # what sweeps against every pinned plan found (the measured pairs stand next to the rules in csrc/gemm_mfma.hip)
     assert query(native.REAL16BF, 24, 96, 10320) == "skinny"                          # K / 2 is not a whole number of stages: no split-K
     assert query(native.REAL16BF, 8, 1288, 10432) == "skinny"                         # only two parts possible
@@ -343,7 +362,8 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 192, 12568, 3264, ta=True, tb=True) == "mfma_256x128_m16_k64"   # K only halves: one round of half tiles beats two parts
     assert query(native.REAL16BF, 664, 7536, 352, tb=True) == "mfma_128x256_m16"      # 13 % padding rows are fine for half tiles
     assert query(native.REAL16BF, 169, 9824, 504, tb=True) == "mfma_64x64"            # a second row of half tiles that is mostly padding is not
-    assert query(native.REAL16BF, 512, 512, 1024, ta=True) == "mfma_256x128_m16_k64"   # eight half tiles, neither operand k-contiguous: ahead of split-K
+    assert query(native.REAL16BF, 512, 512, 1024, ta=True) == "mfma_128x128_m16_k128"  # sixteen quarter tiles (9.9 us against 15.8 in half tiles)
+    assert query(native.REAL16BF, 512, 512, 960, ta=True) == "mfma_256x128_m16_k64"    # eight half tiles, neither operand k-contiguous: ahead of split-K
     # batches (no split-K pass)
     def query_batched(dt, B, M, N, K, ta=False, tb=False):
         ashape = (B, K, M) if ta else (B, M, K)
@@ -357,10 +377,13 @@ def test_kernel_selection_is_queryable_without_gpu():
         return buf.value.decode()
     assert query_batched(native.REAL16F, 32, 256, 256, 256, tb=True) == "mfma_64x64"                   # benchmark config 2: launch-sized, every CU a workgroup
     assert query_batched(native.REAL16BF, 16, 384, 384, 1024, tb=True) == "mfma_128x256_m16_k64"       # 96 half tiles of a batch, 64 deep
-    assert query_batched(native.REAL16BF, 16, 64, 512, 1024, ta=True) == "mfma_256x128_m16_k64"        # 64 tiles of 256 x 128, A not k-contiguous
-    assert query_batched(native.REAL16BF, 4, 256, 256, 4096, ta=True) == "mfma_256x256_m16_k64_tail"   # four tiles cut along k
-    assert query_batched(native.REAL16BF, 16, 256, 256, 2048, ta=True, tb=True) == "mfma_256x256_m16_k64_tail"
-    assert query_batched(native.REAL16BF, 4, 128, 128, 4096, tb=True) == "mfma_64x64"                  # mostly padding, both k-contiguous
+    assert query_batched(native.REAL16BF, 16, 64, 512, 1024, ta=True) == "mfma_128x128_m16_k128"       # 64 quarter tiles, half padding
+    assert query_batched(native.REAL16BF, 16, 64, 512, 960, ta=True) == "mfma_256x128_m16_k64"         # 64 tiles of 256 x 128, A not k-contiguous
+    assert query_batched(native.REAL16BF, 4, 256, 256, 4096, ta=True) == "mfma_128x128_m16_k128"       # 16 quarter tiles (24 us against 40 shared: a batch has no split-K)
+    assert query_batched(native.REAL16BF, 16, 256, 256, 2048, ta=True, tb=True) == "mfma_128x128_m16_k128"
+    assert query_batched(native.REAL16BF, 4, 128, 128, 4096, tb=True) == "mfma_128x128_m16_k128"
+    assert query_batched(native.REAL16BF, 4, 128, 128, 4032, tb=True) == "mfma_64x64"                  # mostly padding, both k-contiguous
+    assert query_batched(native.REAL16BF, 16, 512, 512, 4096) == "mfma_256x256_m16_k64_tail"           # 256 quarter tiles of small problems: operand traffic
     assert query_batched(native.REAL16BF, 64, 256, 256, 1024, tb=True) == "mfma_128x256_m16_k64"           # 128 half tiles in one round
     assert query_batched(native.REAL16BF, 64, 256, 1024, 256, tb=True) == "mfma_256x256_m16_k64"       # 512 half tiles: whole tiles
     assert query_batched(native.REAL16BF, 64, 384, 384, 4096, tb=True) == "mfma_256x256_k64"           # a last row of tiles half padding

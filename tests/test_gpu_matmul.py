@@ -717,13 +717,17 @@ def test_splitk_epilogues_vs_oracle_and_nan(act, tmp_path):
 
 
 def test_splitk_is_the_choice_for_few_tiles_and_long_k():
-    a = srt.Tensor(H.encode(np.zeros((512, 4096), np.float32), H.BF16))
-    b = srt.Tensor(H.encode(np.zeros((4096, 4096), np.float32), H.BF16))
-    out = srt.Tensor(shape=[512, 4096], dtype=a.dtype)
-    assert query_kernel(a, False, b, False, out) == "mfma_256x256_splitk"
-    a2 = srt.Tensor(H.encode(np.zeros((512, 2048), np.float32), H.BF16))       # K = 2048: not worth the extra pass
-    b2 = srt.Tensor(H.encode(np.zeros((2048, 4096), np.float32), H.BF16))
+    a = srt.Tensor(H.encode(np.zeros((256, 4096), np.float32), H.BF16))
+    b = srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16))
+    out = srt.Tensor(shape=[256, 2048], dtype=a.dtype)
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_splitk"      # eight whole tiles = 32 quarter tiles
+    a2 = srt.Tensor(H.encode(np.zeros((256, 2048), np.float32), H.BF16))       # K = 2048: not worth the extra pass
+    b2 = srt.Tensor(H.encode(np.zeros((2048, 2048), np.float32), H.BF16))
     assert query_kernel(a2, False, b2, False, out) != "mfma_256x256_splitk"
+    a3 = srt.Tensor(H.encode(np.zeros((512, 4096), np.float32), H.BF16))       # 128 quarter tiles: one round of those instead
+    b3 = srt.Tensor(H.encode(np.zeros((4096, 4096), np.float32), H.BF16))
+    out3 = srt.Tensor(shape=[512, 4096], dtype=a.dtype)
+    assert query_kernel(a3, False, b3, False, out3) == "mfma_128x128_m16_k128"
 
 
 # ---- the 128 x 256 form of the 16x16x32 kernel ---------------------------------------------------------

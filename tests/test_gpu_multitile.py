@@ -326,7 +326,7 @@ def test_column_major_dense_through_the_flipped_kernels(dt):
     srt.PlanCache.clear()
     r = H.rng(808)
     relu = srt.ActivationType.relu
-    for (M, N, K, want) in [(2056, 4088, 512, DEEP), (1024, 4096, 4096, TAIL), (1016, 4088, 4096, TAIL)]:
+    for (M, N, K, want) in [(2056, 4088, 512, DEEP), (3072, 1536, 8192, TAIL), (3064, 1528, 8192, TAIL), (1016, 4088, 4096, QUARTER)]:
         a = r.integers(-2, 3, (M, K)).astype(np.float32)
         w = r.integers(-2, 3, (K, N)).astype(np.float32)
         bias = r.integers(-40, 41, N).astype(np.float32)
@@ -419,22 +419,26 @@ def test_tail_sharing_batched_clipped_and_repeatable(tmp_path):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-def test_few_tile_batches_with_long_k_share_their_tiles(ta, tb):
-    """A batch has no split-K pass; the heuristic cuts its few tiles along k with the tail-sharing kernel.
-    Every tile of the launch is a shared one here (three parts each), the batches have their own operands,
-    and the tiles have ragged edges: integer operands, bit-exact in every layout, unpinned."""
-    srt.PlanCache.clear()
+def test_few_tile_batches_with_long_k(ta, tb, tmp_path):
+    """A batch has no split-K pass.  The heuristic gives its few tiles to the 128 x 128 quarter tile (one round of them);
+    pinned, the tail-sharing kernel cuts every tile of the launch along k (three parts each).  The batches have their own
+    operands and the tiles have ragged edges: integer operands, bit-exact in every layout, both ways."""
     r = H.rng(515)
     for (B_, M, N, K, dt) in [(4, 256, 256, 4096, H.BF16), (5, 200, 520, 4096, H.F16), (16, 136, 144, 8192, H.BF16)]:
         a = r.integers(-2, 3, (B_, K, M) if ta else (B_, M, K)).astype(np.float32)
         w = r.integers(-2, 3, (B_, N, K) if tb else (B_, K, N)).astype(np.float32)
         at, wt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(w, dt))
-        out = srt.matmul(at, wt, ta, tb)
-        assert query_kernel(at, ta, wt, tb, out) == TAIL, (B_, M, N, K)
         am = np.swapaxes(a, 1, 2) if ta else a
         wm = np.swapaxes(w, 1, 2) if tb else w
         exact = np.einsum("bmk,bkn->bmn", am.astype(np.int64), wm.astype(np.int64))
-        assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt)), (B_, M, N, K)
+        for plan in (QUARTER, TAIL):
+            srt.PlanCache.clear()
+            if plan == TAIL:
+                pin(tmp_path, TAIL, dt, M, N, K, ta, tb, batch=B_)
+            out = srt.matmul(at, wt, ta, tb)
+            assert query_kernel(at, ta, wt, tb, out) == plan, (B_, M, N, K)
+            assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt)), (plan, B_, M, N, K)
+    srt.PlanCache.clear()
 
 
 def test_tail_sharing_on_two_queues_at_once():
@@ -446,7 +450,7 @@ def test_tail_sharing_on_two_queues_at_once():
     q0, q1 = p.devices[1].queues[0], p.devices[1].queues[1]
     r = H.rng(616)
     jobs = []
-    for (q, (M, N, K)) in [(q0, (1024, 4096, 4096)), (q1, (2048, 2048, 8192))]:
+    for (q, (M, N, K)) in [(q0, (3072, 3072, 4096)), (q1, (3072, 1536, 8192))]:
         a = r.integers(-2, 3, (M, K)).astype(np.float32)
         w = r.integers(-2, 3, (N, K)).astype(np.float32)
         at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
