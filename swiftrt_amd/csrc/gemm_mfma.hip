@@ -1027,19 +1027,26 @@ bool mfma_prefers_splitk(const GemmProblem& p) {
 //   two rounds (257-512 tiles): 3-20 % behind the half and whole tiles.
 // With 64 rows half of every tile is padding: against two k-contiguous operands the streaming kernel stays ahead (64 x 4096 x
 // 2048 x . W^T: 11.5 against 14.8), in the other layouts the tile still wins (x . W 14.8 against 16.7 streamed, x^T . W 14.9
-// against 21.1 in parts); with fewer rows it is not asked.
+// against 21.1 in parts).  With fewer rows a k-contiguous A goes to the streaming kernel or split-K; one that is not has
+// neither a streaming kernel nor a 128-row half tile, and the tile wins although it is mostly padding (8 x 14336 x 4096 x^T . W^T
+// 25.7 against 31.8 in parts, x^T . W 29.0 against 32.1; 32 x 4096 x 2048 16.8 against 20.9; 16 x 4096 x 1024 17.1 against 20.2).
 bool mfma_prefers_quarter(const GemmProblem& p) {
   const int config = mfma_config(p, 14);
-  if (config == 0 || p.M < 64 || p.N < 64 || (p.M == 64 && (config & 3) == 3)) return false;
+  const bool a_kc = (config & 2) != 0, b_kc = (config & 1) != 0;
+  if (config == 0 || p.N < 64) return false;
+  if (a_kc && (p.M < 64 || (p.M == 64 && b_kc))) return false;
   const long long tq = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (tq > compute_units()) return false;
   if (p.batch > 1) {
     // A batch has no split-K pass, so few tiles and a long k loop are no exception (4 x 128 x 128 x 4096: 23.7 us against
-    // 40.3 shared; 16 x 128 x 128 x 4096 24.5 against 40.9; 4 x 384 x 384 x 4096 26 against 40).  But its problems share no
-    // operand: with more than half a device's worth of tiles from small problems the operand traffic, twice a half
-    // tile's, sets the pace (16 x 512 x 512 x 4096, 256 tiles: 66-75 us against 55-56 shared; 64 x 256 x 256 x 1024: 23.5
+    // 40.3 shared; 16 x 128 x 128 x 4096 24.5 against 40.9; 16 x 384 x 384 x 4096, 144 tiles: 45 against 49-56).  But its
+    // problems share no operand: with a device's worth of tiles from small problems the operand traffic, twice a half
+    // tile's, sets the pace (16 x 512 x 512 x 4096, 256 tiles: 61-75 us against 55-56 shared; 64 x 256 x 256 x 1024: 23.5
     // against 18.7 in half tiles) -- unless a problem alone is 32 tiles or more (4 x 512 x 2048 x 4096: 34.5 against 47).
-    return 2 * tq <= compute_units() || tq / p.batch >= 32;
+    if (4 * tq <= 3 * compute_units() || tq / p.batch >= 32) return true;
+    // (an A that is not k-contiguous has no 128-row half tile to fall back on: 64-row problems, 64 x 64 x 512 x 1024 17-18
+    // against 19-23, x 4096: 60 against 70-72; x^T . W with a short k loop, 16 x 256 x 1024 x 1024 18.5 against 23.6)
+    return !a_kc && (p.M <= 64 || (!b_kc && p.K <= 1024));
   }
   if (p.K <= 2048) return true;
   if (p.K <= 4096) return tq >= 48;   // (512 x 1536 x 4096, 48 tiles: 25.3 against 28.4 in parts)

@@ -363,6 +363,9 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 664, 7536, 352, tb=True) == "mfma_128x256_m16"      # 13 % padding rows are fine for half tiles
     assert query(native.REAL16BF, 169, 9824, 504, tb=True) == "mfma_64x64"            # a second row of half tiles that is mostly padding is not
     assert query(native.REAL16BF, 512, 512, 1024, ta=True) == "mfma_128x128_m16_k128"  # sixteen quarter tiles (9.9 us against 15.8 in half tiles)
+    assert query(native.REAL16BF, 8, 14336, 4096, ta=True, tb=True) == "mfma_128x128_m16_k128"   # a handful of rows of an m-contiguous A: no streaming kernel, 112 quarter tiles beat the parts
+    assert query(native.REAL16BF, 32, 4096, 2048, ta=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16BF, 32, 4096, 4096, ta=True) == "mfma_256x256_splitk"              # 32 tiles at K = 4096: parts
     assert query(native.REAL16BF, 512, 512, 960, ta=True) == "mfma_256x128_m16_k64"    # eight half tiles, neither operand k-contiguous: ahead of split-K
     # batches (no split-K pass)
     def query_batched(dt, B, M, N, K, ta=False, tb=False):
@@ -376,7 +379,8 @@ def test_kernel_selection_is_queryable_without_gpu():
         assert L.srtMatmulQueryKernel(ctypes.byref(ad), int(ta), ctypes.byref(bd), int(tb), ctypes.byref(od), p, p, p, buf, 64) == 0
         return buf.value.decode()
     assert query_batched(native.REAL16F, 32, 256, 256, 256, tb=True) == "mfma_64x64"                   # benchmark config 2: launch-sized, every CU a workgroup
-    assert query_batched(native.REAL16BF, 16, 384, 384, 1024, tb=True) == "mfma_128x256_m16_k64"       # 96 half tiles of a batch, 64 deep
+    assert query_batched(native.REAL16BF, 16, 384, 384, 1024, tb=True) == "mfma_128x128_m16_k128"      # 144 quarter tiles of a batch (15.0 us against 16.1 in half tiles)
+    assert query_batched(native.REAL16BF, 16, 384, 384, 960, tb=True) == "mfma_128x256_m16_k64"        # 96 half tiles of a batch, 64 deep
     assert query_batched(native.REAL16BF, 16, 64, 512, 1024, ta=True) == "mfma_128x128_m16_k128"       # 64 quarter tiles, half padding
     assert query_batched(native.REAL16BF, 16, 64, 512, 960, ta=True) == "mfma_256x128_m16_k64"         # 64 tiles of 256 x 128, A not k-contiguous
     assert query_batched(native.REAL16BF, 4, 256, 256, 4096, ta=True) == "mfma_128x128_m16_k128"       # 16 quarter tiles (24 us against 40 shared: a batch has no split-K)

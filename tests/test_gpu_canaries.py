@@ -146,6 +146,17 @@ def test_every_plan_keeps_inside_batched_views_with_gaps(dt, tmp_path):
         assert "mfma_256x256_m16_k64" in ran and "mfma_64x64" in ran and "generic" in ran, ran
 
 
+def test_quarter_tile_keeps_inside_small_and_batched_views(tmp_path):
+    """The 128 x 128 tile on results much smaller than a tile (8 and 40 rows of an m-contiguous A, 72 columns), on ragged
+    edges in both directions, and on batches whose matrices lie two apart with sentinel columns either side of every row."""
+    Q = ("mfma_128x128_m16_k128",)
+    for (M, N, K, batch, ta, tb) in [(8, 72, 512, 1, True, False), (40, 1096, 640, 1, True, True), (136, 200, 512, 1, False, False),
+                                     (264, 328, 512, 3, False, True), (72, 136, 1024, 5, True, False)]:
+        for dt in (H.BF16, H.F16):
+            ran = run_matmul_case(tmp_path, dt, M, N, K, batch, ta, tb, Q, 730 + M + batch)
+            assert ran == list(Q), (M, N, K, batch, ta, tb, dt)
+
+
 def test_plans_for_unaligned_views_keep_inside(tmp_path):
     """N not a multiple of 8, odd row pitches and bases off a 16-byte boundary: the element-wise staging kernels
     and the generic kernel (the 16-byte store paths do not qualify and must not be chosen)."""
