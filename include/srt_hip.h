@@ -226,7 +226,7 @@ srtStatus srtMatmulBiasActivation(const void* a, const srtTensorDescriptor* aDes
                                   void* out, const srtTensorDescriptor* oDesc, srtStream stream);
 
 /* Name of the kernel family the dispatcher selects for this problem ("mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail",
- * "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_256x256_m16", "mfma_256x256", "skinny", "generic", ...; the full
+ * "mfma_128x128_m16_k128", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_256x256_m16", "mfma_256x256", "skinny", "generic", ...; the full
  * list is with srtMatmulTune), written into `name`; nothing is launched.  A 16-bit problem
  * whose operands span 1 Gi elements or more runs as several launches over halves of its batch, M or N;
  * the name is then that of the first piece's kernel followed by "/pieces".  Diagnostic only
@@ -257,6 +257,8 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
  * "mfma_256x256_m16_k64_split" (the same kernel with its last round in 192-wide tiles: only ever a tuned or loaded plan),
  * "mfma_128x256_m16_k64" and "mfma_256x128_m16_k64" (the same kernel body on half tiles, for grids that would leave compute
  * units idle in 256 x 256 tiles: 128 rows when A is contiguous along k, 128 columns when it is not),
+ * "mfma_128x128_m16_k128" (128 x 128 tiles on 128-deep staging units, any layout, K a multiple of 128 and at least 512: what
+ * problems of up to one tile per compute unit run on),
  * "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
  * "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any" (16-bit
  * operands of any stride and alignment), "skinny", "f32_mfma_64x64", "f32_mfma_splitk", "generic").
