@@ -162,7 +162,7 @@ def test_mfma_tiles_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, M, N, K, ke
     b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
     a_st, b_st = H.encode(a, dt), H.encode(b, dt)
     got = gpu_matmul(a_st, b_st, ta, tb, want_kernel=kernel)
-    exact = (np.swapaxes(a, 0, 1) if ta else a).astype(np.int64) @ (np.swapaxes(b, 0, 1) if tb else b).astype(np.int64)
+    exact = (np.swapaxes(a, 0, 1) if ta else a).astype(np.float64) @ (np.swapaxes(b, 0, 1) if tb else b).astype(np.float64)
     assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
     a = (r.standard_normal(a.shape) / np.sqrt(K)).astype(np.float32)
     b = r.standard_normal(b.shape).astype(np.float32)
@@ -184,7 +184,7 @@ def test_result_view_with_odd_pitch_takes_the_128_tile(dt):
     out = big[:, :N]
     assert query_kernel(at, False, bt, False, out) == "mfma_128x128"
     srt.current_queue().matmul(at, False, bt, False, out)
-    exact = a.astype(np.int64) @ b.astype(np.int64)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
     assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), dt))
     assert np.all(H.decode(big.array()[:, N:]) == 0)          # the padding columns are untouched
 
@@ -229,7 +229,7 @@ def test_f32_split_k_row_major_ragged_and_batched():
         a = r.integers(-3, 4, lead + (M, K)).astype(np.float32)
         b = r.integers(-3, 4, lead + (K, N)).astype(np.float32)
         got = gpu_matmul(a, b, want_kernel="f32_mfma")
-        assert np.array_equal(got, (a.astype(np.int64) @ b.astype(np.int64)).astype(np.float32)), (M, N, K)
+        assert np.array_equal(got, (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)), (M, N, K)
         a = r.uniform(-1, 1, a.shape).astype(np.float32)
         b = r.uniform(-1, 1, b.shape).astype(np.float32)
         check_against_fp64(gpu_matmul(a, b), a, b, False, False, H.F32)
@@ -252,7 +252,7 @@ def test_f32_128_tile_all_layouts_ragged(ta, tb):
     a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
     b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
     got = gpu_matmul(a, b, ta, tb, want_kernel="f32_mfma")
-    exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+    exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
     assert np.array_equal(got, exact.astype(np.float32))
     a = r.uniform(-1, 1, a.shape).astype(np.float32)
     b = r.uniform(-1, 1, b.shape).astype(np.float32)
@@ -271,7 +271,7 @@ def test_f32_128_tile_all_layouts_ragged(ta, tb):
         av = srt.Tensor(padded)[:, :K]
         bi = r.integers(-3, 4, (K, N)).astype(np.float32)
         out2 = srt.matmul(av, srt.Tensor(bi))
-        assert np.array_equal(out2.array(), (av_host.astype(np.int64) @ bi.astype(np.int64)).astype(np.float32))
+        assert np.array_equal(out2.array(), (av_host.astype(np.float64) @ bi.astype(np.float64)).astype(np.float32))
 
 
 def test_cfg2_f16_batched_transpose_rhs():
@@ -353,7 +353,7 @@ def test_skinny_ragged_and_integer_exact(dt):
         x = r.integers(-2, 3, (M, K)).astype(np.float32)
         w = r.integers(-2, 3, (N, K)).astype(np.float32)
         got = gpu_matmul(H.encode(x, dt), H.encode(w, dt), tb=True, want_kernel="skinny")
-        exact = (x.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32)
+        exact = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32)
         assert np.array_equal(got.view(np.uint16), H.encode(exact, dt).view(np.uint16)), (M, N, K)
 
 
@@ -370,7 +370,7 @@ def test_skinny_wide_groups_integer_exact_bias_and_batch(dt):
         out = srt.Tensor(shape=[M, N], dtype=xt.dtype)
         assert query_kernel(xt, False, wt, True, out) == "skinny"
         srt.current_queue().matmul(xt, False, wt, True, out, bias=bt, activation=srt.ActivationType.relu)
-        exact = np.maximum(x.astype(np.int64) @ w.astype(np.int64).T + b.astype(np.int64)[None, :], 0)
+        exact = np.maximum(x.astype(np.float64) @ w.astype(np.float64).T + b.astype(np.float64)[None, :], 0)
         assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
     B_, M, N, K = 4, 32, 3100, 136        # 4 x 49 workgroups of 64 columns
     x = r.integers(-2, 3, (B_, M, K)).astype(np.float32)
@@ -378,7 +378,7 @@ def test_skinny_wide_groups_integer_exact_bias_and_batch(dt):
     xt, wt = srt.Tensor(H.encode(x, dt)), srt.Tensor(H.encode(w, dt))
     out = srt.matmul(xt, wt, transposed_rhs=True)
     assert query_kernel(xt, False, wt, True, out) == "skinny"
-    exact = x.astype(np.int64) @ np.swapaxes(w, 1, 2).astype(np.int64)
+    exact = x.astype(np.float64) @ np.swapaxes(w, 1, 2).astype(np.float64)
     assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16))
 
 
@@ -585,7 +585,7 @@ def test_m16_kernel_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
         a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
         b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
         got = gpu_matmul(H.encode(a, dt), H.encode(b, dt), ta, tb, want_kernel="mfma_256x256_m16")
-        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
         assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
     M, N, K = 2040, 2056, 264
     pin_m16(tmp_path, dt, M, N, K, ta, tb)
@@ -632,7 +632,7 @@ def test_m16_kernel_batched_short_k_and_nan(tmp_path):
         at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
         out = srt.matmul(at, wt)
         assert query_kernel(at, False, wt, False, out) == "mfma_256x256_m16"
-        exact = a.astype(np.int64) @ w.astype(np.int64)
+        exact = a.astype(np.float64) @ w.astype(np.float64)
         assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), H.BF16)), K
     M = N = 1536
     a = np.zeros((M, 64), np.float32)
@@ -676,7 +676,7 @@ def test_splitk_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
         a = r.integers(-2, 3, (K, M) if ta else (M, K)).astype(np.float32)
         b = r.integers(-2, 3, (N, K) if tb else (K, N)).astype(np.float32)
         got = gpu_matmul(H.encode(a, dt), H.encode(b, dt), ta, tb, want_kernel="mfma_256x256_splitk")
-        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
         assert np.array_equal(got.view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
     M, N, K = 520, 776, 2048
     pin_plan(tmp_path, "mfma_256x256_splitk", dt, M, N, K, ta, tb)
@@ -842,7 +842,7 @@ def test_k64_kernel_batched_short_k_and_nan(tmp_path):
         pin_plan_for_shape(tmp_path, "mfma_256x256_k64", H.BF16, M, N, K, batch=B_)
         out = srt.matmul(at, wt, transposed_rhs=True)
         assert query_kernel(at, False, wt, True, out) == "mfma_256x256_k64"
-        exact = a.astype(np.int64) @ np.swapaxes(w, 1, 2).astype(np.int64)
+        exact = a.astype(np.float64) @ np.swapaxes(w, 1, 2).astype(np.float64)
         assert np.array_equal(out.array(), H.encode(exact.astype(np.float32), H.BF16)), K
     a = np.zeros((3584, 64), np.float32)
     w = np.zeros((3584, 64), np.float32)
@@ -870,7 +870,7 @@ def test_ring_kernel_batched_broadcast_and_column_major(dt, tmp_path):
     pin_plan_for_shape(tmp_path, "mfma_256x256", dt, M, N, K, batch=B_)
     assert query_kernel(at, False, w3, False, out) == "mfma_256x256"
     got = srt.matmul(at, w3).array()
-    exact = H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), dt)
+    exact = H.encode((a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), dt)
     assert np.array_equal(got.view(np.uint16), exact.view(np.uint16))
     # broadcast weight: same storage for every batch (batch stride 0), built as a view descriptor by hand
     q = srt.current_queue()
@@ -890,7 +890,7 @@ def test_ring_kernel_batched_broadcast_and_column_major(dt, tmp_path):
     pin_plan_for_shape(tmp_path, "mfma_256x256", dt, M2, N2, K2)
     yc = srt.matmul(xc, wc, bias=srt.Tensor(H.encode(b2, dt)))
     assert yc.order == srt.Order.col and query_kernel(xc, False, wc, False, yc) == "mfma_256x256"
-    want = H.encode((x.astype(np.int64) @ w2.astype(np.int64) + b2.astype(np.int64)[None, :]).astype(np.float32), dt)
+    want = H.encode((x.astype(np.float64) @ w2.astype(np.float64) + b2.astype(np.float64)[None, :]).astype(np.float32), dt)
     assert np.array_equal(yc.array().view(np.uint16), want.view(np.uint16))
     # and relu on top (bias per row after the transposition inside the library)
     layer = srt.Dense(wc, srt.Tensor(H.encode(b2, dt)), srt.ActivationType.relu)

@@ -162,7 +162,7 @@ def test_quarter_tile_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path)
         out = srt.Tensor(shape=[M, N], dtype=H.NP_STORAGE[dt])
         assert query_kernel(at, ta, bt, tb, out) == QUARTER
         srt.current_queue().matmul(at, ta, bt, tb, out)
-        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
         assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
     M, N, K = 2040, 2056, 1024
     pin(tmp_path, QUARTER, dt, M, N, K, ta, tb)
@@ -211,7 +211,7 @@ def test_quarter_tile_batched_and_nan(tmp_path):
     at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
     out = srt.matmul(at, wt)
     assert query_kernel(at, False, wt, False, out) == QUARTER
-    assert np.array_equal(out.array(), H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), H.BF16))
+    assert np.array_equal(out.array(), H.encode((a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), H.BF16))
     M = N = 768
     K = 512
     a = np.zeros((M, K), np.float32)
@@ -249,7 +249,7 @@ def test_k64_m16_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
         out = srt.Tensor(shape=[M, N], dtype=H.NP_STORAGE[dt])
         assert query_kernel(at, ta, bt, tb, out) == DEEP
         srt.current_queue().matmul(at, ta, bt, tb, out)
-        exact = (a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
         assert np.array_equal(out.array().view(np.uint16), H.encode(exact.astype(np.float32), dt).view(np.uint16)), (M, N, K)
     M, N, K = 2040, 2056, 512
     pin(tmp_path, DEEP, dt, M, N, K, ta, tb)
@@ -299,7 +299,7 @@ def test_k64_m16_batched_column_major_and_nan(tmp_path):
     at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
     out = srt.matmul(at, wt)
     assert query_kernel(at, False, wt, False, out) == DEEP
-    assert np.array_equal(out.array(), H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), H.BF16))
+    assert np.array_equal(out.array(), H.encode((a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), H.BF16))
     M = N = 1536
     K = 256
     a = np.zeros((M, K), np.float32)
@@ -395,7 +395,7 @@ def test_tail_sharing_batched_clipped_and_repeatable(tmp_path):
     at, wt = srt.Tensor(H.encode(a, H.BF16)), srt.Tensor(H.encode(w, H.BF16))
     out = srt.matmul(at, wt)
     assert query_kernel(at, False, wt, False, out) == TAIL
-    assert np.array_equal(out.array(), H.encode((a.astype(np.int64) @ w.astype(np.int64)).astype(np.float32), H.BF16))
+    assert np.array_equal(out.array(), H.encode((a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), H.BF16))
 
     M, N, K = 2048, 4096, 4096
     x = srt.Tensor(H.encode((r.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32), H.BF16))
@@ -430,7 +430,7 @@ def test_few_tile_batches_with_long_k(ta, tb, tmp_path):
         at, wt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(w, dt))
         am = np.swapaxes(a, 1, 2) if ta else a
         wm = np.swapaxes(w, 1, 2) if tb else w
-        exact = np.einsum("bmk,bkn->bmn", am.astype(np.int64), wm.astype(np.int64))
+        exact = am.astype(np.float64) @ wm.astype(np.float64)   # (small integers: exact in fp64)
         for plan in (QUARTER, TAIL):
             srt.PlanCache.clear()
             if plan == TAIL:
@@ -457,7 +457,7 @@ def test_tail_sharing_on_two_queues_at_once():
         outs = [srt.Tensor(shape=[M, N], dtype=np.uint16) for _ in range(6)]
         assert query_kernel(at, False, wt, True, outs[0]) == TAIL, (M, N, K)
         at.device_read(q); wt.device_read(q)
-        want = H.encode((a.astype(np.int64) @ w.astype(np.int64).T).astype(np.float32), H.BF16)
+        want = H.encode((a.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32), H.BF16)
         jobs.append((q, at, wt, outs, want))
     q0.wait_for_completion(); q1.wait_for_completion()
     for i in range(6):
@@ -506,8 +506,8 @@ def test_tail_sharing_every_way_of_cutting(tmp_path):
         # and a sampled row of each batch against the exact product
         for z in range(batch):
             row = int(r.integers(0, M))
-            a_row = (a[z][:, row] if ta else a[z][row]).astype(np.int64)
-            b_mat = (b[z].T if tb else b[z]).astype(np.int64)
+            a_row = (a[z][:, row] if ta else a[z][row]).astype(np.float64)
+            b_mat = (b[z].T if tb else b[z]).astype(np.float64)
             want = H.encode((a_row @ b_mat).astype(np.float32), dt)
             assert np.array_equal(got[TAIL][z, row].view(np.uint16), want.view(np.uint16)), (tm, tn, z, row)
 
