@@ -257,7 +257,7 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
  * "mfma_256x256_m16_k64_split" (the same kernel with its last round in 192-wide tiles: only ever a tuned or loaded plan),
  * "mfma_128x256_m16_k64" and "mfma_256x128_m16_k64" (the same kernel body on half tiles, for grids that would leave compute
  * units idle in 256 x 256 tiles: 128 rows when A is contiguous along k, 128 columns when it is not),
- * "mfma_128x128_m16_k128" (128 x 128 tiles on 128-deep staging units, any layout, K a multiple of 128 and at least 512: what
+ * "mfma_128x128_m16_k128" (128 x 128 tiles on 128-deep staging units, any layout, K a multiple of 128 and at least 256: what
  * problems of up to one tile per compute unit run on),
  * "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
  * "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any" (16-bit

@@ -681,7 +681,7 @@ int mfma_config(const GemmProblem& p, int tile) {
   if (layout < 0 || tile < 1 || (tile > 6 && (tile < 9 || tile > 14))) return 0;
   if ((tile == 1 || tile >= 4) && !ring_fits_problem(p, (layout & 2) != 0, (layout & 1) != 0)) return 0;
   if ((tile == 9 || tile == 12 || tile == 13) && !(p.K % 64 == 0 && p.K >= 256)) return 0;   // whole 64-deep units, at least four
-  if (tile == 14 && !(p.K % 128 == 0 && p.K >= 512)) return 0;   // whole 128-deep units, at least four
+  if (tile == 14 && !(p.K % 128 == 0 && p.K >= 256)) return 0;   // whole 128-deep units, at least two
   if (tile == 10) {   // left-over tiles to share, k in whole quads, no transcendental activation
     const bool trans = p.activation == srtActivationSigmoid || p.activation == srtActivationTanh || p.activation == srtActivationElu;
     if (trans || !m16d_tail_fits_BF16_xx(p)) return 0;
@@ -1043,7 +1043,10 @@ bool mfma_prefers_quarter(const GemmProblem& p) {
     // problems share no operand: with a device's worth of tiles from small problems the operand traffic, twice a half
     // tile's, sets the pace (16 x 512 x 512 x 4096, 256 tiles: 61-75 us against 55-56 shared; 64 x 256 x 256 x 1024: 23.5
     // against 18.7 in half tiles) -- unless a problem alone is 32 tiles or more (4 x 512 x 2048 x 4096: 34.5 against 47).
-    if (4 * tq <= 3 * compute_units() || tq / p.batch >= 32) return true;
+    // With two or three units per tile the launch is mostly its fixed costs and the traffic does not show (16 x 512 x 512 x 256:
+    // 6.5 us against 8.0-8.7 in half tiles; 64 x 256 x 256 x 256: 7.5-7.8 against 8.9-9.9; benchmark config 2, 32 x 256^3 in
+    // fp16: 6.4 against 7.0-7.2 in 64 x 64 tiles).
+    if (4 * tq <= 3 * compute_units() || tq / p.batch >= 32 || p.K <= 384) return true;
     // (an A that is not k-contiguous has no 128-row half tile to fall back on: 64-row problems, 64 x 64 x 512 x 1024 17-18
     // against 19-23, x 4096: 60 against 70-72; x^T . W with a short k loop, 16 x 256 x 1024 x 1024 18.5 against 23.6)
     return !a_kc && (p.M <= 64 || (!b_kc && p.K <= 1024));

@@ -9,7 +9,8 @@
 // 16 MFMAs = 256 cycles, and two things follow.
 //   * A unit of staging is 128 rows (or columns) x 128 k = 32 KiB, twice as deep as the 256-wide kernels': a
 //     super-stage -- four slices, 64 MFMAs per wave -- then lasts as long as the 128 x 256 half tile's, and two of them
-//     cover the load latency.  K must be a multiple of 128 and at least 512.
+//     cover the load latency.  K must be a multiple of 128 and at least 256 (with two or three units per tile every
+//     request of the main loop already belongs to the workgroup's next tile).
 //   * The fragments of a slice cannot wait for registers to fall free inside it (the 256-wide kernels re-read each
 //     B tile "right behind its last MFMA", 32 MFMAs ahead of its next use; here that would be 8).  There are
 //     registers to spare instead: two fragment sets, the next slice's eight fragments read into the idle set while
@@ -163,7 +164,7 @@ __device__ __forceinline__ void gemm_m16q_body(const GemmProblem& p) {
   const uint32_t kstep_a = A_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * lda * 2);   // bytes per super-stage
   const uint32_t kstep_b = B_KC ? (uint32_t)(DK * 2) : (uint32_t)(DK * ldb * 2);
   const uint32_t lstep_a = Loader<A_KC>::step(lda), lstep_b = Loader<B_KC>::step(ldb);
-  const int S = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least four)
+  const int S = p.K / DK;   // super-stages per tile (the host admits whole ones only, at least two)
 
   // per-XCD start of the k walk for an A stored k x m (see gemm_ring_kernel)
   const int rot = !A_KC ? (int)(((unsigned)(blockIdx.x & 7) * (unsigned)S) / 8u) : 0;
@@ -337,7 +338,7 @@ __device__ __forceinline__ void gemm_m16q_body(const GemmProblem& p) {
     };
     super_stage(std::true_type{}, 0);
     {
-      int s = 1;   // S >= 4: no guard in front of the loop
+      int s = 1;   // S >= 2: no guard in front of the loop
       do super_stage(std::false_type{}, s); while (++s < S);
     }
 

@@ -123,7 +123,26 @@ def test_result_alias_rule_never_accepts_views_that_share_an_element():
     if L.srtGetDeviceCount(ctypes.byref(count)) == 0 and count.value > 0:
         pytest.skip("placeholder pointers: only on a host without a device")
     g = np.random.Generator(np.random.Philox(1234))
-    base = 1 << 22
+    refusals = (native.ERROR_INVALID_VALUE, native.ERROR_NOT_SUPPORTED)
+
+    # the verdict depends on where the views lie relative to one another, not on where the buffer lies: interleaved
+    # batches and column slices are told apart at any base address (a pitch of 3072 bytes against bases 1 KiB apart)
+    for shift in (0, 4, 1024, 2048, 1536, 3068, 12345 * 4):
+        base = (1 << 22) + shift
+        ad, k1 = native.make_descriptor(native.REAL32F, (3, 16, 24), (768, 24, 1), native.ORDER_ROW)
+        bd, k2 = native.make_descriptor(native.REAL32F, (3, 24, 24), (576, 24, 1), native.ORDER_ROW)
+        st = L.srtMatmul(ctypes.c_void_p(base), ctypes.byref(ad), 0, ctypes.c_void_p(1 << 30), ctypes.byref(bd), 0,
+                         ctypes.c_void_p(base + 4 * 384), ctypes.byref(ad), None)
+        assert st not in refusals, shift
+        ad, k1 = native.make_descriptor(native.REAL32F, (48, 32), (96, 1), native.ORDER_ROW)
+        bd, k2 = native.make_descriptor(native.REAL32F, (32, 32), (32, 1), native.ORDER_ROW)
+        st = L.srtMatmul(ctypes.c_void_p(base), ctypes.byref(ad), 0, ctypes.c_void_p(1 << 30), ctypes.byref(bd), 0,
+                         ctypes.c_void_p(base + 4 * 64), ctypes.byref(ad), None)
+        assert st not in refusals, shift
+        # ... and the same views one row further along than a whole pitch apart still share their elements
+        st = L.srtMatmul(ctypes.c_void_p(base), ctypes.byref(ad), 0, ctypes.c_void_p(1 << 30), ctypes.byref(bd), 0,
+                         ctypes.c_void_p(base + 4 * (96 + 16)), ctypes.byref(ad), None)
+        assert st == native.ERROR_INVALID_VALUE, shift
 
     def view(rows, cols):
         kind = int(g.integers(0, 4))
@@ -151,11 +170,12 @@ def test_result_alias_rule_never_accepts_views_that_share_an_element():
         ad, k1 = native.make_descriptor(native.REAL32F, (M, K), a_st, native.ORDER_ROW)
         bd, k2 = native.make_descriptor(native.REAL32F, (K, N), (N, 1), native.ORDER_ROW)
         od, k3 = native.make_descriptor(native.REAL32F, (M, N), o_st, native.ORDER_ROW)
+        base = (1 << 22) + 4 * int(g.integers(0, 4096))
         st = L.srtMatmul(ctypes.c_void_p(base + 4 * a_off), ctypes.byref(ad), 0, ctypes.c_void_p(1 << 30), ctypes.byref(bd), 0,
                          ctypes.c_void_p(base + 4 * o_off), ctypes.byref(od), None)
         shares = bool(elements(a_off, (M, K), a_st) & elements(o_off, (M, N), o_st))
         overlapping += shares
-        if st in (native.ERROR_INVALID_VALUE, native.ERROR_NOT_SUPPORTED):
+        if st in refusals:
             refused += 1
         else:
             accepted += 1
@@ -334,8 +354,10 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 1024, 1024, 1984, tb=True) == "mfma_64x64"          # 32 half tiles, both k-contiguous
     assert query(native.REAL16BF, 512, 4096, 2048) == "mfma_128x128_m16_k128"
     assert query(native.REAL16BF, 512, 4096, 1984) == "mfma_128x256_m16_k64"              # K too short to split
-    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_128x256_m16_k64"               # short k loops too (8.4 us against 10.0)
-    assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_64x64"
+    assert query(native.REAL16BF, 512, 4096, 256) == "mfma_128x128_m16_k128"              # short k loops too (two 128-deep units)
+    assert query(native.REAL16BF, 512, 4096, 192) == "mfma_128x256_m16"                   # (8.4 us against 10.0 in whole tiles)
+    assert query(native.REAL16F, 256, 256, 256, tb=True) == "mfma_128x128_m16_k128"
+    assert query(native.REAL16F, 256, 256, 192, tb=True) == "mfma_64x64"
     assert query(native.REAL16BF, 1, 14336, 4096, tb=True) == "skinny"
     assert query(native.REAL16BF, 32, 14336, 4096, tb=True) == "skinny"
     # 33..64 rows: the streaming kernel when its workgroups make one round that fills the device
@@ -378,7 +400,8 @@ def test_kernel_selection_is_queryable_without_gpu():
         p = ctypes.c_void_p(256)
         assert L.srtMatmulQueryKernel(ctypes.byref(ad), int(ta), ctypes.byref(bd), int(tb), ctypes.byref(od), p, p, p, buf, 64) == 0
         return buf.value.decode()
-    assert query_batched(native.REAL16F, 32, 256, 256, 256, tb=True) == "mfma_64x64"                   # benchmark config 2: launch-sized, every CU a workgroup
+    assert query_batched(native.REAL16F, 32, 256, 256, 256, tb=True) == "mfma_128x128_m16_k128"        # benchmark config 2: launch-sized, 128 quarter tiles (6.4 us against 7.0-7.2 in 64 x 64 tiles)
+    assert query_batched(native.REAL16F, 32, 256, 256, 192, tb=True) == "mfma_64x64"                   # every CU a workgroup
     assert query_batched(native.REAL16BF, 16, 384, 384, 1024, tb=True) == "mfma_128x128_m16_k128"      # 144 quarter tiles of a batch (15.0 us against 16.1 in half tiles)
     assert query_batched(native.REAL16BF, 16, 384, 384, 960, tb=True) == "mfma_128x256_m16_k64"        # 96 half tiles of a batch, 64 deep
     assert query_batched(native.REAL16BF, 16, 64, 512, 1024, ta=True) == "mfma_128x128_m16_k128"       # 64 quarter tiles, half padding

@@ -112,8 +112,8 @@ def check_plan(tmp_path, plan, dt, M, N, K, ta, tb, with_bias_relu=False):
 
 def plans_for(ta, tb, K):
     plans = ["mfma_256x256_m16_k64", "mfma_256x256_m16", "mfma_256x256"]
-    if K % 128 == 0 and K >= 512:
-        plans.append("mfma_128x128_m16_k128")    # the quarter tile: whole 128-deep units, at least four
+    if K % 128 == 0 and K >= 256:
+        plans.append("mfma_128x128_m16_k128")    # the quarter tile: whole 128-deep units, at least two
     if not ta and tb:
         plans.append("mfma_256x256_k64")    # two k-contiguous operands
     if not ta:
@@ -150,11 +150,12 @@ QUARTER = "mfma_128x128_m16_k128"
 @pytest.mark.parametrize("dt", [H.BF16, H.F16])
 @pytest.mark.parametrize("ta,tb", LAYOUTS)
 def test_quarter_tile_integer_bit_exact_and_random_vs_fp64(dt, ta, tb, tmp_path):
-    """Every staging layout; the shortest admissible k loop (four units), an odd number of units, ragged edges in M and
-    N (a last tile of 8 rows, of 8 columns), one tile and several per workgroup (1190 tiles), fewer tiles than workgroups;
-    then random operands against the fp64 product."""
+    """Every staging layout; the shortest admissible k loops (two and three units: every request beyond the first fill
+    belongs to the next tile), an odd number of units, ragged edges in M and N (a last tile of 8 rows, of 8 columns), one
+    tile and several per workgroup (1225 tiles), fewer tiles than workgroups; then random operands against the fp64 product."""
     r = H.rng(311)
-    for (M, N, K) in [(256, 384, 512), (1000, 520, 640), (2048, 2056, 896), (4400, 4360, 512), (136, 128, 1152)]:
+    for (M, N, K) in [(256, 384, 512), (1000, 520, 640), (2048, 2056, 896), (4400, 4360, 512), (136, 128, 1152),
+                      (4400, 4360, 256), (2056, 2048, 384), (136, 72, 256)]:
         pin(tmp_path, QUARTER, dt, M, N, K, ta, tb)
         a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
         b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
