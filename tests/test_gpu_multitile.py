@@ -202,6 +202,40 @@ def test_quarter_tile_epilogues_vs_oracle(act, dt, tw, tmp_path):
     assert np.all(np.abs(got[rows] - want) <= tol * np.maximum(np.abs(want), 1.0))
 
 
+def test_quarter_tile_broadcast_weight_and_column_major():
+    """The heuristic's own choice on a batch against one shared weight (batch stride 0, the descriptor built by hand) and on
+    a column-major call with bias and relu (computed as the transposed problem, bias per row of what the kernel stores)."""
+    srt.PlanCache.clear()
+    r = H.rng(37)
+    q = srt.current_queue()
+    for dt in (H.BF16, H.F16):
+        B_, M, N, K = 3, 520, 392, 512
+        a = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
+        w = r.integers(-3, 4, (K, N)).astype(np.float32)
+        at, wt = srt.Tensor(H.encode(a, dt)), srt.Tensor(H.encode(w, dt))
+        out = srt.Tensor(shape=[B_, M, N], dtype=H.NP_STORAGE[dt])
+        ad, k1 = at.descriptor()
+        bd, k2 = native.make_descriptor(native.REAL16F if dt == H.F16 else native.REAL16BF, (B_, K, N), (0, N, 1), native.ORDER_ROW)
+        od, k3 = out.descriptor()
+        buf = ctypes.create_string_buffer(64)
+        native.check(native.lib().srtMatmulQueryKernel(ctypes.byref(ad), 0, ctypes.byref(bd), 0, ctypes.byref(od), at.device_read(q),
+                                                       wt.device_read(q), out.device_read(q), buf, 64))
+        assert buf.value.decode() == QUARTER
+        native.check(native.lib().srtMatmul(at.device_read(q), ctypes.byref(ad), 0, wt.device_read(q), ctypes.byref(bd), 0,
+                                            out.device_read_write(q), ctypes.byref(od), q.stream))
+        exact = H.encode((a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), dt)
+        assert np.array_equal(out.array().view(np.uint16), exact.view(np.uint16)), dt
+        M2, N2, K2 = 776, 520, 640
+        x = r.integers(-3, 4, (M2, K2)).astype(np.float32)
+        w2 = r.integers(-3, 4, (K2, N2)).astype(np.float32)
+        b2 = r.integers(-30, 31, N2).astype(np.float32)
+        xc, wc = srt.Tensor(H.encode(x, dt), order=srt.Order.col), srt.Tensor(H.encode(w2, dt), order=srt.Order.col)
+        yc = srt.Dense(wc, srt.Tensor(H.encode(b2, dt)), srt.ActivationType.relu)(xc)
+        assert yc.order == srt.Order.col and query_kernel(xc, False, wc, False, yc) == QUARTER
+        want = np.maximum(x.astype(np.float64) @ w2.astype(np.float64) + b2.astype(np.float64)[None, :], 0)
+        assert np.array_equal(yc.array().view(np.uint16), H.encode(want.astype(np.float32), dt).view(np.uint16)), dt
+
+
 def test_quarter_tile_batched_and_nan(tmp_path):
     """Strided batch (tiles of several batches per workgroup), and NaN / inf results encoded as the reference's codec does."""
     r = H.rng(31)
