@@ -717,7 +717,9 @@ static bool narrow_round(const GemmProblem& p, int layout) {
     if (p.batch > 1) return layout == 1 && p.K < 8192 && p.M <= 128 && 2 * tn > compute_units();
     // (with fewer rows four parts of the k loop do better when K can be cut in four: 384 x 6144 x 4096 36.0 us in parts against
     // 43.4; 192 x 12568 x 3264, which only halves: 36.0 against 41.7)
-    return layout == 1 && p.K < 8192 && tn >= 96 && (p.M >= 1024 || mfma_splitk_parts(p) < 4);
+    // (x^T . W only where the k extent is not in whole quads of 64-deep units, so that no tiles can be shared: 1048 x 6392 x 3456
+    // 49.8 us against 61.2 whole)
+    return (layout == 1 || p.K % 256 != 0) && p.K < 8192 && tn >= 96 && (p.M >= 1024 || mfma_splitk_parts(p) < 4);
   }
   // (tiles that are three quarters padding rows only while they leave half the device free: 64 x 64 x 512 x 1024, 256 of them,
   // 27.1 us against 23.1 in 128 whole tiles)
@@ -850,7 +852,7 @@ int mfma_select(const GemmProblem& p) {
   const long long ring_from = layout == 3 ? 96
                             // (312 x 6136 x 80, 48 tiles: 9.9 us against 8.7; at K = 256 the 64-deep kernel is ahead from 36 tiles:
                             // 1536 x 1536 x 256 11.3 us against 12.1, 1024 x 3072 x 256 11.5 against 12.6)
-                            : layout == 0 ? (p.K >= 1024 ? 1 : p.K >= 512 ? 8 : p.K >= 256 ? 32 : 64)
+                            : layout == 0 ? (p.K >= 1024 ? 1 : p.K >= 512 ? 8 : p.K >= 256 ? 32 : 48)   // (888 x 3616 x 176, 60 tiles: 11.6 us against 17.1 in 64 x 64 tiles)
                             : p.K < 1024 ? 32 : layout == 1 ? (p.batch > 1 ? 16 : 40) : 24;
   //  * the 64-deep form of the 16x16x32 kernel (whole-line loads of k-contiguous operands, one barrier per 128
   //    MFMAs) is ahead of the 32-deep one in every layout once the device is half full (8192^3, same run:
@@ -1034,7 +1036,10 @@ bool mfma_prefers_quarter(const GemmProblem& p) {
   const int config = mfma_config(p, 14);
   const bool a_kc = (config & 2) != 0, b_kc = (config & 1) != 0;
   if (config == 0 || p.N < 64) return false;
-  if (a_kc && (p.M < 64 || (p.M == 64 && b_kc))) return false;
+  // (33-63 rows against an n-contiguous weight and a k loop of two or three units: 48 x 4712 x 256 6.6 us against 7.7 in half
+  // tiles, 43 x 472 x 256 6.2 against 7.2 streamed; at K = 640 the streaming kernel is ahead again, 24 x 384 x 640 6.3 against 8.1)
+  const bool short_nn = a_kc && !b_kc && p.M > 32 && p.K <= 384;
+  if (a_kc && !short_nn && (p.M < 64 || (p.M == 64 && b_kc))) return false;
   const long long tq = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (tq > compute_units()) return false;
   if (p.batch > 1) {
@@ -1052,8 +1057,24 @@ bool mfma_prefers_quarter(const GemmProblem& p) {
     return !a_kc && (p.M <= 64 || (!b_kc && p.K <= 1024));
   }
   if (p.K <= 2048) return true;
-  if (p.K <= 4096) return tq >= 48;   // (512 x 1536 x 4096, 48 tiles: 25.3 against 28.4 in parts)
-  return tq * 73 >= p.K;              // 112 tiles at K = 8192
+  // Beyond that the rival is split-K, and what it is worth depends on how deep it can cut (the cut must leave whole stages:
+  // 4096 goes in eight parts of 512, but 3200, 4480 or 6016 only in four) and on the partial sums it moves.  Two estimates, in
+  // microseconds, fitted to the sweeps:
+  //   quarter tiles   5 + 4.8 per 1024 k, whatever the tile count up to 192, a quarter more at 256
+  //   split-K         10 + 20 per 1024 k of a part (9 + 12 on the half tiles that at most 128 rows of a k-contiguous A run on)
+  //                   + the partial sums, parts x M x N x 8 bytes written and read at 6 TB/s
+  // measured / estimated for split-K: 256 x 2048 x 4096 in eight 24.2-25.9 / 25.6, 512 x 1536 x 4096 28.4 / 28.4, 512 x 4096 x 8192
+  // 48-52 / 52.4, 8 x 1728 x 3200 in four 24.5 / 25.6, 476 x 1936 x 8448 in eight 35.5 / 40.4, 8 x 2848 x 9984 34.1 / 34.6, 128 x
+  // 2048 x 4096 on half tiles 18.5 / 17.1; for quarter tiles: K = 3200 20.0 / 20.0, 4480 26.6 / 26.0, 6016 34.0 / 33.2, 8448 45.2 / 44.6,
+  // 1024 x 4096 x 8192 (256 tiles) 58.7 / 54.3.
+  const int parts = mfma_splitk_parts(p);
+  if (parts < 2) return true;
+  const double part_k = (double)(p.K / parts) / 1024.0;
+  const double sums_us = (double)parts * (double)p.M * (double)p.N * 8.0 / 6.0e6;
+  const double split_us = (a_kc && p.M <= 128 ? 9.0 + 12.0 * part_k : 10.0 + 20.0 * part_k) + sums_us;
+  const double fill = tq > 192 ? 1.0 + 0.25 * (double)(tq - 192) / 64.0 : 1.0;
+  const double quarter_us = (5.0 + 4.8 * (double)p.K / 1024.0) * fill;
+  return quarter_us <= split_us;
 }
 
 // Whether the heuristic takes the tail-sharing form of the 64-deep kernel (tile 10): the tiles left over

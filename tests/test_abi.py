@@ -303,14 +303,17 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 4096, 4096, 1024, tb=True) == "mfma_256x256_m16_k64"
     # few tiles and a long k loop: K split over the idle compute units -- when that buys more than the
     # half-height tiles a k-contiguous A allows
-    assert query(native.REAL16BF, 256, 2048, 4096) == "mfma_256x256_splitk"           # eight whole tiles in eight parts
-    assert query(native.REAL16BF, 256, 2048, 4096, tb=True) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 128, 2048, 4096) == "mfma_256x256_splitk"           # eight half tiles in eight parts (18.5 us against 25 in quarter tiles)
+    assert query(native.REAL16BF, 128, 2048, 4096, tb=True) == "mfma_256x256_splitk"
+    assert query(native.REAL16BF, 256, 1024, 8192) == "mfma_256x256_splitk"           # four whole tiles in sixteen parts
     # ... unless one round of 128 x 128 quarter tiles holds the problem and the k loop is short enough for them (K <= 2048: always;
     # 4096: from 48 tiles; beyond: from K / 73 tiles)
     assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_128x128_m16_k128"         # 128 quarter tiles (25.5 us against 38 in parts)
     assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_128x128_m16_k128"
     assert query(native.REAL16BF, 512, 1536, 4096) == "mfma_128x128_m16_k128"         # 48
-    assert query(native.REAL16BF, 384, 1536, 4096) == "mfma_256x256_splitk"           # 36: parts
+    assert query(native.REAL16BF, 256, 2048, 4096) == "mfma_128x128_m16_k128"         # 32: a tie with eight parts (24.4 us against 24.1-25.9)
+    assert query(native.REAL16BF, 8, 1728, 3200, ta=True, tb=True) == "mfma_128x128_m16_k128"   # K = 3200 only goes in four parts of 800: 20.0 us against 24.5
+    assert query(native.REAL16BF, 476, 1936, 8448) == "mfma_256x256_splitk"           # eight parts of 1056 against a k loop of 8448: 35.5 us against 45.2
     assert query(native.REAL16BF, 512, 2048, 8192) == "mfma_256x256_splitk"           # 64 at K = 8192: parts
     assert query(native.REAL16BF, 1024, 4096, 4096) == "mfma_128x128_m16_k128"        # 256 quarter tiles (31.8 us against 42 shared)
     # 64 to 160 whole tiles beyond one round of quarter tiles: the tail-sharing form of the 64-deep kernel (every tile cut

@@ -717,11 +717,11 @@ def test_splitk_epilogues_vs_oracle_and_nan(act, tmp_path):
 
 
 def test_splitk_is_the_choice_for_few_tiles_and_long_k():
-    a = srt.Tensor(H.encode(np.zeros((256, 4096), np.float32), H.BF16))
+    a = srt.Tensor(H.encode(np.zeros((128, 4096), np.float32), H.BF16))
     b = srt.Tensor(H.encode(np.zeros((4096, 2048), np.float32), H.BF16))
-    out = srt.Tensor(shape=[256, 2048], dtype=a.dtype)
-    assert query_kernel(a, False, b, False, out) == "mfma_256x256_splitk"      # eight whole tiles = 32 quarter tiles
-    a2 = srt.Tensor(H.encode(np.zeros((256, 2048), np.float32), H.BF16))       # K = 2048: not worth the extra pass
+    out = srt.Tensor(shape=[128, 2048], dtype=a.dtype)
+    assert query_kernel(a, False, b, False, out) == "mfma_256x256_splitk"      # eight half tiles in eight parts
+    a2 = srt.Tensor(H.encode(np.zeros((128, 2048), np.float32), H.BF16))       # K = 2048: not worth the extra pass
     b2 = srt.Tensor(H.encode(np.zeros((2048, 2048), np.float32), H.BF16))
     assert query_kernel(a2, False, b2, False, out) != "mfma_256x256_splitk"
     a3 = srt.Tensor(H.encode(np.zeros((512, 4096), np.float32), H.BF16))       # 128 quarter tiles: one round of those instead
