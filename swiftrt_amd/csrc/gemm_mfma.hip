@@ -1060,20 +1060,21 @@ bool mfma_prefers_quarter(const GemmProblem& p) {
   // Beyond that the rival is split-K, and what it is worth depends on how deep it can cut (the cut must leave whole stages:
   // 4096 goes in eight parts of 512, but 3200, 4480 or 6016 only in four) and on the partial sums it moves.  Two estimates, in
   // microseconds, fitted to the sweeps:
-  //   quarter tiles   5 + 4.8 per 1024 k, whatever the tile count up to 192, a quarter more at 256
-  //   split-K         10 + 20 per 1024 k of a part (9 + 12 on the half tiles that at most 128 rows of a k-contiguous A run on)
-  //                   + the partial sums, parts x M x N x 8 bytes written and read at 6 TB/s
-  // measured / estimated for split-K: 256 x 2048 x 4096 in eight 24.2-25.9 / 25.6, 512 x 1536 x 4096 28.4 / 28.4, 512 x 4096 x 8192
-  // 48-52 / 52.4, 8 x 1728 x 3200 in four 24.5 / 25.6, 476 x 1936 x 8448 in eight 35.5 / 40.4, 8 x 2848 x 9984 34.1 / 34.6, 128 x
-  // 2048 x 4096 on half tiles 18.5 / 17.1; for quarter tiles: K = 3200 20.0 / 20.0, 4480 26.6 / 26.0, 6016 34.0 / 33.2, 8448 45.2 / 44.6,
-  // 1024 x 4096 x 8192 (256 tiles) 58.7 / 54.3.
+  //   quarter tiles   5 + 5 per 1024 k, whatever the tile count up to 192, a quarter more at 256
+  //   split-K         10 + 20 per 1024 k of a part + the partial sums, parts x M x N x 8 bytes written and read at 7 TB/s;
+  //                   on the half tiles that at most 128 rows of a k-contiguous A run on: 9 + 12 per 1024 k + the sums at 5 TB/s
+  // measured / estimated for split-K: 256 x 2048 x 4096 in eight 24.2-25.9 / 24.8, 512 x 1536 x 4096 28.4 / 27.2, 512 x 4096 x 8192
+  // 48-52 / 49.2, 512 x 3072 x 8192 41.3-42.8 / 44.4, 8 x 1728 x 3200 in four 24.5 / 25.6, 476 x 1936 x 8448 in eight 35.5 / 39.1,
+  // 8 x 2848 x 9984 34.1 / 34.6; on half tiles 128 x 2048 x 4096 18.5 / 18.4, 128 x 8192 x 4096 27.5-30 / 28.4; for quarter tiles:
+  // K = 3200 20.0 / 20.6, 4096 24.2-25.5 / 25, 4480 26.6 / 26.9, 6016 34.0 / 34.4, 8192 44.7-46.6 / 45, 1024 x 4096 x 8192 (256
+  // tiles) 58.7 / 56.3.
   const int parts = mfma_splitk_parts(p);
   if (parts < 2) return true;
   const double part_k = (double)(p.K / parts) / 1024.0;
-  const double sums_us = (double)parts * (double)p.M * (double)p.N * 8.0 / 6.0e6;
-  const double split_us = (a_kc && p.M <= 128 ? 9.0 + 12.0 * part_k : 10.0 + 20.0 * part_k) + sums_us;
+  const double sums = (double)parts * (double)p.M * (double)p.N * 8.0;   // bytes
+  const double split_us = a_kc && p.M <= 128 ? 9.0 + 12.0 * part_k + sums / 5.0e6 : 10.0 + 20.0 * part_k + sums / 7.0e6;
   const double fill = tq > 192 ? 1.0 + 0.25 * (double)(tq - 192) / 64.0 : 1.0;
-  const double quarter_us = (5.0 + 4.8 * (double)p.K / 1024.0) * fill;
+  const double quarter_us = (5.0 + 5.0 * (double)p.K / 1024.0) * fill;
   return quarter_us <= split_us;
 }
 

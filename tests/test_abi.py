@@ -311,7 +311,8 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 512, 4096, 4096) == "mfma_128x128_m16_k128"         # 128 quarter tiles (25.5 us against 38 in parts)
     assert query(native.REAL16BF, 512, 4096, 4096, tb=True) == "mfma_128x128_m16_k128"
     assert query(native.REAL16BF, 512, 1536, 4096) == "mfma_128x128_m16_k128"         # 48
-    assert query(native.REAL16BF, 256, 2048, 4096) == "mfma_128x128_m16_k128"         # 32: a tie with eight parts (24.4 us against 24.1-25.9)
+    assert query(native.REAL16BF, 256, 2048, 4096) == "mfma_256x256_splitk"           # 32: a tie with eight parts (24.4 us against 24.1-25.9)
+    assert query(native.REAL16BF, 384, 1536, 4096) == "mfma_128x128_m16_k128"         # 36 (25.0-25.2 against 24.9-26.0)
     assert query(native.REAL16BF, 8, 1728, 3200, ta=True, tb=True) == "mfma_128x128_m16_k128"   # K = 3200 only goes in four parts of 800: 20.0 us against 24.5
     assert query(native.REAL16BF, 476, 1936, 8448) == "mfma_256x256_splitk"           # eight parts of 1056 against a k loop of 8448: 35.5 us against 45.2
     assert query(native.REAL16BF, 512, 2048, 8192) == "mfma_256x256_splitk"           # 64 at K = 8192: parts
