@@ -467,7 +467,86 @@ bool splitk_vec_fits(const GemmProblem& p) {
   return true;
 }
 
+// ---- split-K over the 128 x 128 vector kernel -----------------------------------------------------
+// The 128 x 128 kernel leans on several workgroups per compute unit to hide its k stages' load latency and barriers
+// (4096^3, four per unit: 117-121 TFLOP/s; 2048^3, one per unit: 92), and a problem of fewer tiles than units
+// leaves units idle on top (512 x 4096 x 4096: 128 tiles).  Such a problem's k range is cut into S equal parts that
+// run as S "batches" of the kernel (operand batch stride = one part's k extent), each storing its accumulators to a
+// workspace [S][M][N]; a second kernel adds the parts in a fixed order and applies bias and activation.  fp32
+// throughout; the result does not depend on timing.
+__global__ __launch_bounds__(256) void f32_parts_reduce_kernel(const float* part, int parts, GemmProblem p) {
+  const int n4 = (p.N + 3) / 4;   // one lane per four consecutive columns
+  const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (id >= (long long)p.M * n4) return;
+  const int m = (int)(id / n4), n = (int)(id - (long long)m * n4) * 4;
+  const long long mn = (long long)p.M * p.N;
+  const float* src = part + (long long)m * p.N + n;
+  float* C = (float*)p.C;
+  Epilogue<F32> ep(p);
+  if ((p.N & 3) == 0) {   // the workspace's rows are 16-byte aligned
+    f32x4v_t sum = *reinterpret_cast<const f32x4v_t*>(src);
+    for (int s = 1; s < parts; ++s) sum += *reinterpret_cast<const f32x4v_t*>(src + s * mn);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      C[(long long)m * p.scm + (long long)(n + e) * p.scn] = ep.finish(sum[e], ep.bias_at(m, n + e));
+  } else {
+    for (int e = 0; e < 4 && n + e < p.N; ++e) {
+      float sum = src[e];
+      for (int s = 1; s < parts; ++s) sum += src[e + s * mn];
+      C[(long long)m * p.scm + (long long)(n + e) * p.scn] = ep.finish(sum, ep.bias_at(m, n + e));
+    }
+  }
+}
+
 }  // namespace
+
+// Parts the k range of `p` is cut into for the pass above, or 0 when the problem does not take it: a single matrix
+// of more than 64 rows (fewer: the 32 x 32 kernel), operands the 128 x 128 vector kernel reads, fewer tiles than two
+// per compute unit, parts of whole k stages and at least 256 deep.  The smallest power of two that gives every unit
+// two workgroups, or the largest the k extent allows.
+int f32_tile_parts(const GemmProblem& p) {
+  if (p.dtype != srtReal32F || p.batch != 1 || p.M <= 64 || p.K < 512) return 0;
+  if (!mfma128_vec_fits(p) || (p.M + 127) / 128 > 65535) return 0;
+  if ((long long)p.M * p.N >= (1LL << 31)) return 0;
+  const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  const long long want = 2LL * compute_units();
+  if (tiles >= want) return 0;
+  int parts = 0;
+  for (int s = 2; s <= 16; s *= 2) {
+    if (p.K % (s * FK) != 0 || p.K / s < 256) break;
+    parts = s;
+    if (tiles * s >= want) break;
+  }
+  return parts;
+}
+
+hipError_t launch_f32_tile_parts(const GemmProblem& p, hipStream_t stream) {
+  const int parts = f32_tile_parts(p);
+  if (parts < 2) return hipErrorInvalidValue;
+  void* workspace = nullptr;
+  const size_t bytes = (size_t)parts * p.M * p.N * sizeof(float);
+  if (srtDeviceAllocate(&workspace, bytes, reinterpret_cast<srtStream>(stream)) != srtSuccess) return hipErrorOutOfMemory;
+  GemmProblem q = p;
+  q.K = p.K / parts;
+  q.batch = parts;
+  q.sab = (long long)q.K * p.sak;   // part s starts q.K further along k
+  q.sbb = (long long)q.K * p.sbk;
+  q.C = workspace;
+  q.scm = p.N;
+  q.scn = 1;
+  q.scb = (long long)p.M * p.N;
+  q.bias = nullptr;
+  q.activation = srtActivationIdentity;
+  hipError_t e = launch_mfma128_vec(q, stream);
+  if (e == hipSuccess) {
+    const long long lanes = (long long)p.M * ((p.N + 3) / 4);
+    hipLaunchKernelGGL(f32_parts_reduce_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream,
+                       (const float*)workspace, parts, p);
+    e = launch_status(stream);
+  }
+  (void)srtDeviceFree(workspace);   // stream-ordered: reused only by work queued after the kernels above
+  return e;
+}
 
 bool f32_mfma_supported(const GemmProblem& p) {
   if (p.dtype != srtReal32F) return false;
@@ -477,9 +556,11 @@ bool f32_mfma_supported(const GemmProblem& p) {
 }
 
 // The split-K variant pays when 64 x 64 tiles alone would leave most CUs idle.
+// With up to 64 rows it pays whatever the tile count: larger tiles would be mostly padding (32 x 14336 x 4096: 60 us
+// against 181 in 64 x 64 tiles).
 bool f32_mfma_prefers_splitk(const GemmProblem& p) {
   const long long tiles64 = (long long)((p.M + FT - 1) / FT) * ((p.N + FT - 1) / FT) * p.batch;
-  return tiles64 < 192 && p.K >= 64;
+  return (tiles64 <= 256 || p.M <= 64) && p.K >= 64;   // (1024^3, 256 tiles: 33 us against 43 in parts and 49 in 64 x 64 tiles)
 }
 
 hipError_t launch_f32_mfma_variant(const GemmProblem& p, bool splitk, hipStream_t stream) {

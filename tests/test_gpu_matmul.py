@@ -730,6 +730,45 @@ def test_splitk_is_the_choice_for_few_tiles_and_long_k():
     assert query_kernel(a3, False, b3, False, out3) == "mfma_128x128_m16_k128"
 
 
+# ---- fp32: the k range in parts over the 128 x 128 tiles ------------------------------------------------
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_f32_tile_parts_integer_bit_exact_bias_relu_and_random_vs_fp64(ta, tb, tmp_path):
+    """fp32 problems of fewer 128 x 128 tiles than two per compute unit run their k range in 2-16 parts with the sums in
+    a second kernel: integer operands bit-exact (parts of 256, 512 and 1024 k; ragged M and N; N not a multiple of 4 with a
+    k-contiguous B; bias and relu applied after the sum), then random operands against the fp64 product -- pinned and as
+    the heuristic's own choice."""
+    r = H.rng(330)
+    PARTS = "f32_mfma_128x128_parts"
+    shapes = [(512, 1024, 1024), (520, 1000, 2048), (136, 264, 4096), (2048, 2048, 512)]
+    if tb:
+        shapes.append((200, 1001, 1024))
+    for (M, N, K) in shapes:
+        a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+        bias = r.integers(-20, 21, N).astype(np.float32)
+        at, bt, biast = srt.Tensor(a), srt.Tensor(b), srt.Tensor(bias)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+        for pinned in (True, False):
+            srt.PlanCache.clear()
+            if pinned:
+                pin_plan(tmp_path, PARTS, H.F32, M, N, K, ta, tb)
+            out = srt.Tensor(shape=[M, N], dtype=np.float32)
+            assert query_kernel(at, ta, bt, tb, out) == "f32_mfma"
+            srt.current_queue().matmul(at, ta, bt, tb, out)
+            assert np.array_equal(out.array(), exact.astype(np.float32)), (M, N, K, pinned)
+        srt.PlanCache.clear()
+        pin_plan(tmp_path, PARTS, H.F32, M, N, K, ta, tb, bias=True, act=srt.ActivationType.relu)
+        out = srt.Tensor(shape=[M, N], dtype=np.float32)
+        srt.current_queue().matmul(at, ta, bt, tb, out, bias=biast, activation=srt.ActivationType.relu)
+        assert np.array_equal(out.array(), np.maximum(exact + bias[None, :], 0).astype(np.float32)), (M, N, K, "bias+relu")
+    M, N, K = 1000, 1032, 2048
+    a_st = (r.standard_normal((K, M) if ta else (M, K)) / np.sqrt(K)).astype(np.float32)
+    b_st = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    pin_plan(tmp_path, PARTS, H.F32, M, N, K, ta, tb)
+    check_against_fp64(gpu_matmul(a_st, b_st, ta, tb, want_kernel="f32_mfma"), a_st, b_st, ta, tb, H.F32)
+    srt.PlanCache.clear()
+
+
 # ---- the 128 x 256 form of the 16x16x32 kernel ---------------------------------------------------------
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("tb", [False, True])
