@@ -276,6 +276,8 @@ bool f32_mfma_supported(const GemmProblem& p);
 hipError_t launch_f32_mfma(const GemmProblem& p, hipStream_t stream);
 bool f32_mfma_prefers_splitk(const GemmProblem& p);
 hipError_t launch_f32_mfma_variant(const GemmProblem& p, bool splitk, hipStream_t stream);
+bool f32_ring_fits(const GemmProblem& p);
+hipError_t launch_f32_ring(const GemmProblem& p, hipStream_t stream);
 int f32_tile_parts(const GemmProblem& p);
 hipError_t launch_f32_tile_parts(const GemmProblem& p, hipStream_t stream);
 

@@ -12,6 +12,7 @@
 //                       K between them and sum through LDS; row-major operands take a variant that
 //                       keeps a wave's whole k range in flight
 #include "gemm_common.h"
+#include "gemm_f32_ring.h"
 
 namespace srt {
 
@@ -500,16 +501,73 @@ __global__ __launch_bounds__(256) void f32_parts_reduce_kernel(const float* part
 
 }  // namespace
 
+// ---- the 128 x 128 ring kernel (gemm_f32_ring.h) ----------------------------------------------------
+// Preconditions: both operands contiguous along k or along m / n with 16-byte aligned rows and whole 16-byte vectors,
+// K in whole 64-deep units (at least two), 32-bit byte offsets that reach every operand (rows of a partial last tile
+// included).
+bool f32_ring_fits(const GemmProblem& p) {
+  if (p.dtype != srtReal32F || !mfma128_vec_fits(p)) return false;
+  if (p.K % f32r::DK != 0 || p.K < 2 * f32r::DK) return false;
+  if (p.batch > 65535 || p.sab < 0 || p.sbb < 0 || p.sam < 0 || p.sak < 0 || p.sbk < 0 || p.sbn < 0 || p.scm < 0 || p.scn < 0) return false;
+  const bool a_kc = p.sak == 1, b_kc = p.sbk == 1 && p.sbn != 1;
+  const long long lda = a_kc ? p.sam : p.sak, ldb = b_kc ? p.sbn : p.sbk;
+  const long long nb = p.batch - 1;
+  const long long a_reach = nb * p.sab + (a_kc ? ((long long)p.M + 128) * lda + p.K : ((long long)p.K + 64) * lda + p.M + 128);
+  const long long b_reach = nb * p.sbb + (b_kc ? ((long long)p.N + 128) * ldb + p.K : ((long long)p.K + 64) * ldb + p.N + 128);
+  const long long lim = 0x7fffffffLL / 4 - 4096;   // in elements: byte offsets stay below 2^31
+  if (!(a_reach < lim && b_reach < lim)) return false;
+  const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  return tiles < (1LL << 30);
+}
+
+hipError_t launch_f32_ring(const GemmProblem& p, hipStream_t stream) {
+  const bool a_kc = p.sak == 1, b_kc = p.sbk == 1 && p.sbn != 1;
+  constexpr int lds_bytes = f32r::UNITS * f32r::UNIT;
+  const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  const int grid = ring::persistent_grid(tiles);
+  auto go = [&](auto kernel, std::atomic<uint32_t>& configured) {
+    if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(ring::NT), lds_bytes, stream, p);
+    return launch_status(stream);
+  };
+  static std::atomic<uint32_t> c00{0}, c01{0}, c10{0}, c11{0};
+  if (a_kc && b_kc) return go(f32r::gemm_f32_ring_kernel<true, true>, c11);
+  if (a_kc) return go(f32r::gemm_f32_ring_kernel<true, false>, c10);
+  if (b_kc) return go(f32r::gemm_f32_ring_kernel<false, true>, c01);
+  return go(f32r::gemm_f32_ring_kernel<false, false>, c00);
+}
+
 // Parts the k range of `p` is cut into for the pass above, or 0 when the problem does not take it: a single matrix
-// of more than 64 rows (fewer: the 32 x 32 kernel), operands the 128 x 128 vector kernel reads, fewer tiles than two
-// per compute unit, parts of whole k stages and at least 256 deep.  The smallest power of two that gives every unit
-// two workgroups, or the largest the k extent allows.
+// of more than 64 rows (fewer: the 32 x 32 kernel) whose operands the 128 x 128 kernels read, and too few tiles.
+// On the ring kernel (parts of whole 64-deep units, at least two each) the count comes from an estimate of the time,
+// in microseconds: rounds of the persistent grid x 59 per 1024 k of a part (a 128 x 128 tile at nine tenths of a
+// unit's fp32 matrix rate) + 8, and for S > 1 parts the sums, S x M x N x 8 bytes at 6 TB/s, + 5 for the second
+// launch.  Measured / estimated: 512 x 4096 x 4096 whole 242 / 250, in two 140 / 139; 1536^3 whole 99.9 / 98.6, in two
+// 119 / 110; 1024^3 whole 70 / 68, in four 37.6 / 33.7.  More parts must buy a tenth to be taken.  The register-staged
+// kernel wants two workgroups per unit and parts of at least 256.
 int f32_tile_parts(const GemmProblem& p) {
-  if (p.dtype != srtReal32F || p.batch != 1 || p.M <= 64 || p.K < 512) return 0;
+  if (p.dtype != srtReal32F || p.batch != 1 || p.M <= 64 || p.K < 256) return 0;
   if (!mfma128_vec_fits(p) || (p.M + 127) / 128 > 65535) return 0;
   if ((long long)p.M * p.N >= (1LL << 31)) return 0;
   const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128);
-  const long long want = 2LL * compute_units();
+  const int cus = compute_units();
+  if (f32_ring_fits(p)) {
+    if (tiles >= cus) return 0;
+    int best = 1;
+    double best_us = 0.0;
+    for (int s = 1; s <= 16; s *= 2) {
+      if (p.K % (s * f32r::DK) != 0 || p.K / s < 2 * f32r::DK) break;
+      const double rounds = (double)((tiles * s + cus - 1) / cus);
+      double us = rounds * 59.0 * (double)(p.K / s) / 1024.0 + 8.0;
+      if (s > 1) us += (double)s * (double)p.M * (double)p.N * 8.0 / 6.0e6 + 5.0;
+      if (s == 1 || us < 0.9 * best_us) {
+        best = s;
+        best_us = us;
+      }
+    }
+    return best >= 2 ? best : 0;
+  }
+  const long long want = 2LL * cus;
   if (tiles >= want) return 0;
   int parts = 0;
   for (int s = 2; s <= 16; s *= 2) {
@@ -537,7 +595,7 @@ hipError_t launch_f32_tile_parts(const GemmProblem& p, hipStream_t stream) {
   q.scb = (long long)p.M * p.N;
   q.bias = nullptr;
   q.activation = srtActivationIdentity;
-  hipError_t e = launch_mfma128_vec(q, stream);
+  hipError_t e = f32_ring_fits(q) ? launch_f32_ring(q, stream) : launch_mfma128_vec(q, stream);
   if (e == hipSuccess) {
     const long long lanes = (long long)p.M * ((p.N + 3) / 4);
     hipLaunchKernelGGL(f32_parts_reduce_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream,

@@ -769,6 +769,48 @@ def test_f32_tile_parts_integer_bit_exact_bias_relu_and_random_vs_fp64(ta, tb, t
     srt.PlanCache.clear()
 
 
+# ---- fp32: the 128 x 128 ring kernel ----------------------------------------------------------------------
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_f32_ring_kernel_integer_bit_exact_bias_relu_batch_and_random_vs_fp64(ta, tb, tmp_path):
+    """Every staging layout of the fp32 ring kernel; k loops of two, three and an odd number of 64-deep units; ragged edges
+    in M and N (a last tile of 8 rows, of 4 columns); one tile and several per workgroup (1225 tiles); fewer tiles than
+    workgroups; bias and relu; a strided batch; then random operands against the fp64 product."""
+    r = H.rng(340)
+    RING = "f32_mfma_128x128_ring"
+    for (M, N, K) in [(256, 384, 128), (1000, 516, 192), (2048, 2056, 320), (4400, 4356, 128), (136, 132, 1152)]:
+        a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
+        b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
+        bias = r.integers(-20, 21, N).astype(np.float32)
+        at, bt, biast = srt.Tensor(a), srt.Tensor(b), srt.Tensor(bias)
+        exact = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+        pin_plan(tmp_path, RING, H.F32, M, N, K, ta, tb)
+        out = srt.Tensor(shape=[M, N], dtype=np.float32)
+        srt.current_queue().matmul(at, ta, bt, tb, out)
+        assert np.array_equal(out.array(), exact.astype(np.float32)), (M, N, K)
+        pin_plan(tmp_path, RING, H.F32, M, N, K, ta, tb, bias=True, act=srt.ActivationType.relu)
+        out = srt.Tensor(shape=[M, N], dtype=np.float32)
+        srt.current_queue().matmul(at, ta, bt, tb, out, bias=biast, activation=srt.ActivationType.relu)
+        assert np.array_equal(out.array(), np.maximum(exact + bias[None, :], 0).astype(np.float32)), (M, N, K, "bias+relu")
+    B_, M, N, K = 3, 520, 392, 256
+    a = r.integers(-3, 4, (B_, K, M) if ta else (B_, M, K)).astype(np.float32)
+    b = r.integers(-3, 4, (B_, N, K) if tb else (B_, K, N)).astype(np.float32)
+    f = tmp_path / "plan.txt"
+    layout = (2 if ta else 1) | (4 if tb else 8) | 16 | 64
+    f.write_text(f"{H.F32} {M} {N} {K} {B_} {layout} {int(srt.ActivationType.identity) << 1} {RING}\n")
+    srt.PlanCache.clear()
+    srt.PlanCache.load(f)
+    out = srt.matmul(srt.Tensor(a), srt.Tensor(b), ta, tb)
+    am = np.swapaxes(a, 1, 2) if ta else a
+    bm = np.swapaxes(b, 1, 2) if tb else b
+    assert np.array_equal(out.array(), (am.astype(np.float64) @ bm.astype(np.float64)).astype(np.float32))
+    M, N, K = 1000, 1032, 2048
+    a_st = (r.standard_normal((K, M) if ta else (M, K)) / np.sqrt(K)).astype(np.float32)
+    b_st = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    pin_plan(tmp_path, RING, H.F32, M, N, K, ta, tb)
+    check_against_fp64(gpu_matmul(a_st, b_st, ta, tb, want_kernel="f32_mfma"), a_st, b_st, ta, tb, H.F32)
+    srt.PlanCache.clear()
+
+
 # ---- the 128 x 256 form of the 16x16x32 kernel ---------------------------------------------------------
 @pytest.mark.parametrize("dt", [H.F16, H.BF16])
 @pytest.mark.parametrize("tb", [False, True])
