@@ -137,6 +137,73 @@ struct TileAt {
   int m0, n0, bz;
 };
 
+// ---- accumulators -> result.  Lane l of accumulator tile (i, j) holds column 32 j + l % 32 and rows
+// 32 i + 8 (q / 4) + 4 (l / 32) + q % 4, q = 0..15. ----
+// The activation fixed at compile time, BIAS: a bias per column (both values a lane needs are fetched before the first
+// store: a wait on a load is a wait on everything in flight, the next tile's requests included, so there is one per
+// tile and none without a bias); INTERIOR: the tile lies inside the result.
+// (acc + 0 where there is no bias, as the general form has it: the same bits whatever the path.)
+template <int ACT, bool BIAS, bool INTERIOR>
+__device__ __forceinline__ void store_tile(const GemmProblem& p, const TileAt& t, f32x16_t (&acc)[2][2], int wm0, int wn0, int lane) {
+  const int r = lane & 31, h = lane >> 5;
+  float* C = (float*)p.C + (long long)t.bz * p.scb;
+  float b[2] = {0.0f, 0.0f};
+  if constexpr (BIAS) {
+    const float* bias = (const float*)p.bias;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = t.n0 + wn0 + 32 * j + r;
+      if (INTERIOR || n < p.N) b[j] = bias[(long long)n * p.sbias];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = t.n0 + wn0 + 32 * j + r;
+      const int mb = t.m0 + wm0 + 32 * i + 4 * h;
+      const bool n_in = INTERIOR || n < p.N;
+      float* c = C + (long long)mb * p.scm + (long long)n * p.scn;
+      asm volatile("" : "+a"(acc[i][j]));
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int mo = 8 * (q >> 2) + (q & 3);
+        if (INTERIOR || (n_in && mb + mo < p.M)) c[(long long)mo * p.scm] = activation_ct<ACT>(p.coef, acc[i][j][q] + b[j]);
+      }
+    }
+  }
+}
+template <int ACT>
+__device__ __forceinline__ void store_tile_for(const GemmProblem& p, const TileAt& t, f32x16_t (&acc)[2][2], int wm0, int wn0, int lane) {
+  const bool interior = t.m0 + TILE <= p.M && t.n0 + TILE <= p.N;
+  if (p.bias) {
+    if (interior) store_tile<ACT, true, true>(p, t, acc, wm0, wn0, lane);
+    else store_tile<ACT, true, false>(p, t, acc, wm0, wn0, lane);
+  } else {
+    if (interior) store_tile<ACT, false, true>(p, t, acc, wm0, wn0, lane);
+    else store_tile<ACT, false, false>(p, t, acc, wm0, wn0, lane);
+  }
+}
+// Any epilogue of the interface (the activation switched per element).
+__device__ __forceinline__ void store_tile_any(const GemmProblem& p, const TileAt& t, f32x16_t (&acc)[2][2], int wm0, int wn0, int lane) {
+  const int r = lane & 31, h = lane >> 5;
+  float* C = (float*)p.C + (long long)t.bz * p.scb;
+  Epilogue<F32> ep(p);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = t.n0 + wn0 + 32 * j + r;
+      asm volatile("" : "+a"(acc[i][j]));
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const int m = t.m0 + wm0 + 32 * i + 8 * (q >> 2) + 4 * h + (q & 3);
+        if (m < p.M && n < p.N) C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(acc[i][j][q], ep.bias_at(m, n));
+      }
+    }
+  }
+}
+
 template <bool A_KC, bool B_KC>
 __device__ __forceinline__ void gemm_f32_ring_body(const GemmProblem& p) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
@@ -217,19 +284,16 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmProblem& p) {
       issue_a(la, xa1, cur_tile.offa + kstep_a);
       issue_b(lb, xb1, cur_tile.offb + kstep_b);
       asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
-    } else {
-      issue_b(lb, xb1, cur_tile.offb + kstep_b);
-    }
+    }   // (later tiles: the previous tile's boundary has requested B_1 already)
     first_tile = false;
     SRT_FENCE();
 
     const int vn = v + grid;
     const bool has_next = vn < total;
     const TileAt next_tile = locate((int)select_lt(vn, total, (uint32_t)vn, (uint32_t)v));
-    // A requests below limit_a are real (A'_0 and A'_1 of the next tile); of B only B'_0: B'_1 is requested
-    // at the top of the next tile
+    // requests below the limit are real: those of this tile and the first two super-stages of the next
     const int limit_a = (int)select_lt(vn, total, (uint32_t)(S + 2), (uint32_t)S);
-    const int limit_b = (int)select_lt(vn, total, (uint32_t)(S + 1), (uint32_t)S);
+    const int limit_b = limit_a;
 
     f32x16_t acc[2][2];   // defined by the MFMAs of the tile's first k pair
     f32x4v_t af[2][2], bf[2][2];   // [fragment set][tile]
@@ -357,31 +421,21 @@ __device__ __forceinline__ void gemm_f32_ring_body(const GemmProblem& p) {
       do super_stage(std::false_type{}, s); while (++s < S);
     }
 
-    // ---- epilogue: straight from the accumulators (a half wave stores 128 contiguous bytes of a row) ----
-    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+    // ---- tile boundary: nothing to wait for.  The next tile's first two super-stages are requested (A'_0, B'_0 landed
+    // and seen by every wave at the last sync; A'_1, B'_1 in flight into slots nobody reads any more), and the slot the
+    // next request goes to was last read before that sync.  The stores count in vmcnt with the loads: the next sync
+    // waits for "all but the newest eight", which the loads, returning in order, satisfy no later than before. ----
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");   // the last MFMA's 16 passes, before its registers are read
+    // ---- epilogue: straight from the accumulators (a half wave stores 128 contiguous bytes of a row), specialised
+    // once per tile for the common epilogues: a tile is 64 stores per lane with nothing to overlap them ----
     {
       const int le = lane_id();
-      const int r = le & 31, h = le >> 5;
-      float* C = (float*)p.C + (long long)cur_tile.bz * p.scb;
-      Epilogue<F32> ep(p);
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int n = cur_tile.n0 + wn0 + 32 * j + r;
-          asm volatile("" : "+a"(acc[i][j]));
-#pragma unroll
-          for (int q = 0; q < 16; ++q) {
-            const int m = cur_tile.m0 + wm0 + 32 * i + 8 * (q >> 2) + 4 * h + (q & 3);
-            if (m < p.M && n < p.N) C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(acc[i][j][q], ep.bias_at(m, n));
-          }
-        }
-      }
+      const bool plain_bias = !p.bias || !p.bias_per_row;
+      if (plain_bias && p.activation == srtActivationIdentity) store_tile_for<srtActivationIdentity>(p, cur_tile, acc, wm0, wn0, le);
+      else if (plain_bias && p.activation == srtActivationRelu) store_tile_for<srtActivationRelu>(p, cur_tile, acc, wm0, wn0, le);
+      else store_tile_any(p, cur_tile, acc, wm0, wn0, le);
     }
     if (!has_next) break;
-    // every load in flight has landed (A'_0, B'_0, A'_1 of the next tile), in every wave, before B'_1 is requested
-    // into the slot whose last reads were this tile's
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     v = vn;
     cur_tile = next_tile;
   }

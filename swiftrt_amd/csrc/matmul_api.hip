@@ -401,6 +401,11 @@ srtStatus run(const GemmProblem& p, hipStream_t stream) {
     const int c = plan == kPlanM16DTail ? srt::mfma_config(p, 9) : srt::mfma_select(p);
     e = c ? srt::launch_mfma(p, c, stream) : srt::launch_generic(p, stream);
   }
+  if (plan == kPlanF32Parts && e == hipErrorOutOfMemory) {
+    // likewise for the fp32 parts: the whole k range per tile, no workspace
+    (void)hipGetLastError();
+    e = srt::f32_ring_fits(p) ? srt::launch_f32_ring(p, stream) : srt::launch_f32_mfma_variant(p, false, stream);
+  }
   return srt::from_hip(e);
 }
 
@@ -492,7 +497,7 @@ srtStatus srtMatmulTune(const void* a, const srtTensorDescriptor* aDesc, int32_t
     if (plan == kPlanGeneric && fallback != kPlanGeneric && 2.0 * p.M * p.N * p.K * p.batch > 1e9) continue;
     const int warm = 2, reps = 8;
     for (int i = 0; i < warm && err == hipSuccess; ++i) err = launch_plan(p, plan, hs);
-    if ((plan == kPlanSplitK || plan == kPlanM16DTail) && err == hipErrorOutOfMemory) {
+    if ((plan == kPlanSplitK || plan == kPlanM16DTail || plan == kPlanF32Parts) && err == hipErrorOutOfMemory) {
       // no room for this plan's workspace (nothing was launched): it is not a candidate, as in run()
       (void)hipGetLastError();
       err = hipSuccess;

@@ -791,6 +791,22 @@ def test_f32_ring_kernel_integer_bit_exact_bias_relu_batch_and_random_vs_fp64(ta
         out = srt.Tensor(shape=[M, N], dtype=np.float32)
         srt.current_queue().matmul(at, ta, bt, tb, out, bias=biast, activation=srt.ActivationType.relu)
         assert np.array_equal(out.array(), np.maximum(exact + bias[None, :], 0).astype(np.float32)), (M, N, K, "bias+relu")
+        if K > 192:
+            continue
+        # the other forms of the store code: a bias alone, relu alone, an activation switched per element
+        pin_plan(tmp_path, RING, H.F32, M, N, K, ta, tb, bias=True)
+        out = srt.Tensor(shape=[M, N], dtype=np.float32)
+        srt.current_queue().matmul(at, ta, bt, tb, out, bias=biast)
+        assert np.array_equal(out.array(), (exact + bias[None, :]).astype(np.float32)), (M, N, K, "bias")
+        pin_plan(tmp_path, RING, H.F32, M, N, K, ta, tb, act=srt.ActivationType.relu)
+        out = srt.Tensor(shape=[M, N], dtype=np.float32)
+        srt.current_queue().matmul(at, ta, bt, tb, out, activation=srt.ActivationType.relu)
+        assert np.array_equal(out.array(), np.maximum(exact, 0).astype(np.float32)), (M, N, K, "relu")
+        pin_plan(tmp_path, RING, H.F32, M, N, K, ta, tb, bias=True, act=srt.ActivationType.tanh)
+        out = srt.Tensor(shape=[M, N], dtype=np.float32)
+        srt.current_queue().matmul(srt.Tensor(a / 64), ta, bt, tb, out, bias=srt.Tensor(bias / 16), activation=srt.ActivationType.tanh)
+        want = np.tanh(exact / 64 + bias[None, :].astype(np.float64) / 16)   # the products and sums stay exact at this scale
+        assert np.max(np.abs(out.array() - want)) <= 1e-6, (M, N, K, "bias+tanh")
     B_, M, N, K = 3, 520, 392, 256
     a = r.integers(-3, 4, (B_, K, M) if ta else (B_, M, K)).astype(np.float32)
     b = r.integers(-3, 4, (B_, N, K) if tb else (B_, K, N)).astype(np.float32)
