@@ -203,6 +203,51 @@ struct Epilogue {
       v = sizeof(typename T::storage) == 2 ? apply_activation_16(activation, coef, v) : apply_activation(activation, coef, v);
     return T::from_float(v);
   }
+
+  // The same for a run of COUNT sums of one lane, in place and still in fp32 (the caller rounds and stores):
+  // v[q] = activation(v[q] + bias), where at(q, &m, &n) gives the element's place and whether it exists.  The bias
+  // values are fetched first and the run ends before the caller's first store: loads and stores share one counter,
+  // so a store that follows a (conditional) load of its own waits for every earlier store's acknowledgement, and a
+  // lane's stores then go out one round trip apart.  Identity and relu are switched once per run, not per element.
+  template <int ACT, bool BIAS, int COUNT, typename At>
+  __device__ __forceinline__ void finish_run_ct(float (&v)[COUNT], At&& at) const {
+    float b[COUNT];
+#pragma unroll
+    for (int q = 0; q < COUNT; ++q) {
+      b[q] = 0.0f;
+      if constexpr (BIAS) {
+        int m = 0, n = 0;
+        if (at(q, &m, &n)) b[q] = T::to_float(bias[(long long)(per_row ? m : n) * sbias]);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < COUNT; ++q) v[q] = activation_ct<ACT>(coef, v[q] + b[q]);
+  }
+  template <int COUNT, typename At>
+  __device__ __forceinline__ void finish_run(float (&v)[COUNT], At&& at) const {
+    if (activation == srtActivationIdentity) {
+      if (bias) finish_run_ct<srtActivationIdentity, true>(v, at);
+      else finish_run_ct<srtActivationIdentity, false>(v, at);
+    } else if (activation == srtActivationRelu) {
+      if (bias) finish_run_ct<srtActivationRelu, true>(v, at);
+      else finish_run_ct<srtActivationRelu, false>(v, at);
+    } else {
+      float b[COUNT];
+#pragma unroll
+      for (int q = 0; q < COUNT; ++q) b[q] = 0.0f;
+      if (bias) {
+#pragma unroll
+        for (int q = 0; q < COUNT; ++q) {
+          int m = 0, n = 0;
+          if (at(q, &m, &n)) b[q] = T::to_float(bias[(long long)(per_row ? m : n) * sbias]);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < COUNT; ++q)
+        v[q] = sizeof(typename T::storage) == 2 ? apply_activation_16(activation, coef, v[q] + b[q])
+                                                : apply_activation(activation, coef, v[q] + b[q]);
+    }
+  }
 };
 
 // Raises a kernel's dynamic-LDS limit above the 64 KiB default, once per device (the attribute

@@ -110,10 +110,19 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(GemmProblem p) {
     if (n >= p.N) continue;
 #pragma unroll
     for (int i = 0; i < TW; ++i) {
+      const int mb = m0 + wm + 32 * i + 4 * kh;
+      float out[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) out[v] = acc[i][j][v];
+      ep.finish_run(out, [&](int v, int* m, int* nn) {
+        *m = mb + 8 * (v >> 2) + (v & 3);
+        *nn = n;
+        return *m < p.M;
+      });
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm + 32 * i + 8 * (v >> 2) + 4 * kh + (v & 3);
-        if (m < p.M) C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(acc[i][j][v], ep.bias_at(m, n));
+        const int m = mb + 8 * (v >> 2) + (v & 3);
+        if (m < p.M) C[(long long)m * p.scm + (long long)n * p.scn] = out[v];
       }
     }
   }
@@ -234,12 +243,22 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma128_vec_kernel(GemmProblem p
                           (reinterpret_cast<uintptr_t>(p.C) & 7u) == 0 && n + 1 < p.N;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
+    float out[2][16];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) out[j][v] = acc[i][j][v];
+      ep.finish_run(out[j], [&](int v, int* m, int* nn) {
+        *m = m0 + wm + 2 * (8 * (v >> 2) + 4 * kh + (v & 3)) + i;
+        *nn = n + j;
+        return *m < p.M && *nn < p.N;
+      });
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int m = m0 + wm + 2 * (8 * (v >> 2) + 4 * kh + (v & 3)) + i;
       if (m >= p.M) continue;
-      const float c0 = n < p.N ? ep.finish(acc[i][0][v], ep.bias_at(m, n)) : 0.0f;
-      const float c1 = n + 1 < p.N ? ep.finish(acc[i][1][v], ep.bias_at(m, n + 1)) : 0.0f;
+      const float c0 = out[0][v], c1 = out[1][v];
       if (pair_store) {
         const f32x2v_t c = {c0, c1};
         *reinterpret_cast<f32x2v_t*>(C + (long long)m * p.scm + n) = c;
@@ -342,14 +361,21 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_splitk_kernel(GemmProblem p
   Epilogue<F32> ep(p);
   const int n = n0 + r;
   if (n >= p.N) return;
+  const int mb = m0 + 8 * wave + 4 * kh;
+  float out[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int v = 4 * wave + i;
-    const int m = m0 + 8 * wave + 4 * kh + i;
-    if (m >= p.M) continue;
-    const float s = (red[0][v][lane] + red[1][v][lane]) + (red[2][v][lane] + red[3][v][lane]);
-    C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, ep.bias_at(m, n));
+    out[i] = (red[0][v][lane] + red[1][v][lane]) + (red[2][v][lane] + red[3][v][lane]);
   }
+  ep.finish_run(out, [&](int i, int* m, int* nn) {
+    *m = mb + i;
+    *nn = n;
+    return *m < p.M;
+  });
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (mb + i < p.M) C[(long long)(mb + i) * p.scm + (long long)n * p.scn] = out[i];
 }
 
 // ---- 32 x 32 tiles, the 4 waves split K; row-major operands, whole k range in flight ------------
@@ -449,14 +475,21 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_splitk_vec_kernel(GemmProbl
   Epilogue<F32> ep(p);
   const int n = n0 + r;
   if (n >= p.N) return;
+  const int mb = m0 + 8 * wave + 4 * kh;
+  float out[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int v = 4 * wave + i;
-    const int m = m0 + 8 * wave + 4 * kh + i;
-    if (m >= p.M) continue;
-    const float s = (red[0][v][lane] + red[1][v][lane]) + (red[2][v][lane] + red[3][v][lane]);
-    C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, ep.bias_at(m, n));
+    out[i] = (red[0][v][lane] + red[1][v][lane]) + (red[2][v][lane] + red[3][v][lane]);
   }
+  ep.finish_run(out, [&](int i, int* m, int* nn) {
+    *m = mb + i;
+    *nn = n;
+    return *m < p.M;
+  });
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (mb + i < p.M) C[(long long)(mb + i) * p.scm + (long long)n * p.scn] = out[i];
 }
 
 // Preconditions of the vector variant: both operands row-major with 16-byte aligned rows.
@@ -487,9 +520,19 @@ __global__ __launch_bounds__(256) void f32_parts_reduce_kernel(const float* part
   if ((p.N & 3) == 0) {   // the workspace's rows are 16-byte aligned
     f32x4v_t sum = *reinterpret_cast<const f32x4v_t*>(src);
     for (int s = 1; s < parts; ++s) sum += *reinterpret_cast<const f32x4v_t*>(src + s * mn);
+    float out[4] = {sum[0], sum[1], sum[2], sum[3]};
+    ep.finish_run(out, [&](int e, int* mm, int* nn) {
+      *mm = m;
+      *nn = n + e;
+      return true;
+    });
+    if (p.scn == 1 && (p.scm & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0) {
+      const f32x4v_t o = {out[0], out[1], out[2], out[3]};
+      *reinterpret_cast<f32x4v_t*>(C + (long long)m * p.scm + n) = o;
+    } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      C[(long long)m * p.scm + (long long)(n + e) * p.scn] = ep.finish(sum[e], ep.bias_at(m, n + e));
+      for (int e = 0; e < 4; ++e) C[(long long)m * p.scm + (long long)(n + e) * p.scn] = out[e];
+    }
   } else {
     for (int e = 0; e < 4 && n + e < p.N; ++e) {
       float sum = src[e];

@@ -194,11 +194,20 @@ __device__ __forceinline__ void store_tile_any(const GemmProblem& p, const TileA
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int n = t.n0 + wn0 + 32 * j + r;
+      const int mb = t.m0 + wm0 + 32 * i + 4 * h;
       asm volatile("" : "+a"(acc[i][j]));
+      float out[16];
+#pragma unroll
+      for (int q = 0; q < 16; ++q) out[q] = acc[i][j][q];
+      ep.finish_run(out, [&](int q, int* m, int* nn) {
+        *m = mb + 8 * (q >> 2) + (q & 3);
+        *nn = n;
+        return *m < p.M && n < p.N;
+      });
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        const int m = t.m0 + wm0 + 32 * i + 8 * (q >> 2) + 4 * h + (q & 3);
-        if (m < p.M && n < p.N) C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(acc[i][j][q], ep.bias_at(m, n));
+        const int m = mb + 8 * (q >> 2) + (q & 3);
+        if (m < p.M && n < p.N) C[(long long)m * p.scm + (long long)n * p.scn] = out[q];
       }
     }
   }

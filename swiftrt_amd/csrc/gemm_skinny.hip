@@ -293,20 +293,26 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   for (int t = 0; t < NW; ++t) {
     const int n = n0 + 32 * t + r;
     if (n >= p.N || 32 * t + r >= cols) continue;
-    const float bcol = ep.per_row ? 0.0f : ep.bias_at(0, n);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
+      const int mb = 32 * mt + 8 * wave + 4 * h;
+      float out[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int v = 4 * wave + i;
-        const int m = 32 * mt + 8 * wave + 4 * h + i;
-        if (m >= p.M) continue;
         float s = 0.0f;
 #pragma unroll
         for (int w = 0; w < SK_WAVES; ++w) s += red[(((t * MT + mt) * SK_WAVES + w) * 16 + v) * 64 + lane];
-        const float bv = ep.per_row ? ep.bias_at(m, n) : bcol;
-        C[(long long)m * p.scm + (long long)n * p.scn] = ep.finish(s, bv);
+        out[i] = s;
       }
+      ep.finish_run(out, [&](int i, int* m, int* nn) {
+        *m = mb + i;
+        *nn = n;
+        return *m < p.M;
+      });
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (mb + i < p.M) C[(long long)(mb + i) * p.scm + (long long)n * p.scn] = T::from_float(out[i]);
     }
   }
 }
