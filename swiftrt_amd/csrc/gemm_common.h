@@ -322,7 +322,8 @@ hipError_t launch_f32_mfma(const GemmProblem& p, hipStream_t stream);
 bool f32_mfma_prefers_splitk(const GemmProblem& p);
 hipError_t launch_f32_mfma_variant(const GemmProblem& p, bool splitk, hipStream_t stream);
 bool f32_ring_fits(const GemmProblem& p);
-hipError_t launch_f32_ring(const GemmProblem& p, hipStream_t stream);
+int f32_ring_choice(const GemmProblem& p);   // among the fp32 kernels, for a problem f32_ring_fits admits
+hipError_t launch_f32_ring(const GemmProblem& p, hipStream_t stream, int shape);
 int f32_tile_parts(const GemmProblem& p);
 hipError_t launch_f32_tile_parts(const GemmProblem& p, hipStream_t stream);
 

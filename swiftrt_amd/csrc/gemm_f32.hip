@@ -563,31 +563,42 @@ bool f32_ring_fits(const GemmProblem& p) {
   return tiles < (1LL << 30);
 }
 
-hipError_t launch_f32_ring(const GemmProblem& p, hipStream_t stream) {
+// shape 0: 128 x 128 tiles, 1: 64 x 128, 2: 64 x 64 (the same kernel with one MFMA tile per wave along m, or along both)
+hipError_t launch_f32_ring(const GemmProblem& p, hipStream_t stream, int shape) {
   const bool a_kc = p.sak == 1, b_kc = p.sbk == 1 && p.sbn != 1;
   constexpr int lds_bytes = f32r::UNITS * f32r::UNIT;
-  const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  const int tile_m = shape == 0 ? 128 : 64, tile_n = shape == 2 ? 64 : 128;
+  const long long tiles = (long long)((p.M + tile_m - 1) / tile_m) * ((p.N + tile_n - 1) / tile_n) * p.batch;
   const int grid = ring::persistent_grid(tiles);
   auto go = [&](auto kernel, std::atomic<uint32_t>& configured) {
     if (hipError_t e = ensure_lds_limit(reinterpret_cast<const void*>(kernel), lds_bytes, configured); e != hipSuccess) return e;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(ring::NT), lds_bytes, stream, p);
     return launch_status(stream);
   };
-  static std::atomic<uint32_t> c00{0}, c01{0}, c10{0}, c11{0};
-  if (a_kc && b_kc) return go(f32r::gemm_f32_ring_kernel<true, true>, c11);
-  if (a_kc) return go(f32r::gemm_f32_ring_kernel<true, false>, c10);
-  if (b_kc) return go(f32r::gemm_f32_ring_kernel<false, true>, c01);
-  return go(f32r::gemm_f32_ring_kernel<false, false>, c00);
+  static std::atomic<uint32_t> configured[3][4];
+  auto layout = [&](auto tm, auto tn, std::atomic<uint32_t>* c) {
+    constexpr int TM = decltype(tm)::value, TN = decltype(tn)::value;
+    if (a_kc && b_kc) return go(f32r::gemm_f32_ring_kernel<true, true, TM, TN>, c[3]);
+    if (a_kc) return go(f32r::gemm_f32_ring_kernel<true, false, TM, TN>, c[2]);
+    if (b_kc) return go(f32r::gemm_f32_ring_kernel<false, true, TM, TN>, c[1]);
+    return go(f32r::gemm_f32_ring_kernel<false, false, TM, TN>, c[0]);
+  };
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  if (shape == 0) return layout(I2{}, I2{}, configured[0]);
+  if (shape == 1) return layout(I1{}, I2{}, configured[1]);
+  if (shape == 2) return layout(I1{}, I1{}, configured[2]);
+  return hipErrorInvalidValue;
 }
 
 // Parts the k range of `p` is cut into for the pass above, or 0 when the problem does not take it: a single matrix
 // of more than 64 rows (fewer: the 32 x 32 kernel) whose operands the 128 x 128 kernels read, and too few tiles.
 // On the ring kernel (parts of whole 64-deep units, at least two each) the count comes from an estimate of the time,
 // in microseconds: rounds of the persistent grid x 59 per 1024 k of a part (a 128 x 128 tile at nine tenths of a
-// unit's fp32 matrix rate) + 8, and for S > 1 parts the sums, S x M x N x 8 bytes at 6 TB/s, + 5 for the second
-// launch.  Measured / estimated: 512 x 4096 x 4096 whole 242 / 250, in two 140 / 139; 1536^3 whole 99.9 / 98.6, in two
-// 119 / 110; 1024^3 whole 70 / 68, in four 37.6 / 33.7.  More parts must buy a tenth to be taken.  The register-staged
-// kernel wants two workgroups per unit and parts of at least 256.
+// unit's fp32 matrix rate) + 4, and for S > 1 parts the sums, S x M x N x 8 bytes at 6 TB/s, + 5 for the second
+// launch.  Measured / estimated: 512 x 4096 x 4096 whole 236 / 240, in two 129 / 133; 256 x 8192 x 8192 in two 258 / 251.
+// More parts must buy a tenth to be taken.  The register-staged kernel wants two workgroups per unit and parts of at
+// least 256.
 int f32_tile_parts(const GemmProblem& p) {
   if (p.dtype != srtReal32F || p.batch != 1 || p.M <= 64 || p.K < 256) return 0;
   if (!mfma128_vec_fits(p) || (p.M + 127) / 128 > 65535) return 0;
@@ -601,7 +612,7 @@ int f32_tile_parts(const GemmProblem& p) {
     for (int s = 1; s <= 16; s *= 2) {
       if (p.K % (s * f32r::DK) != 0 || p.K / s < 2 * f32r::DK) break;
       const double rounds = (double)((tiles * s + cus - 1) / cus);
-      double us = rounds * 59.0 * (double)(p.K / s) / 1024.0 + 8.0;
+      double us = rounds * 59.0 * (double)(p.K / s) / 1024.0 + 4.0;
       if (s > 1) us += (double)s * (double)p.M * (double)p.N * 8.0 / 6.0e6 + 5.0;
       if (s == 1 || us < 0.9 * best_us) {
         best = s;
@@ -638,7 +649,7 @@ hipError_t launch_f32_tile_parts(const GemmProblem& p, hipStream_t stream) {
   q.scb = (long long)p.M * p.N;
   q.bias = nullptr;
   q.activation = srtActivationIdentity;
-  hipError_t e = f32_ring_fits(q) ? launch_f32_ring(q, stream) : launch_mfma128_vec(q, stream);
+  hipError_t e = f32_ring_fits(q) ? launch_f32_ring(q, stream, 0) : launch_mfma128_vec(q, stream);
   if (e == hipSuccess) {
     const long long lanes = (long long)p.M * ((p.N + 3) / 4);
     hipLaunchKernelGGL(f32_parts_reduce_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream,
@@ -655,6 +666,51 @@ bool f32_mfma_supported(const GemmProblem& p) {
   if ((p.M + 31) / 32 > 65535 || p.batch > 65535) return false;
   return true;
 }
+
+// Which fp32 kernel a problem the ring kernel reads should run on, by estimates of the time in microseconds (each
+// fitted to measurements on one device, 256 units; R(t) = rounds of t tiles over the units):
+//   128 x 128 tiles   R x 59 per 1024 k + 4        (2048^3 124 / 122, 1024 x 4096 x 4096 239 / 240, 1536^3 92 / 92)
+//   64 x 128 tiles    R x 30.5 per 1024 k + 4      (512 x 4096 x 4096 125 / 126, 256 x 8192 x 8192 255 / 248, 1536^3 95 / 96)
+//   64 x 64 tiles     R x 16.5 per 1024 k + 4      (1024^3 20.3 / 20.5, 64 x 14336 x 4096 71 / 70, 1536^3 77 / 78, 768^3 15.9 / 16.4)
+//   k in parts on 128 x 128 tiles: f32_tile_parts' estimate
+//   32 x 32 tiles, k split over the waves: every workgroup reads 64 x K x 4 bytes, at 32 bytes/ns alone on its unit and 31
+//   per unit when they share (both operands row-major: 16-byte loads), 16 and 21.5 otherwise, + 3
+//                      (512^3 6.7 / 7.1, 1024^3 31 / 37 and 42 / 52, 32 x 14336 x 4096 59 / 62 and 90 / 88, 128 x 512 x 4096 35 / 36 and 68 / 69)
+// Smaller tiles cost more per flop (more operand bytes per MFMA through L2 and LDS) and win by filling the device:
+// 1024^3 20 us on 256 tiles of 64 x 64 against 31-42 on 32 x 32 and 62 on 64 tiles of 128 x 128.
+// Returns 0: 128 x 128, 1: 64 x 128, 2: 64 x 64, 3: parts, 4: the 32 x 32 kernel.
+int f32_ring_choice(const GemmProblem& p) {
+  const int cus = compute_units();
+  auto rounds = [&](int tm, int tn) {
+    const long long t = (long long)((p.M + tm - 1) / tm) * ((p.N + tn - 1) / tn) * p.batch;
+    return (double)((t + cus - 1) / cus);
+  };
+  const double k = (double)p.K / 1024.0;
+  double best = rounds(128, 128) * 59.0 * k + 4.0;
+  int choice = 0;
+  auto offer = [&](int c, double us) {
+    if (us < best) {
+      best = us;
+      choice = c;
+    }
+  };
+  offer(1, rounds(64, 128) * 30.5 * k + 4.0);
+  offer(2, rounds(64, 64) * 16.5 * k + 4.0);
+  if (const int s = f32_tile_parts(p); s >= 2) {
+    const long long tiles = (long long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+    offer(3, (double)((tiles * s + cus - 1) / cus) * 59.0 * (double)(p.K / s) / 1024.0 + 4.0 +
+                 (double)s * (double)p.M * (double)p.N * 8.0 / 6.0e6 + 5.0);
+  }
+  if (f32_mfma_supported(p)) {
+    const double tiles32 = (double)((p.M + 31) / 32) * (double)((p.N + 31) / 32) * (double)p.batch;
+    const double bytes = 64.0 * (double)p.K * 4.0;   // per workgroup
+    const bool vec = splitk_vec_fits(p);
+    const double alone = bytes / (vec ? 32.0e3 : 16.0e3), shared = tiles32 / cus * bytes / (vec ? 31.0e3 : 21.5e3);
+    offer(4, (alone > shared ? alone : shared) + 3.0);
+  }
+  return choice;
+}
+
 
 // The split-K variant pays when 64 x 64 tiles alone would leave most CUs idle.
 // With up to 64 rows it pays whatever the tile count: larger tiles would be mostly padding (32 x 14336 x 4096: 60 us

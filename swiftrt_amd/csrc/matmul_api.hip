@@ -114,14 +114,14 @@ srtStatus build_problem(const void* a, const srtTensorDescriptor* ad, int tA,
 // (the role of ExecutionPlanCache / ExecutionPlanner, platform/common/ExecutionPlanner.swift:20-29,
 // and of the empty CudaMatmul2.tune, platform/cuda/functions/CudaMatmul.swift:112-120).
 enum Plan { kPlanGeneric, kPlanSkinny, kPlanRing256, kPlanMfma128, kPlanMfma64, kPlanF32Tile64, kPlanF32SplitK,
-            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanM16DSplit, kPlanM16DH, kPlanM16DN, kPlanM16Q, kPlanF32Parts, kPlanF32Ring, kPlanCount };
+            kPlanKc64, kPlanM16, kPlanSplitK, kPlanM16H, kPlanAny128, kPlanAny64, kPlanM16D, kPlanM16DTail, kPlanM16DSplit, kPlanM16DH, kPlanM16DN, kPlanM16Q, kPlanF32Parts, kPlanF32Ring, kPlanF32Ring64x128, kPlanF32Ring64, kPlanCount };
 
 const char* const kPlanNames[kPlanCount] = {"generic", "skinny", "mfma_256x256", "mfma_128x128", "mfma_64x64",
                                             "f32_mfma_64x64", "f32_mfma_splitk", "mfma_256x256_k64",
                                             "mfma_256x256_m16", "mfma_256x256_splitk", "mfma_128x256_m16",
                                             "mfma_128x128_any", "mfma_64x64_any", "mfma_256x256_m16_k64",
                                             "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split",
-                                            "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128", "f32_mfma_128x128_parts", "f32_mfma_128x128_ring"};
+                                            "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128", "f32_mfma_128x128_parts", "f32_mfma_128x128_ring", "f32_mfma_64x128_ring", "f32_mfma_64x64_ring"};
 
 bool plan_supported(const GemmProblem& p, Plan plan) {
   switch (plan) {
@@ -142,7 +142,9 @@ bool plan_supported(const GemmProblem& p, Plan plan) {
     case kPlanM16DN: return srt::mfma_config(p, 13) != 0;
     case kPlanM16Q: return srt::mfma_config(p, 14) != 0;
     case kPlanF32Parts: return srt::f32_mfma_supported(p) && srt::f32_tile_parts(p) >= 2;
-    case kPlanF32Ring: return srt::f32_ring_fits(p);
+    case kPlanF32Ring:
+    case kPlanF32Ring64x128:
+    case kPlanF32Ring64: return srt::f32_ring_fits(p);
     case kPlanF32Tile64: return srt::f32_mfma_supported(p) && (p.M + 63) / 64 <= 65535;
     case kPlanF32SplitK: return srt::f32_mfma_supported(p);
     default: return srt::generic_supported(p);
@@ -190,14 +192,21 @@ Plan heuristic_plan(const GemmProblem& p) {
     }
   }
   if (srt::f32_mfma_supported(p)) {
-    // launch-sized problems and up to 64 rows: 32 x 32 tiles whose four waves split K (512^3: 7.1 us against 36 in parts)
+    // what the ring kernel reads: the fastest of its three tile shapes, the k range in parts and the 32 x 32 kernel,
+    // by their time estimates
+    if (srt::f32_ring_fits(p)) {
+      switch (srt::f32_ring_choice(p)) {
+        case 0: return kPlanF32Ring;
+        case 1: return kPlanF32Ring64x128;
+        case 2: return kPlanF32Ring64;
+        case 3: return kPlanF32Parts;
+        default: return kPlanF32SplitK;
+      }
+    }
+    // launch-sized problems and up to 64 rows: 32 x 32 tiles whose four waves split K
     if (srt::f32_mfma_prefers_splitk(p)) return kPlanF32SplitK;
     // a single matrix of too few 128 x 128 tiles for the device: its k range in parts on those tiles
     if (srt::f32_tile_parts(p) >= 2) return kPlanF32Parts;
-    // the ring kernel otherwise, where it applies (4096^3: 142-145 TFLOP/s against 116-120 for the register-staged
-    // kernel; 2048^3, one tile per unit: 131 us against 186; 1536^3, 144 tiles: 100 against 119 in two parts)
-    if (srt::f32_ring_fits(p) && (long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch >= srt::compute_units() / 4)
-      return kPlanF32Ring;
     return kPlanF32Tile64;
   }
   return kPlanGeneric;
@@ -222,7 +231,9 @@ hipError_t launch_plan(const GemmProblem& p, Plan plan, hipStream_t stream) {
     case kPlanM16DN: return srt::launch_mfma(p, srt::mfma_config(p, 13), stream);
     case kPlanM16Q: return srt::launch_mfma(p, srt::mfma_config(p, 14), stream);
     case kPlanF32Parts: return srt::launch_f32_tile_parts(p, stream);
-    case kPlanF32Ring: return srt::launch_f32_ring(p, stream);
+    case kPlanF32Ring: return srt::launch_f32_ring(p, stream, 0);
+    case kPlanF32Ring64x128: return srt::launch_f32_ring(p, stream, 1);
+    case kPlanF32Ring64: return srt::launch_f32_ring(p, stream, 2);
     case kPlanF32Tile64: return srt::launch_f32_mfma_variant(p, false, stream);
     case kPlanF32SplitK: return srt::launch_f32_mfma_variant(p, true, stream);
     default: return srt::launch_generic(p, stream);
@@ -404,7 +415,7 @@ srtStatus run(const GemmProblem& p, hipStream_t stream) {
   if (plan == kPlanF32Parts && e == hipErrorOutOfMemory) {
     // likewise for the fp32 parts: the whole k range per tile, no workspace
     (void)hipGetLastError();
-    e = srt::f32_ring_fits(p) ? srt::launch_f32_ring(p, stream) : srt::launch_f32_mfma_variant(p, false, stream);
+    e = srt::f32_ring_fits(p) ? srt::launch_f32_ring(p, stream, 0) : srt::launch_f32_mfma_variant(p, false, stream);
   }
   return srt::from_hip(e);
 }
@@ -452,7 +463,7 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
     while (!has_cached_plan(piece) && split_for_reach(piece, &lo, &hi)) { piece = lo; pieces = true; }
     const Plan plan = select(piece);
     n = kPlanNames[plan];
-    if (plan == kPlanF32Tile64 || plan == kPlanF32SplitK || plan == kPlanF32Parts || plan == kPlanF32Ring) n = "f32_mfma";   // one family name for the fp32 tiles
+    if (plan == kPlanF32Tile64 || plan == kPlanF32SplitK || plan == kPlanF32Parts || plan == kPlanF32Ring || plan == kPlanF32Ring64x128 || plan == kPlanF32Ring64) n = "f32_mfma";   // one family name for the fp32 tiles
     if (pieces) {
       std::snprintf(name, nameCapacity, "%s/pieces", n);
       return srtSuccess;

@@ -22,7 +22,7 @@ SENTINEL = {np.dtype(np.uint16): 0x7B5A, np.dtype(np.float16): 0x7B5A, np.dtype(
 ALL_PLANS_16 = ("mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split", "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
                 "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128", "mfma_128x128", "mfma_64x64", "mfma_128x128_any",
                 "mfma_64x64_any", "skinny", "generic")
-ALL_PLANS_32 = ("f32_mfma_64x64", "f32_mfma_splitk", "f32_mfma_128x128_parts", "f32_mfma_128x128_ring", "generic")
+ALL_PLANS_32 = ("f32_mfma_64x64", "f32_mfma_splitk", "f32_mfma_128x128_parts", "f32_mfma_128x128_ring", "f32_mfma_64x128_ring", "f32_mfma_64x64_ring", "generic")
 
 
 @pytest.fixture(autouse=True)

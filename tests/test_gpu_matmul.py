@@ -769,14 +769,15 @@ def test_f32_tile_parts_integer_bit_exact_bias_relu_and_random_vs_fp64(ta, tb, t
     srt.PlanCache.clear()
 
 
-# ---- fp32: the 128 x 128 ring kernel ----------------------------------------------------------------------
+# ---- fp32: the ring kernel in its three tile shapes ----------------------------------------------------------
+@pytest.mark.parametrize("RING", ["f32_mfma_128x128_ring", "f32_mfma_64x128_ring", "f32_mfma_64x64_ring"])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-def test_f32_ring_kernel_integer_bit_exact_bias_relu_batch_and_random_vs_fp64(ta, tb, tmp_path):
-    """Every staging layout of the fp32 ring kernel; k loops of two, three and an odd number of 64-deep units; ragged edges
-    in M and N (a last tile of 8 rows, of 4 columns); one tile and several per workgroup (1225 tiles); fewer tiles than
-    workgroups; bias and relu; a strided batch; then random operands against the fp64 product."""
+def test_f32_ring_kernel_integer_bit_exact_bias_relu_batch_and_random_vs_fp64(ta, tb, RING, tmp_path):
+    """Every staging layout and tile shape of the fp32 ring kernel; k loops of two, three and an odd number of 64-deep
+    units; ragged edges in M and N (a last tile of 8 rows, of 4 columns); one tile and several per workgroup (1225 tiles
+    of 128 x 128); fewer tiles than workgroups; bias and relu; a strided batch; then random operands against the fp64
+    product."""
     r = H.rng(340)
-    RING = "f32_mfma_128x128_ring"
     for (M, N, K) in [(256, 384, 128), (1000, 516, 192), (2048, 2056, 320), (4400, 4356, 128), (136, 132, 1152)]:
         a = r.integers(-3, 4, (K, M) if ta else (M, K)).astype(np.float32)
         b = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
