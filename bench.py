@@ -126,7 +126,7 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
     ap.add_argument("--only", default=None,
                     help="run one configuration alone, a few launches, and exit (for profilers): headline, cfg3_tn, cfg3_nt, "
-                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, few_tiles, fp16_4096, fp32_4096, dense_backward, add, "
+                         "cfg4_dense, cfg5_m1, cfg5_m8, cfg5_m32, cfg2, cfg1, few_tiles, fp16_4096, fp32_4096, skinny_f32_m8, dense_backward, add, "
                          "add_bias, tanh, cast")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -225,7 +225,7 @@ class Bench:
     """The configurations, each as one prepared foreign call per step."""
 
     SECONDARY = ("cfg3_tn", "cfg3_nt", "cfg4_dense", "cfg4_dense_backward", "cfg5_m1", "cfg5_m8", "cfg5_m32", "cfg2", "cfg1", "few_tiles",
-                 "fp16_4096", "fp32_4096")
+                 "fp16_4096", "fp32_4096", "skinny_f32_m8")
 
     def __init__(self, srt, native, q):
         self.srt, self.native, self.q = srt, native, q
@@ -339,6 +339,18 @@ class Bench:
             return {"name": f"cfg5 skinny bf16 M={m} K=4096 N=14336 transposeRhs", "call": lambda i: calls[i % 4](i),
                     "kernel": prepared[0][1], "flops": 2.0 * m * 4096 * 14336,
                     "bytes": 2 * (m * 4096 + 14336 * 4096 + m * 14336), "bound": "hbm", "dtype": "bf16", "steps": 200,
+                    "keep": (ws, calls)}
+        if name == "skinny_f32_m8":
+            # not one of the five benchmark configurations: configuration 5's shape in the reference's default type
+            g = rng(8)
+            ws = [srt.Tensor(g.standard_normal((14336, 4096), dtype=np.float32) / np.float32(64)) for _ in range(2)]
+            xs = srt.Tensor(g.standard_normal((8, 4096), dtype=np.float32))
+            o = srt.Tensor(shape=[8, 14336], dtype=np.float32)
+            prepared = [self.prepared(xs, False, w_, True, o) for w_ in ws]
+            calls = [p[0] for p in prepared]
+            return {"name": "skinny fp32 M=8 K=4096 N=14336 transposeRhs", "call": lambda i: calls[i % 2](i),
+                    "kernel": prepared[0][1], "flops": 2.0 * 8 * 4096 * 14336,
+                    "bytes": 4 * (8 * 4096 + 14336 * 4096 + 8 * 14336), "bound": "hbm", "dtype": "f32", "steps": 200,
                     "keep": (ws, calls)}
         if name == "cfg2":
             g = rng(1)

@@ -55,8 +55,21 @@ __device__ __forceinline__ f32x16_t mfma32s<F16>(u32x4_t a, u32x4_t b, f32x16_t 
                                                 c, 0, 0, 0);
 }
 
+// fp32: a 16-byte fragment holds four k values; component m of both operands is the k pair (8 s + m, 8 s + 4 + m) of the
+// two half waves, and the four pairs take four v_mfma_f32_32x32x2_f32.
+template <>
+__device__ __forceinline__ f32x16_t mfma32s<F32>(u32x4_t a, u32x4_t b, f32x16_t c) {
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  const f32x4_t af = __builtin_bit_cast(f32x4_t, a), bf = __builtin_bit_cast(f32x4_t, b);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.x, bf.x, c, 0, 0, 0);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.y, bf.y, c, 0, 0, 0);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.z, bf.z, c, 0, 0, 0);
+  c = __builtin_amdgcn_mfma_f32_32x32x2f32(af.w, bf.w, c, 0, 0, 0);
+  return c;
+}
+
 constexpr int SK_WAVES = 4;
-constexpr int SK_KB = 64;          // k per block step (128 bytes per row)
+constexpr int SK_KB = 64;          // k per block step of a 16-bit type (128 bytes per row; fp32: 32)
 constexpr int SK_WTILE = 32 * 128;    // one 32-row W tile of a ring slot: 32 rows x 128 B
 constexpr uint32_t SK_OOB = 0x80000000u;
 
@@ -100,6 +113,10 @@ __device__ __forceinline__ void sk_load_to_lds(u32x4_t rsrc, uint32_t lds_addr, 
 template <typename T, int XR, int NW, bool W_MN = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem p) {
   constexpr int RB = 64 * NW;   // W_MN: bytes of a k row in LDS
+  constexpr int ES = (int)sizeof(typename T::storage);   // element size; an n-contiguous weight is 16-bit only
+  constexpr int EPC = 16 / ES;                           // elements per 16-byte chunk
+  constexpr int KBE = 128 / ES;                          // k per block
+  static_assert(ES == 2 || !W_MN, "the n-contiguous form reads with 16-bit transposing loads");
   using Shape = SkinnyShape<XR, NW>;
   constexpr int SK_WBYTES = Shape::WBYTES;
   constexpr int MT = Shape::MT;
@@ -117,15 +134,15 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
   const int n0 = blockIdx.x * cols;
   const int bz = blockIdx.y;
 
-  const uint16_t* X = (const uint16_t*)p.A + (long long)bz * p.sab;
-  const uint16_t* W = (const uint16_t*)p.B + (long long)bz * p.sbb;
+  const typename T::storage* X = (const typename T::storage*)p.A + (long long)bz * p.sab;
+  const typename T::storage* W = (const typename T::storage*)p.B + (long long)bz * p.sbb;
 
   // both operands through bounds-checked buffers: rows >= N (>= M) and k >= K read zero
-  const uint32_t w_bytes = W_MN ? (uint32_t)(((long long)(p.K - 1) * p.sbk + p.N) * 2)
-                                : (uint32_t)(((long long)(p.N - 1) * p.sbn + p.K) * 2);
+  const uint32_t w_bytes = W_MN ? (uint32_t)(((long long)(p.K - 1) * p.sbk + p.N) * ES)
+                                : (uint32_t)(((long long)(p.N - 1) * p.sbn + p.K) * ES);
   const uint64_t wp = reinterpret_cast<uint64_t>(W);
   const u32x4_t rw = {(uint32_t)wp, (uint32_t)(wp >> 32) & 0xffffu, w_bytes, 0x00020000u};
-  const uint32_t x_bytes = (uint32_t)(((long long)(p.M - 1) * p.sam + p.K) * 2);
+  const uint32_t x_bytes = (uint32_t)(((long long)(p.M - 1) * p.sam + p.K) * ES);
   const uint64_t xp = reinterpret_cast<uint64_t>(X);
   const u32x4_t rx = {(uint32_t)xp, (uint32_t)(xp >> 32) & 0xffffu, x_bytes, 0x00020000u};
 
@@ -151,14 +168,14 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     } else {
       wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
       const int n = n0 + row;
-      wvoff[i] = (n < p.N && row < cols) ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * 8) * 2) : SK_OOB;
+      wvoff[i] = (n < p.N && row < cols) ? (uint32_t)(((long long)n * p.sbn + wchunk[i] * EPC) * ES) : SK_OOB;
     }
   }
 #pragma unroll
   for (int i = 0; i < XR / 8; ++i) {
     const int row = 8 * i + lrow;
     xchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
-    xvoff[i] = row < p.M ? (uint32_t)(((long long)row * p.sam + xchunk[i] * 8) * 2) : SK_OOB;
+    xvoff[i] = row < p.M ? (uint32_t)(((long long)row * p.sam + xchunk[i] * EPC) * ES) : SK_OOB;
   }
   (void)lchunk;
   const uint32_t my_ring = lds + (uint32_t)wave * (DEPTH * Shape::SLOT);
@@ -184,13 +201,13 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     }
   }
 
-  const int KB = (p.K + SK_KB - 1) / SK_KB;   // k blocks in total; this wave takes wave, wave + 4, ...
-  const int k_chunks = p.K / 8;                // valid 16-byte chunks per row
+  const int KB = (p.K + KBE - 1) / KBE;   // k blocks in total; this wave takes wave, wave + 4, ...
+  const int k_chunks = p.K / EPC;          // valid 16-byte chunks per row
 
   auto issue = [&](int kb, int slot) {
     const bool live = kb < KB;
     const uint32_t base = my_ring + (uint32_t)slot * Shape::SLOT;
-    const uint32_t soff = (uint32_t)kb * (SK_KB * 2);
+    const uint32_t soff = (uint32_t)kb * 128u;   // bytes of a block per row
     const uint32_t soff_w = W_MN ? (uint32_t)kb * (uint32_t)(SK_KB * 2) * (uint32_t)p.sbk : soff;
 #pragma unroll
     for (int i = 0; i < 4 * NW; ++i) {
@@ -288,7 +305,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
 
   // wave w finishes accumulator registers 4w .. 4w+3: rows m = 8 w + 4 h + i, column n
   Epilogue<T> ep(p);
-  uint16_t* C = (uint16_t*)p.C + (long long)bz * p.scb;
+  typename T::storage* C = (typename T::storage*)p.C + (long long)bz * p.scb;
 #pragma unroll
   for (int t = 0; t < NW; ++t) {
     const int n = n0 + 32 * t + r;
@@ -329,7 +346,24 @@ hipError_t launch_skinny_shape(const GemmProblem& p, hipStream_t stream) {
 }
 
 template <typename T>
+hipError_t launch_skinny_type16(const GemmProblem& p, hipStream_t stream);
+
+template <typename T>
 hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
+  if constexpr (sizeof(typename T::storage) == 4) {
+    // fp32: the k-contiguous weight, up to 32 rows.  A block of 128 bytes per row is 32 k and sixteen MFMAs per tile,
+    // eight times the matrix time per byte of a 16-bit type: two tiles per workgroup would leave it bound by the matrix
+    // pipe with one workgroup per unit, so the form is always one tile, two workgroups per unit.
+    if (p.M <= 8) return launch_skinny_shape<T, 8, 1>(p, stream);
+    if (p.M <= 16) return launch_skinny_shape<T, 16, 1>(p, stream);
+    return launch_skinny_shape<T, 32, 1>(p, stream);
+  } else {
+    return launch_skinny_type16<T>(p, stream);
+  }
+}
+
+template <typename T>
+hipError_t launch_skinny_type16(const GemmProblem& p, hipStream_t stream) {
   if (p.sbk != 1) {   // n-contiguous weight
     // Always 64 columns per workgroup, i.e. whole 128-byte lines of a k row.  (With 32 columns the
     // two workgroups that share a line each pull it from memory: 11008 columns x 4096 took 39 us
@@ -366,6 +400,20 @@ inline bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr
 }  // namespace
 
 bool skinny_supported(const GemmProblem& p) {
+  if (p.dtype == srtReal32F) {
+    // fp32: up to 32 rows against a k-contiguous weight; the same conditions at four elements per 16-byte chunk
+    if (p.M > 32 || p.M < 1 || p.K < 1 || p.N < 32 || p.batch > 65535) return false;
+    if (p.sak != 1 || p.sbk != 1 || p.sbn == 1) return false;
+    if ((p.K % 4) != 0) return false;
+    if ((p.sam % 4) != 0 && p.M > 1) return false;
+    if ((p.sbn % 4) != 0 && p.N > 1) return false;
+    if ((p.sab % 4) != 0 || (p.sbb % 4) != 0) return false;
+    if (p.sam < 0 || p.sbn < 0 || p.scm < 0 || p.scn < 0) return false;
+    if (!aligned16(p.A) || !aligned16(p.B)) return false;
+    if (((long long)p.M + 8) * p.sam + p.K >= (0x7fffffffLL / 4 - 4096)) return false;
+    if (((long long)p.N + 32) * p.sbn + p.K >= (0x7fffffffLL / 4 - 4096)) return false;
+    return true;
+  }
   if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return false;
   if (p.M > 64 || p.M < 1 || p.K < 1) return false;
   if (p.sak != 1) return false;                         // x is k-contiguous
@@ -405,6 +453,11 @@ bool skinny_supported(const GemmProblem& p) {
 // loop when they are few; deeper problems go to split-K (8 x 4096 x 8192: 25 us against 37 us; 8 x 1024 x 8192: 21 against 36)
 // and more than 256 workgroups to the 128 x 256 tiles (8 x 28672 x 1024: 16 us against 19 us).
 bool skinny_preferred(const GemmProblem& p) {
+  // fp32 (up to 32 rows, x . W^T): ahead of every other fp32 kernel on 80 shapes of 1-32 rows, 256-32768 columns and
+  // K 256-8192 -- 1 x 14336 x 4096 43 us = 5.5 TB/s against 71 on 64 x 64 tiles and 86 on the 32 x 32 kernel, 8 x 4096 x 4096
+  // 24.5 against 67, 32 x 32768 x 256 11.7 against 12.2 -- so always, short of the many short k loops of a large batch,
+  // where the 16-bit form loses (below) and the fp32 one has not been measured
+  if (p.dtype == srtReal32F) return !((long long)((p.N + 31) / 32) * p.batch > (p.batch > 1 ? 512 : 1024) && p.K < 2048);
   // more than 32 rows, a k loop of a few blocks and many workgroups: the two-tile form's set-up does
   // not pay (64 x 14336 x 64: 7.3 us against 5.5 us for 64 x 64 tiles; K = 256: 7.9 against 6.8; but
   // 64 x 3072 x 256: 5.9 against 6.6)
@@ -428,6 +481,7 @@ bool skinny_preferred(const GemmProblem& p) {
 }
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t stream) {
+  if (p.dtype == srtReal32F) return launch_skinny_type<F32>(p, stream);
   if (p.dtype == srtReal16BF) return launch_skinny_type<BF16>(p, stream);
   return launch_skinny_type<F16>(p, stream);
 }

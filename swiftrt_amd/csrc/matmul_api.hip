@@ -160,7 +160,7 @@ Plan heuristic_plan(const GemmProblem& p) {
   // tiles that leave most of the device idle (24 x 96 x 10320: 32 us against 121 in half tiles; 64 x 144 x 8400 x . W^T: 26
   // against 61 in 64 x 64 tiles; 8 x 1288 x 10432: 44 against 58 in two parts).  With up to 32 rows that is decided ahead
   // of tail sharing, whose tiles would be nearly all padding (28 x 8 x 88 x 7680: 32 us against 59).
-  const bool streams = p.K >= 2048 && srt::skinny_supported(p) && (long long)((p.N + 63) / 64) * p.batch <= 256;
+  const bool streams = p.dtype != srtReal32F && p.K >= 2048 && srt::skinny_supported(p) && (long long)((p.N + 63) / 64) * p.batch <= 256;
   const bool few_parts = srt::mfma_splitk_parts(p) <= 2;
   if (streams && few_parts && p.M <= 32) return kPlanSkinny;
   // tiles left over after the whole rounds and a long k loop: cut along k for the idle compute units

@@ -371,6 +371,12 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL16BF, 64, 11008, 4096, tb=True) == "mfma_256x256_splitk"  # 344 workgroups: not one round
     assert query(native.REAL16BF, 65, 14336, 4096, tb=True) == "mfma_128x128_m16_k128"  # 112 quarter tiles, half padding
     assert query(native.REAL16BF, 65, 14336, 4032, tb=True) == "mfma_256x256_splitk"
+    # fp32, up to 32 rows against a k-contiguous weight: the streaming kernel too (four k values per 16-byte chunk)
+    assert query(native.REAL32F, 1, 14336, 4096, tb=True) == "skinny"
+    assert query(native.REAL32F, 32, 256, 1024, tb=True) == "skinny"
+    assert query(native.REAL32F, 32, 14336, 4098, tb=True) == "f32_mfma"              # K not in whole 16-byte chunks
+    assert query(native.REAL32F, 33, 14336, 4096, tb=True) == "f32_mfma"
+    assert query(native.REAL32F, 8, 14336, 4096) == "f32_mfma"                        # an n-contiguous weight: the fp32 tiles
     # x . W with an n-contiguous W: the streaming kernel within one round of 64-column workgroups and a short k loop
     assert query(native.REAL16BF, 8, 14336, 4096) == "skinny"
     assert query(native.REAL16BF, 32, 4096, 2048) == "skinny"
