@@ -69,7 +69,6 @@ __device__ __forceinline__ f32x16_t mfma32s<F32>(u32x4_t a, u32x4_t b, f32x16_t 
 }
 
 constexpr int SK_WAVES = 4;
-constexpr int SK_KB = 64;          // k per block step of a 16-bit type (128 bytes per row; fp32: 32)
 constexpr int SK_WTILE = 32 * 128;    // one 32-row W tile of a ring slot: 32 rows x 128 B
 constexpr uint32_t SK_OOB = 0x80000000u;
 
@@ -112,11 +111,11 @@ __device__ __forceinline__ void sk_load_to_lds(u32x4_t rsrc, uint32_t lds_addr, 
 // of every k row.
 template <typename T, int XR, int NW, bool W_MN = false>
 __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem p) {
-  constexpr int RB = 64 * NW;   // W_MN: bytes of a k row in LDS
-  constexpr int ES = (int)sizeof(typename T::storage);   // element size; an n-contiguous weight is 16-bit only
+  constexpr int ES = (int)sizeof(typename T::storage);   // element size
   constexpr int EPC = 16 / ES;                           // elements per 16-byte chunk
   constexpr int KBE = 128 / ES;                          // k per block
-  static_assert(ES == 2 || !W_MN, "the n-contiguous form reads with 16-bit transposing loads");
+  constexpr int RB = 32 * NW * ES;   // W_MN: bytes of a k row in LDS (the workgroup's 32 NW columns)
+  static_assert(ES == 2 || !W_MN || NW == 1, "fp32 against an n-contiguous weight: one tile of 32 columns = whole 128-byte lines");
   using Shape = SkinnyShape<XR, NW>;
   constexpr int SK_WBYTES = Shape::WBYTES;
   constexpr int MT = Shape::MT;
@@ -162,9 +161,9 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
       const int krow = (1024 / RB) * i + lane / (RB / 16);
       const int pos = lane % (RB / 16);
       const int c = NW == 2 ? pos ^ (((krow >> 1) & 1) << 2) : pos;
-      const int n = n0 + 8 * c;
+      const int n = n0 + EPC * c;
       wchunk[i] = krow;
-      wvoff[i] = n < p.N ? (uint32_t)(((long long)krow * p.sbk + n) * 2) : SK_OOB;
+      wvoff[i] = n < p.N ? (uint32_t)(((long long)krow * p.sbk + n) * ES) : SK_OOB;
     } else {
       wchunk[i] = (lane & 7) ^ ((row >> 1) & 7);
       const int n = n0 + row;
@@ -208,10 +207,10 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
     const bool live = kb < KB;
     const uint32_t base = my_ring + (uint32_t)slot * Shape::SLOT;
     const uint32_t soff = (uint32_t)kb * 128u;   // bytes of a block per row
-    const uint32_t soff_w = W_MN ? (uint32_t)kb * (uint32_t)(SK_KB * 2) * (uint32_t)p.sbk : soff;
+    const uint32_t soff_w = W_MN ? (uint32_t)kb * (uint32_t)(KBE * ES) * (uint32_t)p.sbk : soff;
 #pragma unroll
     for (int i = 0; i < 4 * NW; ++i) {
-      const bool in_k = live && (W_MN ? kb * SK_KB + wchunk[i] < p.K : (kb * 8 + wchunk[i]) < k_chunks);
+      const bool in_k = live && (W_MN ? kb * KBE + wchunk[i] < p.K : (kb * 8 + wchunk[i]) < k_chunks);
       sk_load_to_lds<true>(rw, base + (uint32_t)i * 1024u, in_k ? wvoff[i] : SK_OOB, soff_w);
     }
 #pragma unroll
@@ -261,7 +260,14 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(GemmProblem 
       for (int s = 0; s < 4; ++s) {
 #pragma unroll
         for (int t = 0; t < NW; ++t) {
-          if (W_MN) {
+          if constexpr (W_MN && ES == 4) {
+            // fp32: the four k rows 8 s + 4 h + 0..3 of column r, one dword each (the half waves meet on the same
+            // banks, 512 bytes apart: two passes per read, of sixteen reads per block against sixteen MFMAs)
+            const uint32_t a = base + (uint32_t)((8 * s + 4 * h) * RB + r * 4);
+            wf[t][s] = u32x4_t{*reinterpret_cast<const SRT_LDS uint32_t*>(a), *reinterpret_cast<const SRT_LDS uint32_t*>(a + RB),
+                               *reinterpret_cast<const SRT_LDS uint32_t*>(a + 2 * RB),
+                               *reinterpret_cast<const SRT_LDS uint32_t*>(a + 3 * RB)};
+          } else if constexpr (W_MN) {
             const uint32_t a = base + rdw[t & 1] + s * (16 * RB);
             const u32x2_t lo = __builtin_bit_cast(
                 u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<SRT_LDS s16x4_t*>(a)));
@@ -354,6 +360,11 @@ hipError_t launch_skinny_type(const GemmProblem& p, hipStream_t stream) {
     // fp32: the k-contiguous weight, up to 32 rows.  A block of 128 bytes per row is 32 k and sixteen MFMAs per tile,
     // eight times the matrix time per byte of a 16-bit type: two tiles per workgroup would leave it bound by the matrix
     // pipe with one workgroup per unit, so the form is always one tile, two workgroups per unit.
+    if (p.sbk != 1) {   // n-contiguous weight: 32 columns per workgroup are whole 128-byte lines of a k row
+      if (p.M <= 8) return launch_skinny_shape<T, 8, 1, true>(p, stream);
+      if (p.M <= 16) return launch_skinny_shape<T, 16, 1, true>(p, stream);
+      return launch_skinny_shape<T, 32, 1, true>(p, stream);
+    }
     if (p.M <= 8) return launch_skinny_shape<T, 8, 1>(p, stream);
     if (p.M <= 16) return launch_skinny_shape<T, 16, 1>(p, stream);
     return launch_skinny_shape<T, 32, 1>(p, stream);
@@ -403,16 +414,19 @@ bool skinny_supported(const GemmProblem& p) {
   if (p.dtype == srtReal32F) {
     // fp32: up to 32 rows against a k-contiguous weight; the same conditions at four elements per 16-byte chunk
     if (p.M > 32 || p.M < 1 || p.K < 1 || p.N < 32 || p.batch > 65535) return false;
-    if (p.sak != 1 || p.sbk != 1 || p.sbn == 1) return false;
-    if ((p.K % 4) != 0) return false;
+    if (p.sak != 1 || (p.K % 4) != 0) return false;
     if ((p.sam % 4) != 0 && p.M > 1) return false;
-    if ((p.sbn % 4) != 0 && p.N > 1) return false;
     if ((p.sab % 4) != 0 || (p.sbb % 4) != 0) return false;
-    if (p.sam < 0 || p.sbn < 0 || p.scm < 0 || p.scn < 0) return false;
+    if (p.sam < 0 || p.scm < 0 || p.scn < 0) return false;
     if (!aligned16(p.A) || !aligned16(p.B)) return false;
     if (((long long)p.M + 8) * p.sam + p.K >= (0x7fffffffLL / 4 - 4096)) return false;
-    if (((long long)p.N + 32) * p.sbn + p.K >= (0x7fffffffLL / 4 - 4096)) return false;
-    return true;
+    if (p.sbk == 1 && p.sbn != 1) {                     // W k-contiguous ([N, K])
+      if ((p.sbn % 4) != 0 || p.sbn < 0) return false;
+      return ((long long)p.N + 32) * p.sbn + p.K < (0x7fffffffLL / 4 - 4096);
+    }
+    if (p.sbn != 1 || (p.N % 4) != 0) return false;     // W n-contiguous ([K, N]): whole 16-byte chunks of a k row
+    if (p.sbk < 4 || (p.sbk % 4) != 0) return false;
+    return ((long long)p.K + 32) * p.sbk + p.N < (0x7fffffffLL / 4 - 4096);
   }
   if (p.dtype != srtReal16BF && p.dtype != srtReal16F) return false;
   if (p.M > 64 || p.M < 1 || p.K < 1) return false;
@@ -453,10 +467,11 @@ bool skinny_supported(const GemmProblem& p) {
 // loop when they are few; deeper problems go to split-K (8 x 4096 x 8192: 25 us against 37 us; 8 x 1024 x 8192: 21 against 36)
 // and more than 256 workgroups to the 128 x 256 tiles (8 x 28672 x 1024: 16 us against 19 us).
 bool skinny_preferred(const GemmProblem& p) {
-  // fp32 (up to 32 rows, x . W^T): ahead of every other fp32 kernel on 80 shapes of 1-32 rows, 256-32768 columns and
+  // fp32 (up to 32 rows): ahead of every other fp32 kernel on 80 shapes x . W^T of 1-32 rows, 256-32768 columns and
   // K 256-8192 -- 1 x 14336 x 4096 43 us = 5.5 TB/s against 71 on 64 x 64 tiles and 86 on the 32 x 32 kernel, 8 x 4096 x 4096
-  // 24.5 against 67, 32 x 32768 x 256 11.7 against 12.2 -- so always, short of the many short k loops of a large batch,
-  // where the 16-bit form loses (below) and the fp32 one has not been measured
+  // 24.5 against 67, 32 x 32768 x 256 11.7 against 12.2 -- and on 48 shapes x . W, where the 32 x 32 kernel has 16-byte loads
+  // (1 x 14336 x 4096 47 us against 57, 8 x 4096 x 4096 25.8 against 36.6, 32 x 14336 x 4096 a tie at 59.5) -- so always, short of
+  // the many short k loops of a large batch, where the 16-bit form loses (below) and the fp32 one has not been measured
   if (p.dtype == srtReal32F) return !((long long)((p.N + 31) / 32) * p.batch > (p.batch > 1 ? 512 : 1024) && p.K < 2048);
   // more than 32 rows, a k loop of a few blocks and many workgroups: the two-tile form's set-up does
   // not pay (64 x 14336 x 64: 7.3 us against 5.5 us for 64 x 64 tiles; K = 256: 7.9 against 6.8; but

@@ -376,7 +376,9 @@ def test_kernel_selection_is_queryable_without_gpu():
     assert query(native.REAL32F, 32, 256, 1024, tb=True) == "skinny"
     assert query(native.REAL32F, 32, 14336, 4098, tb=True) == "f32_mfma"              # K not in whole 16-byte chunks
     assert query(native.REAL32F, 33, 14336, 4096, tb=True) == "f32_mfma"
-    assert query(native.REAL32F, 8, 14336, 4096) == "f32_mfma"                        # an n-contiguous weight: the fp32 tiles
+    assert query(native.REAL32F, 8, 14336, 4096) == "skinny"                          # an n-contiguous weight likewise
+    assert query(native.REAL32F, 8, 14338, 4096) == "f32_mfma"                        # its rows not in whole chunks
+    assert query(native.REAL32F, 8, 14336, 4096, ta=True) == "f32_mfma"               # x must be k-contiguous
     # x . W with an n-contiguous W: the streaming kernel within one round of 64-column workgroups and a short k loop
     assert query(native.REAL16BF, 8, 14336, 4096) == "skinny"
     assert query(native.REAL16BF, 32, 4096, 2048) == "skinny"

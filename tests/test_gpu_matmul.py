@@ -357,8 +357,9 @@ def test_skinny_ragged_and_integer_exact(dt):
         assert np.array_equal(got.view(np.uint16), H.encode(exact, dt).view(np.uint16)), (M, N, K)
 
 
-def test_skinny_fp32_integer_exact_ragged_bias_relu_batch_and_random_vs_fp64(tmp_path):
-    """The streaming kernel on fp32 (x . W^T, up to 32 rows): a 16-byte chunk is four k values and a 128-byte block 32 of
+@pytest.mark.parametrize("tb", [True, False])
+def test_skinny_fp32_integer_exact_ragged_bias_relu_batch_and_random_vs_fp64(tb, tmp_path):
+    """The streaming kernel on fp32 (x . W^T and x . W, up to 32 rows): a 16-byte chunk is four k values and a 128-byte block 32 of
     them; every staged row count (8, 16, 32), K ending inside a block and of a single chunk, N not a multiple of 32, a row
     pitch wider than K, bias and relu, a batch, random operands against the fp64 product."""
     r = H.rng(41)
@@ -366,39 +367,41 @@ def test_skinny_fp32_integer_exact_ragged_bias_relu_batch_and_random_vs_fp64(tmp
 
     def pin(M, N, K, epilogue):   # both alignment classes of the rows: the class counts eight elements whatever the type
         f = tmp_path / "plan.txt"
-        f.write_text(f"{H.F32} {M} {N} {K} 1 85 {epilogue} skinny\n{H.F32} {M} {N} {K} 1 21 {epilogue} skinny\n")
+        lay = 21 if tb else 25
+        f.write_text(f"{H.F32} {M} {N} {K} 1 {lay + 64} {epilogue} skinny\n{H.F32} {M} {N} {K} 1 {lay} {epilogue} skinny\n")
         srt.PlanCache.clear()
         srt.PlanCache.load(f)
 
-    for (M, N, K) in [(1, 33, 4), (5, 100, 72), (8, 4096, 4096), (17, 32, 4100), (32, 1000, 520), (32, 14336, 1024)]:
+    for (M, N, K) in [(1, 33 if tb else 36, 4), (5, 100, 72), (8, 4096, 4096), (17, 32, 4100), (32, 1000, 520), (32, 14336, 1024)]:
         x = r.integers(-3, 4, (M, K)).astype(np.float32)
-        w = r.integers(-3, 4, (N, K)).astype(np.float32)
+        w = r.integers(-3, 4, (N, K) if tb else (K, N)).astype(np.float32)
         bias = r.integers(-20, 21, N).astype(np.float32)
-        exact = x.astype(np.float64) @ w.astype(np.float64).T
+        exact = x.astype(np.float64) @ (w.T if tb else w).astype(np.float64)
         xt, wt, bt = srt.Tensor(x), srt.Tensor(w), srt.Tensor(bias)
         pin(M, N, K, int(srt.ActivationType.identity) << 1)
         out = srt.Tensor(shape=[M, N], dtype=np.float32)
-        assert query_kernel(xt, False, wt, True, out) == "skinny"
-        q.matmul(xt, False, wt, True, out)
+        assert query_kernel(xt, False, wt, tb, out) == "skinny"
+        q.matmul(xt, False, wt, tb, out)
         assert np.array_equal(out.array(), exact.astype(np.float32)), (M, N, K)
         pin(M, N, K, 1 | (int(srt.ActivationType.relu) << 1))
         out = srt.Tensor(shape=[M, N], dtype=np.float32)
-        q.matmul(xt, False, wt, True, out, bias=bt, activation=srt.ActivationType.relu)
+        q.matmul(xt, False, wt, tb, out, bias=bt, activation=srt.ActivationType.relu)
         assert np.array_equal(out.array(), np.maximum(exact + bias[None, :], 0).astype(np.float32)), (M, N, K, "bias+relu")
     B_, M, N, K = 3, 20, 264, 328
     x = r.integers(-3, 4, (B_, M, K)).astype(np.float32)
-    w = r.integers(-3, 4, (B_, N, K)).astype(np.float32)
+    w = r.integers(-3, 4, (B_, N, K) if tb else (B_, K, N)).astype(np.float32)
     f = tmp_path / "plan.txt"
-    f.write_text(f"{H.F32} {M} {N} {K} {B_} 85 10 skinny\n")
+    f.write_text(f"{H.F32} {M} {N} {K} {B_} {85 if tb else 89} 10 skinny\n")
     srt.PlanCache.clear()
     srt.PlanCache.load(f)
-    out = srt.matmul(srt.Tensor(x), srt.Tensor(w), False, True)
-    assert np.array_equal(out.array(), (x.astype(np.float64) @ np.swapaxes(w, 1, 2).astype(np.float64)).astype(np.float32))
+    out = srt.matmul(srt.Tensor(x), srt.Tensor(w), False, tb)
+    wm = np.swapaxes(w, 1, 2) if tb else w
+    assert np.array_equal(out.array(), (x.astype(np.float64) @ wm.astype(np.float64)).astype(np.float32))
     M, N, K = 24, 1032, 2048
     a_st = (r.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
-    w_st = r.standard_normal((N, K)).astype(np.float32)
-    pin_plan(tmp_path, "skinny", H.F32, M, N, K, False, True)
-    check_against_fp64(gpu_matmul(a_st, w_st, False, True, want_kernel="skinny"), a_st, w_st, False, True, H.F32)
+    w_st = r.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    pin_plan(tmp_path, "skinny", H.F32, M, N, K, False, tb)
+    check_against_fp64(gpu_matmul(a_st, w_st, False, tb, want_kernel="skinny"), a_st, w_st, False, tb, H.F32)
     srt.PlanCache.clear()
 
 
