@@ -261,7 +261,7 @@ srtStatus srtMatmulQueryKernel(const srtTensorDescriptor* aDesc, int32_t transpo
  * problems of up to one tile per compute unit run on),
  * "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
  * "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x128", "mfma_64x64", "mfma_128x128_any", "mfma_64x64_any" (16-bit
- * operands of any stride and alignment), "skinny", "f32_mfma_128x128_ring", "f32_mfma_64x128_ring", "f32_mfma_64x64_ring" (one
+ * operands of any stride and alignment), "skinny" (16-bit types up to 64 rows, fp32 up to 32), "f32_mfma_128x128_ring", "f32_mfma_64x128_ring", "f32_mfma_64x64_ring" (one
  * fp32 kernel in three tile shapes: K a multiple of 64 and at least 128, operands contiguous along k or along m / n with
  * 16-byte aligned rows), "f32_mfma_128x128_parts" (its k range cut in parts, for a single matrix of a few tiles and a long k),
  * "f32_mfma_64x64", "f32_mfma_splitk", "generic").
