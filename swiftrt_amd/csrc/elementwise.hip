@@ -23,28 +23,30 @@ constexpr int MAX_RANK = 4;   // after collapsing adjacent dimensions
 constexpr int kVectorsPerLane = 4;   // (two: sigmoid 32.2 -> 30.7 us, bias-broadcast add 33.3 -> 36.8, the rest unchanged)
 
 // ---- operations -----------------------------------------------------------------------------
-struct Add { static __device__ __forceinline__ float apply(float a, float b) { return a + b; } };
-struct Sub { static __device__ __forceinline__ float apply(float a, float b) { return a - b; } };
-struct Mul { static __device__ __forceinline__ float apply(float a, float b) { return a * b; } };
-struct Div { static __device__ __forceinline__ float apply(float a, float b) { return a / b; } };
-struct Max { static __device__ __forceinline__ float apply(float a, float b) { return a >= b ? a : b; } };
-struct Min { static __device__ __forceinline__ float apply(float a, float b) { return a <= b ? a : b; } };
-struct Neg { static __device__ __forceinline__ float apply(float a, float) { return -a; } };
-struct Exp { static __device__ __forceinline__ float apply(float a, float) { return expf(a); } };
-struct Sigmoid { static __device__ __forceinline__ float apply(float a, float) { return 1.0f / (1.0f + expf(-a)); } };
-struct Tanh { static __device__ __forceinline__ float apply(float a, float) { return tanhf(a); } };
+struct Add { static constexpr bool binary = true; static __device__ __forceinline__ float apply(float a, float b) { return a + b; } };
+struct Sub { static constexpr bool binary = true; static __device__ __forceinline__ float apply(float a, float b) { return a - b; } };
+struct Mul { static constexpr bool binary = true; static __device__ __forceinline__ float apply(float a, float b) { return a * b; } };
+struct Div { static constexpr bool binary = true; static __device__ __forceinline__ float apply(float a, float b) { return a / b; } };
+struct Max { static constexpr bool binary = true; static __device__ __forceinline__ float apply(float a, float b) { return a >= b ? a : b; } };
+struct Min { static constexpr bool binary = true; static __device__ __forceinline__ float apply(float a, float b) { return a <= b ? a : b; } };
+struct Neg { static constexpr bool binary = false; static __device__ __forceinline__ float apply(float a, float) { return -a; } };
+struct Exp { static constexpr bool binary = false; static __device__ __forceinline__ float apply(float a, float) { return expf(a); } };
+struct Sigmoid { static constexpr bool binary = false; static __device__ __forceinline__ float apply(float a, float) { return 1.0f / (1.0f + expf(-a)); } };
+struct Tanh { static constexpr bool binary = false; static __device__ __forceinline__ float apply(float a, float) { return tanhf(a); } };
 // For 16-bit results the hardware exponential (a few fp32 ulps) is exact enough by a wide margin:
 // its error is 2^-13 of a half / 2^-16 of a bfloat16 rounding step.  fp32 results keep libm.
-struct ExpFast { static __device__ __forceinline__ float apply(float a, float) { return __expf(a); } };
+struct ExpFast { static constexpr bool binary = false; static __device__ __forceinline__ float apply(float a, float) { return __expf(a); } };
 struct SigmoidFast {
+  static constexpr bool binary = false;
   static __device__ __forceinline__ float apply(float a, float) { return __fdividef(1.0f, 1.0f + __expf(-a)); }
 };
 struct TanhFast {
+  static constexpr bool binary = false;
   // a quotient of two short polynomials, exact to a fraction of a 16-bit rounding step and uniformly so down to
   // the smallest arguments (see activation16_ct)
   static __device__ __forceinline__ float apply(float a, float) { return srt::activation16_ct<srtActivationTanh>(0.0f, a); }
 };
-struct Copy { static __device__ __forceinline__ float apply(float a, float) { return a; } };
+struct Copy { static constexpr bool binary = false; static __device__ __forceinline__ float apply(float a, float) { return a; } };
 
 enum OpCode { kAdd, kSub, kMul, kDiv, kMax, kMin, kNeg, kExp, kSigmoid, kTanh, kCopy };
 
@@ -60,6 +62,7 @@ struct Map {
   float element;                 // the scalar of tensor-element forms (and of fill)
   int b_is_element;
   int fill;                      // no input at all: out = element
+  int b_reused;                  // the second operand is broadcast along some dimension: its lines are read again and again
 };
 
 template <typename T, int V>
@@ -69,7 +72,8 @@ struct alignas(V * sizeof(typename T::storage)) Pack {
 
 // One vector of an input operand.  STREAM: with the non-temporal hint -- an element-wise operand
 // is read once, and without the hint its lines stay in L2 until evicted (the same hint raised a
-// bare streaming read of this device from 5.7 to 6.2 TB/s).
+// bare streaming read of this device from 5.7 to 6.2 TB/s).  A broadcast operand (a bias row under
+// every row of the other operand) is the opposite case: its few lines are wanted in the caches.
 template <typename T, int V, bool STREAM>
 __device__ __forceinline__ Pack<T, V> load_pack(const typename T::storage* p) {
   constexpr int BYTES = V * (int)sizeof(typename T::storage);
@@ -83,7 +87,7 @@ __device__ __forceinline__ Pack<T, V> load_pack(const typename T::storage* p) {
   }
 }
 
-template <typename TI, typename TO, typename Op, int V>
+template <typename TI, typename TO, typename Op, int V, bool B_CACHED = false>
 __global__ __launch_bounds__(256) void map_kernel(Map m) {
   using SI = typename TI::storage;
   using SO = typename TO::storage;
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(256) void map_kernel(Map m) {
 #pragma unroll
       for (int i = 0; i < V; ++i) fb[i] = 0.0f;
     } else if (V > 1 && m.sb[inner] == 1) {
-      const Pack<TI, V> pb = load_pack<TI, V, true>(b + ob);
+      const Pack<TI, V> pb = load_pack<TI, V, !B_CACHED>(b + ob);
 #pragma unroll
       for (int i = 0; i < V; ++i) fb[i] = TI::to_float(pb.v[i]);
     } else {
@@ -169,6 +173,13 @@ hipError_t launch_v(const Map& m, hipStream_t stream) {
   const unsigned long long blocks = (m.total + 256 * kVectorsPerLane - 1) / (256 * kVectorsPerLane);
   if (blocks == 0) return hipSuccess;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  // (a run-time choice between the two kinds of load inside one kernel cost every operation 14 %)
+  if constexpr (V > 1 && Op::binary) {
+    if (m.b_reused) {
+      hipLaunchKernelGGL((map_kernel<TI, TO, Op, V, true>), dim3((unsigned)blocks), dim3(256), 0, stream, m);
+      return launch_status(stream);
+    }
+  }
   hipLaunchKernelGGL((map_kernel<TI, TO, Op, V>), dim3((unsigned)blocks), dim3(256), 0, stream, m);
   return launch_status(stream);
 }
@@ -328,6 +339,9 @@ srtStatus build_map(const srtTensorDescriptor* ad, const srtTensorDescriptor* bd
   }
   if (total > 0xffffffffull) return srtErrorNotSupported;   // the kernel decomposes 32-bit ids
   m->total = total;
+  m->b_reused = 0;
+  for (int d = 0; d < n; ++d)
+    if (bd && shape[d] > 1 && sb[d] == 0) m->b_reused = 1;
   return srtSuccess;
 }
 

@@ -1208,3 +1208,60 @@ def test_fused_transcendentals_keep_their_digits_near_zero(act, dt, plan, M, N, 
     floor = 2.0 ** -24 if dt == H.F16 else 1e-30          # a half's subnormal step
     assert np.all(np.abs(got - want) <= 2 * H.ULP[dt] * np.abs(want) + floor)
     srt.PlanCache.clear()
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_problems_through_the_librarys_own_choice_bit_exact(seed):
+    """Widely random problems -- element type, layout, batch (own or shared right operand), extents drawn
+    log-uniformly with and without alignment, bias, relu / clipped relu -- run on whatever kernel the library
+    picks by itself.  Operands are small integers, so every sum is exact in fp32 and the stored result must
+    equal the exact one rounded once, bit for bit.  The case is named before it runs."""
+    g = np.random.default_rng(seed)
+    q = srt.current_queue()
+    seen = set()
+
+    def logu(lo, hi):
+        return int(np.exp(g.uniform(np.log(lo), np.log(hi + 1))))
+
+    for case in range(250):
+        dt = (H.F32, H.BF16, H.F16)[int(g.integers(0, 3))]
+        ta, tb = bool(g.integers(0, 2)), bool(g.integers(0, 2))
+        batch = int(g.choice([1, 1, 1, 2, 3, 7]))
+        M, N, K = logu(1, 3000), logu(1, 3000), logu(1, 4096)
+        if g.random() < 0.5:
+            M, N, K = max(8, M // 8 * 8), max(8, N // 8 * 8), max(8, K // 8 * 8)
+        if g.random() < 0.4:
+            K = max(64, K // 64 * 64)
+        if g.random() < 0.15:
+            M = int(g.integers(1, 65))
+        if M * N * K * batch > 3e9:
+            continue
+        with_bias = bool(g.integers(0, 2))
+        act = (srt.ActivationType.identity, srt.ActivationType.relu, srt.ActivationType.clippedRelu)[int(g.integers(0, 3))]
+        shared_b = batch > 1 and g.random() < 0.3
+        what = (seed, case, dt, ta, tb, batch, M, N, K, with_bias, act, shared_b)
+        sa = (K, M) if ta else (M, K)
+        sb = (N, K) if tb else (K, N)
+        a = g.integers(-2, 3, (batch,) + sa).astype(np.float32)
+        b = g.integers(-2, 3, ((1,) if shared_b else (batch,)) + sb).astype(np.float32)
+        bias = g.integers(-3, 4, N).astype(np.float32)
+        exact = (a.transpose(0, 2, 1) if ta else a).astype(np.float64) @ (b.transpose(0, 2, 1) if tb else b).astype(np.float64)
+        if with_bias:
+            exact = exact + bias[None, None, :]
+        if act != srt.ActivationType.identity:
+            exact = np.maximum(exact, 0.0)
+        if act == srt.ActivationType.clippedRelu:
+            exact = np.minimum(exact, 6.0)
+        want = H.encode(exact.astype(np.float32), dt)
+        if batch == 1:
+            at, bt = srt.Tensor(H.encode(a[0], dt)), srt.Tensor(H.encode(b[0], dt))
+            out = srt.Tensor(shape=[M, N], dtype=at.dtype)
+            want = want[0]
+        else:
+            at = srt.Tensor(H.encode(a, dt))
+            bt = srt.Tensor.repeating(srt.Tensor(H.encode(b[0], dt)), (batch,) + sb) if shared_b else srt.Tensor(H.encode(b, dt))
+            out = srt.Tensor(shape=[batch, M, N], dtype=at.dtype)
+        seen.add(query_kernel(at, ta, bt, tb, out))
+        q.matmul(at, ta, bt, tb, out, bias=srt.Tensor(H.encode(bias, dt)) if with_bias else None, activation=act, coef=6.0)
+        assert np.array_equal(out.array().view(np.uint8), want.view(np.uint8)), what
+    assert len(seen) >= 5, seen
