@@ -18,6 +18,9 @@ from tests.test_gpu_matmul import query_kernel
 pytestmark = pytest.mark.gpu
 
 SENTINEL = {np.dtype(np.uint16): 0x7B5A, np.dtype(np.float16): 0x7B5A, np.dtype(np.float32): 0x7B5A7B5A}
+# a quiet NaN of each type: around an OPERAND it shows whether anything outside the view reaches a sum
+# (a finite value times a padding zero vanishes, a NaN does not)
+NAN_BITS = {np.dtype(np.uint16): 0x7FC0, np.dtype(np.float16): 0x7E00, np.dtype(np.float32): 0x7FC00000}
 
 ALL_PLANS_16 = ("mfma_256x256_m16_k64", "mfma_256x256_m16_k64_tail", "mfma_256x256_m16_k64_split", "mfma_256x256_m16", "mfma_256x256", "mfma_256x256_k64",
                 "mfma_256x256_splitk", "mfma_128x256_m16", "mfma_128x256_m16_k64", "mfma_256x128_m16_k64", "mfma_128x128_m16_k128", "mfma_128x128", "mfma_64x64", "mfma_128x128_any",
@@ -36,8 +39,9 @@ class Framed:
     """A `shape` view (rank 2 or 3) inside a larger buffer full of the sentinel: `top` rows above and below,
     `left` / `right` elements either side of every row, `between` whole sentinel matrices between batches."""
 
-    def __init__(self, values, top=2, left=8, right=8, between=1):
+    def __init__(self, values, top=2, left=8, right=8, between=1, sentinel=None):
         values = np.asarray(values)
+        sentinel = SENTINEL if sentinel is None else sentinel
         self.np_dtype = values.dtype
         self.bits = np.dtype(np.uint32) if values.dtype == np.float32 else np.dtype(np.uint16)
         shape = values.shape
@@ -46,7 +50,7 @@ class Framed:
         self.rows, self.cols, self.batch = rows, cols, batch
         self.top, self.left = top, left
         self.step = 1 + between
-        big = np.full((batch * self.step, rows + 2 * top, left + cols + right), SENTINEL[values.dtype], self.bits)
+        big = np.full((batch * self.step, rows + 2 * top, left + cols + right), sentinel[values.dtype], self.bits)
         body = values.reshape(batch, rows, cols).view(self.bits)
         big[::self.step, top:top + rows, left:left + cols] = body
         self.before = big.copy()
@@ -78,7 +82,8 @@ def pin(tmp_path, dt, M, N, K, batch, layout, epilogues, plan):
     srt.PlanCache.load(f)
 
 
-def run_matmul_case(tmp_path, dt, M, N, K, batch, ta, tb, plans, seed, left=8, right=8, with_bias=True, relu=True):
+def run_matmul_case(tmp_path, dt, M, N, K, batch, ta, tb, plans, seed, left=8, right=8, with_bias=True, relu=True,
+                    operand_sentinel=None):
     """Every plan of `plans` that takes the problem: exact result inside the views, sentinel everywhere else."""
     g = H.rng(seed)
     lead = (batch,) if batch > 1 else ()
@@ -93,8 +98,9 @@ def run_matmul_case(tmp_path, dt, M, N, K, batch, ta, tb, plans, seed, left=8, r
         exact = np.maximum(exact, 0.0)
     want = H.encode(exact.astype(np.float32), dt)
     act = srt.ActivationType.relu if relu else srt.ActivationType.identity
-    fa, fb = Framed(H.encode(a, dt), left=left, right=right), Framed(H.encode(b, dt), left=left, right=right)
-    fbias = Framed(H.encode(bias, dt).reshape(1, N), top=1, left=left, right=right)
+    fa = Framed(H.encode(a, dt), left=left, right=right, sentinel=operand_sentinel)
+    fb = Framed(H.encode(b, dt), left=left, right=right, sentinel=operand_sentinel)
+    fbias = Framed(H.encode(bias, dt).reshape(1, N), top=1, left=left, right=right, sentinel=operand_sentinel)
     bias_t = srt.Tensor(shape=[N], order=fbias.view.order, _storage=fbias.view.storage, _offset=fbias.view.offset, _strides=[1])
     aligned = all((left + x.shape[-1] + right) % 8 == 0 for x in (a, b)) and (left + N + right) % 8 == 0
     layout = (2 if ta else 1) | (4 if tb else 8) | 16 | (64 if aligned else 0)
@@ -181,6 +187,34 @@ def test_streaming_kernel_keeps_inside_including_its_56_column_tiles(tmp_path):
 def test_fp32_plans_keep_inside(tmp_path):
     for (M, N, K, batch, ta, tb) in [(200, 264, 72, 1, False, False), (130, 70, 33, 1, True, False), (96, 136, 64, 3, False, True)]:
         ran = run_matmul_case(tmp_path, H.F32, M, N, K, batch, ta, tb, ALL_PLANS_32, 780 + M, left=4, right=4)
+        assert "generic" in ran and len(ran) >= 2, ran
+
+
+def test_nothing_outside_an_operand_view_reaches_a_sum(tmp_path):
+    """Operand and bias views framed by NaNs (rows above and below, columns either side of every row, whole NaN matrices
+    between batches): the reference's loops never touch an element outside a view, so every result must still be the exact
+    one.  A kernel that reads a k tail, a ragged row or a neighbouring batch past the view's edge and counts on the other
+    operand's padding zero to cancel it fails here."""
+    cases16 = [(520, 776, 1024, 1), (200, 264, 72, 1), (130, 136, 200, 1), (264, 328, 1032, 1), (264, 328, 256, 3), (72, 136, 1024, 5)]
+    for dt in (H.BF16, H.F16):
+        for (M, N, K, batch) in cases16:
+            for ta, tb in [(False, False), (False, True), (True, False), (True, True)]:
+                ran = run_matmul_case(tmp_path, dt, M, N, K, batch, ta, tb, ALL_PLANS_16, 800 + M + K, operand_sentinel=NAN_BITS)
+                assert "generic" in ran and len(ran) >= 3, ran
+    for (M, N, K, left, right) in [(200, 265, 72, 3, 2), (130, 72, 136, 1, 4), (257, 129, 65, 8, 3)]:
+        for ta, tb in [(False, False), (True, False), (False, True), (True, True)]:
+            ran = run_matmul_case(tmp_path, H.BF16, M, N, K, 1, ta, tb, ALL_PLANS_16, 820 + M, left=left, right=right,
+                                  operand_sentinel=NAN_BITS)
+            assert "mfma_64x64_any" in ran, ran
+    for (M, N, K, tb) in [(32, 14336, 256, True), (24, 14328, 136, True), (8, 1000, 520, True), (8, 1096, 264, False), (40, 2056, 136, False)]:
+        for dt in (H.BF16, H.F32):
+            if dt == H.F32 and M > 32:
+                continue          # the fp32 form streams at most 32 rows
+            ran = run_matmul_case(tmp_path, dt, M, N, K, 1, False, tb, ("skinny",), 840 + M, left=8, right=8, operand_sentinel=NAN_BITS)
+            assert ran == ["skinny"], (dt, M, N, K, tb)
+    for (M, N, K, batch, ta, tb) in [(200, 264, 72, 1, False, False), (130, 70, 33, 1, True, False), (96, 136, 64, 3, False, True),
+                                     (264, 392, 1096, 1, False, True), (520, 264, 2048, 1, True, True), (136, 1032, 516, 2, False, False)]:
+        ran = run_matmul_case(tmp_path, H.F32, M, N, K, batch, ta, tb, ALL_PLANS_32, 860 + M, left=4, right=4, operand_sentinel=NAN_BITS)
         assert "generic" in ran and len(ran) >= 2, ran
 
 
