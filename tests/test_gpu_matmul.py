@@ -1265,3 +1265,38 @@ def test_random_problems_through_the_librarys_own_choice_bit_exact(seed):
         q.matmul(at, ta, bt, tb, out, bias=srt.Tensor(H.encode(bias, dt)) if with_bias else None, activation=act, coef=6.0)
         assert np.array_equal(out.array().view(np.uint8), want.view(np.uint8)), what
     assert len(seen) >= 5, seen
+
+
+@pytest.mark.parametrize("dt,M,N,K,ta,tb", [
+    (H.BF16, 520, 776, 1024, False, False), (H.BF16, 1024, 4096, 4096, False, True), (H.BF16, 2048, 4096, 2048, False, False),
+    (H.BF16, 1024, 8192, 512, True, False), (H.BF16, 3072, 1536, 8192, False, True), (H.BF16, 512, 1024, 4096, False, True),
+    (H.BF16, 8, 1000, 520, False, True), (H.BF16, 8, 1096, 264, False, False), (H.F16, 200, 265, 72, False, False),
+    (H.F16, 264, 328, 256, True, True), (H.F32, 8, 1000, 520, False, True), (H.F32, 8, 1096, 264, False, False),
+    (H.F32, 512, 512, 512, False, False), (H.F32, 1024, 1024, 1024, False, False), (H.F32, 200, 264, 72, True, False),
+    (H.F32, 512, 2048, 4096, False, True), (H.F32, 64, 2048, 4096, False, False)])
+def test_nan_and_inf_stay_in_their_rows_on_the_librarys_own_choice(dt, M, N, K, ta, tb):
+    """One NaN and one infinity in A (B all positive): row 5 of the result is NaN, row 7 is +inf, and every other element
+    is the exact product -- a tile-wide or wave-wide shortcut in an encoder or an epilogue must not let a special value
+    leak into a neighbour's row, whichever kernel the library picks for the shape."""
+    g = H.rng(900 + M + K)
+    a = g.integers(-2, 3, (M, K)).astype(np.float32)
+    b = g.integers(1, 4, (K, N)).astype(np.float32)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    a[5, 1] = np.nan
+    a[7, 2] = np.inf
+    a_st = H.encode(np.ascontiguousarray(a.T) if ta else a, dt)
+    b_st = H.encode(np.ascontiguousarray(b.T) if tb else b, dt)
+    at, bt = srt.Tensor(a_st), srt.Tensor(b_st)
+    out = srt.Tensor(shape=[M, N], dtype=at.dtype)
+    kernel = query_kernel(at, ta, bt, tb, out)
+    srt.current_queue().matmul(at, ta, bt, tb, out)
+    got = out.array()
+    dec = H.decode(got).astype(np.float64)
+    assert np.all(np.isnan(dec[5])), kernel
+    assert np.all(np.isposinf(dec[7])), kernel
+    if dt == H.BF16:
+        assert np.all(got[5] == 0x7FFF), kernel          # the reference codec's NaN (platform/common/BFloat16.swift:53-80)
+    rest = np.ones(M, bool)
+    rest[[5, 7]] = False
+    want = H.encode(exact.astype(np.float32), dt)
+    assert np.array_equal(got[rest].view(np.uint8), want[rest].view(np.uint8)), kernel
