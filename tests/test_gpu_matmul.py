@@ -1300,3 +1300,33 @@ def test_nan_and_inf_stay_in_their_rows_on_the_librarys_own_choice(dt, M, N, K, 
     rest[[5, 7]] = False
     want = H.encode(exact.astype(np.float32), dt)
     assert np.array_equal(got[rest].view(np.uint8), want[rest].view(np.uint8)), kernel
+
+
+@pytest.mark.parametrize("M,N,K,tb", [(64, 64, 64, False), (200, 264, 72, False), (520, 776, 1024, False), (8, 1000, 520, True),
+                                      (1024, 1024, 1024, False), (2048, 4096, 512, False), (4096, 4096, 512, False),
+                                      (512, 1024, 4096, True)])
+@pytest.mark.parametrize("dt,scale_a,scale_b", [
+    (H.F16, 2.0 ** -24, 2.0 ** 6),       # subnormal halves in A, normal results
+    (H.F16, 2.0 ** -12, 2.0 ** -12),     # results among the subnormal halves
+    (H.F32, 2.0 ** -149, 2.0 ** 60),     # subnormal floats in A
+    (H.F32, 2.0 ** -100, 2.0 ** -49),    # products and sums among the subnormal floats
+    (H.BF16, 2.0 ** -133, 2.0 ** 100),   # subnormal bfloat16s in A
+    (H.BF16, 2.0 ** -100, 2.0 ** -33)])  # sums that are subnormal in the fp32 accumulator and in the result
+def test_subnormal_operands_and_results_are_kept(dt, scale_a, scale_b, M, N, K, tb):
+    """The reference's CPU loops run with gradual underflow (Swift Float / Float16 arithmetic): small integers times a
+    power of two that puts the operands, the products or the sums among the subnormals must give the exact scaled integer
+    product -- no flush to zero on the way into the matrix cores, in their accumulators or in the stored result --
+    whichever kernel the library picks."""
+    g = H.rng(950 + M + K)
+    a = g.integers(-2, 3, (M, K)).astype(np.float64) * scale_a
+    b = g.integers(-2, 3, (K, N)).astype(np.float64) * scale_b
+    exact = a @ b
+    a_st = H.encode(a.astype(np.float32), dt)
+    b_st = H.encode(np.ascontiguousarray(b.T if tb else b).astype(np.float32), dt)
+    assert np.array_equal(H.decode(a_st).astype(np.float64), a) and np.count_nonzero(exact) > exact.size // 2
+    at, bt = srt.Tensor(a_st), srt.Tensor(b_st)
+    out = srt.Tensor(shape=[M, N], dtype=at.dtype)
+    kernel = query_kernel(at, False, bt, tb, out)
+    srt.current_queue().matmul(at, False, bt, tb, out)
+    want = H.encode(exact.astype(np.float32), dt)
+    assert np.array_equal(out.array().view(np.uint8), want.view(np.uint8)), kernel
