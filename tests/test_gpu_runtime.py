@@ -7,6 +7,7 @@ import pytest
 
 import swiftrt_amd as srt
 from swiftrt_amd import native
+from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
 
@@ -165,3 +166,64 @@ def test_cpp_host_mirror_runs_the_reference_kats():
     out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stdout + out.stderr
     assert "all checks passed" in out.stdout
+
+
+def test_native_module_from_several_threads_each_with_its_own_stream():
+    """The native module is entered from several threads at once, each driving a stream of its own through the C ABI
+    (the allocator and the plan cache are process globals: platform/cuda/device/CudaDevice.swift:141-160 allocates from
+    whichever thread owns the tensor).  Every thread allocates, copies, multiplies shapes whose kernels take
+    stream-ordered workspaces (split-K parts, shared tiles, fp32 parts) next to small ones, frees, and repeats; every
+    product must be exact and identical from round to round."""
+    import ctypes
+    import threading
+    L = native.lib()
+    shapes = [(native.REAL16BF, 512, 1024, 4096), (native.REAL16BF, 3072, 1536, 4096), (native.REAL32F, 512, 2048, 2048),
+              (native.REAL16BF, 8, 1000, 520), (native.REAL16F, 200, 264, 72), (native.REAL32F, 64, 64, 64),
+              (native.REAL16BF, 1024, 1024, 1024)]
+    codec = {native.REAL16BF: H.BF16, native.REAL16F: H.F16, native.REAL32F: H.F32}
+    problems = []
+    g = H.rng(990)
+    for (dt, M, N, K) in shapes:
+        a = g.integers(-2, 3, (M, K)).astype(np.float32)
+        b = g.integers(-2, 3, (K, N)).astype(np.float32)
+        want = H.encode((a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32), codec[dt])
+        problems.append((dt, M, N, K, np.ascontiguousarray(H.encode(a, codec[dt])), np.ascontiguousarray(H.encode(b, codec[dt])), want))
+    errors = []
+
+    def worker(index):
+        try:
+            native.check(L.srtSetDevice(0))
+            stream = ctypes.c_void_p()
+            native.check(L.srtStreamCreate(ctypes.byref(stream)))
+            for rnd in range(6):
+                for j in range(len(problems)):
+                    dt, M, N, K, a_st, b_st, want = problems[(j + index) % len(problems)]
+                    ptrs = []
+                    for nbytes in (a_st.nbytes, b_st.nbytes, want.nbytes):
+                        p = ctypes.c_void_p()
+                        native.check(L.srtDeviceAllocate(ctypes.byref(p), nbytes, stream))
+                        ptrs.append(p)
+                    native.check(L.srtMemcpyAsync(ptrs[0], a_st.ctypes.data_as(ctypes.c_void_p), a_st.nbytes, native.H2D, stream))
+                    native.check(L.srtMemcpyAsync(ptrs[1], b_st.ctypes.data_as(ctypes.c_void_p), b_st.nbytes, native.H2D, stream))
+                    ad, k1 = native.make_descriptor(dt, (M, K), (K, 1), native.ORDER_ROW)
+                    bd, k2 = native.make_descriptor(dt, (K, N), (N, 1), native.ORDER_ROW)
+                    od, k3 = native.make_descriptor(dt, (M, N), (N, 1), native.ORDER_ROW)
+                    native.check(L.srtMatmul(ptrs[0], ctypes.byref(ad), 0, ptrs[1], ctypes.byref(bd), 0, ptrs[2], ctypes.byref(od), stream))
+                    got = np.empty_like(want)
+                    native.check(L.srtMemcpyAsync(got.ctypes.data_as(ctypes.c_void_p), ptrs[2], got.nbytes, native.D2H, stream))
+                    native.check(L.srtStreamSynchronize(stream))
+                    for p in ptrs:
+                        native.check(L.srtDeviceFree(p))
+                    if not np.array_equal(got.view(np.uint8), want.view(np.uint8)):
+                        errors.append((index, rnd, dt, M, N, K))
+                        return
+            native.check(L.srtStreamSynchronize(stream))
+        except Exception as e:   # noqa: BLE001 -- reported by the parent
+            errors.append((index, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
