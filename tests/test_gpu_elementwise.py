@@ -349,3 +349,65 @@ def test_basic_rnn_cell_fused_and_unfused(dt):
         err = np.abs(H.to64(got) - want)
         bound = 1e-5 if dt == H.F32 else roundings * H.ULP[dt] * np.maximum(np.abs(mm), np.maximum(np.abs(pre), np.abs(want))) + 1e-6
         assert np.all(err <= bound)
+
+
+@pytest.mark.parametrize("seed", [31, 32, 33, 34])
+def test_random_strided_views_bit_exact_and_inside(seed):
+    """Random rank (1-5), extents, storage order (any permutation of the dimensions), padding between rows, start
+    offsets, and inputs broadcast along random dimensions; the result is a padded, permuted view inside a buffer full of a
+    sentinel.  Every supported case must equal the oracle bit for bit inside the view and leave the rest of the result
+    buffer alone; a layout that does not collapse to four dimensions is refused with NotSupported, never miscomputed."""
+    from numpy.lib.stride_tricks import as_strided
+    g = np.random.default_rng(seed)
+    q = srt.current_queue()
+    ran = refused = vector = 0
+
+    def layout(shape, inputs, friendly):
+        rank = len(shape)
+        perm = list(range(rank)) if friendly else list(g.permutation(rank))   # perm[-1] is the innermost dimension in storage
+        strides = [0] * rank
+        running = 1
+        for d in reversed(perm):
+            if inputs and shape[d] > 1 and g.random() < 0.25:
+                continue                                                   # broadcast: stride 0, takes no storage
+            strides[d] = running
+            pad = 0 if g.random() < 0.5 else int(g.integers(1, 4)) * (8 if friendly else 1)
+            running *= shape[d] + pad
+        offset = int(g.integers(0, 4)) * (8 if friendly else 1) + (0 if friendly else int(g.integers(0, 3)))
+        size = offset + sum((e - 1) * s for e, s in zip(shape, strides)) + 1
+        return offset, strides, size
+
+    for case in range(120):
+        dt = DTS[int(g.integers(0, 3))]
+        rank = int(g.integers(1, 6))
+        friendly = g.random() < 0.5
+        shape = [int(g.integers(1, 7)) for _ in range(rank)]
+        shape[-1] = int(g.integers(1, 6)) * 8 if friendly else int(g.integers(1, 40))
+        if rank > 1:
+            shape[int(g.integers(0, rank - 1))] = int(g.integers(1, 40))
+        op, fn = EXACT_BINARY[int(g.integers(0, len(EXACT_BINARY)))]
+        views, gathered = [], []
+        for _ in range(2):
+            off, strides, size = layout(shape, True, friendly)
+            flat = rand_storage(g, (size + 8,), dt)
+            base = srt.Tensor(flat)
+            views.append(srt.Tensor(shape=shape, order=base.order, _storage=base.storage, _offset=off, _strides=strides))
+            gathered.append(np.ascontiguousarray(as_strided(flat[off:], shape, [s * flat.itemsize for s in strides])))
+        off, strides, size = layout(shape, False, friendly)
+        sentinel = H.encode(np.full(size + 8, 12345.0, np.float32), dt)
+        obase = srt.Tensor(sentinel.copy())
+        out = srt.Tensor(shape=shape, order=obase.order, _storage=obase.storage, _offset=off, _strides=strides)
+        what = (seed, case, dt, shape, op, [v.strides for v in views], strides, off)
+        try:
+            getattr(q, fn)(views[0], views[1], out)
+        except srt.NotSupportedError:
+            refused += 1
+            assert rank >= 4, what          # up to three dimensions always collapse to at most four
+            continue
+        want_flat = sentinel.copy()
+        as_strided(want_flat[off:], shape, [s * want_flat.itemsize for s in strides])[...] = ora.elementwise(op, gathered[0], gathered[1])
+        got_flat = obase.array()
+        assert np.array_equal(got_flat.view(np.uint8), want_flat.view(np.uint8)), what
+        ran += 1
+        vector += friendly
+    assert ran >= 90 and vector >= 30, (ran, refused, vector)
