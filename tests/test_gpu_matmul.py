@@ -1330,3 +1330,79 @@ def test_subnormal_operands_and_results_are_kept(dt, scale_a, scale_b, M, N, K, 
     srt.current_queue().matmul(at, False, bt, tb, out)
     want = H.encode(exact.astype(np.float32), dt)
     assert np.array_equal(out.array().view(np.uint8), want.view(np.uint8)), kernel
+
+
+@pytest.mark.parametrize("seed", [41, 42, 43])
+def test_random_operand_and_result_views_through_the_librarys_own_choice(seed):
+    """As the random-problem test, with every tensor a view: row (or, in column-major order, column) pitches wider than the
+    extent by nothing, a multiple of eight or an odd count, first elements at aligned and unaligned offsets, batches
+    lying apart with gaps or -- for an operand -- repeated with stride 0, all of it inside buffers that hold a sentinel
+    elsewhere.  Pitches and alignment decide which kernels qualify; the result must be exact inside its view and the rest
+    of its buffer untouched, whichever kernel that leaves."""
+    from numpy.lib.stride_tricks import as_strided
+    g = np.random.default_rng(seed)
+    q = srt.current_queue()
+    seen = set()
+
+    def logu(lo, hi):
+        return int(np.exp(g.uniform(np.log(lo), np.log(hi + 1))))
+
+    def strided(rows, cols, batch, col_major, may_repeat, aligned):
+        unit = 8 if aligned else 1
+        pad = int(g.choice([0, 0, 8, 24] if aligned else [0, 1, 3, 8, 13]))
+        lead, other = (rows, cols) if col_major else (cols, rows)         # contiguous extent, strided extent
+        pitch = lead + pad
+        offset = int(g.integers(0, 4)) * unit
+        matrix = pitch * other
+        bstride = 0 if (may_repeat and batch > 1 and g.random() < 0.3) else matrix + int(g.integers(0, 3)) * pitch
+        size = offset + (batch - 1) * bstride + matrix + 8
+        strides2 = [1, pitch] if col_major else [pitch, 1]
+        return offset, ([bstride] + strides2) if batch > 1 else strides2, size
+
+    for case in range(150):
+        dt = (H.F32, H.BF16, H.F16)[int(g.integers(0, 3))]
+        ta, tb = bool(g.integers(0, 2)), bool(g.integers(0, 2))
+        batch = int(g.choice([1, 1, 2, 4]))
+        aligned = g.random() < 0.6
+        M, N, K = logu(1, 600), logu(1, 600), logu(1, 2100)
+        if aligned:
+            M, N, K = max(8, M // 8 * 8), max(8, N // 8 * 8), max(8, K // 8 * 8)
+        if g.random() < 0.3:
+            K = max(64, K // 64 * 64)
+        col_major = g.random() < 0.25
+        order = srt.Order.col if col_major else srt.Order.row
+        lead = [batch] if batch > 1 else []
+        tensors, dense = [], []
+        for (rows, cols, repeat) in [((K, M) if ta else (M, K)) + (True,), ((N, K) if tb else (K, N)) + (True,)]:
+            off, strides, size = strided(rows, cols, batch, col_major, repeat, aligned)
+            flat = H.encode(np.full(size, 77.0, np.float32), dt)
+            view = as_strided(flat[off:], lead + [rows, cols], [s * flat.itemsize for s in strides])
+            shape_written = [1 if s == 0 else e for e, s in zip(lead + [rows, cols], strides)]
+            values = g.integers(-2, 3, shape_written).astype(np.float32)
+            view[tuple(slice(0, e) for e in shape_written)] = H.encode(values, dt)
+            base = srt.Tensor(flat)
+            tensors.append(srt.Tensor(shape=lead + [rows, cols], order=order, _storage=base.storage, _offset=off, _strides=strides))
+            full = np.broadcast_to(values, lead + [rows, cols]).astype(np.float64)
+            dense.append(full.reshape(batch, rows, cols))
+        a64 = dense[0].transpose(0, 2, 1) if ta else dense[0]
+        b64 = dense[1].transpose(0, 2, 1) if tb else dense[1]
+        bias = g.integers(-3, 4, N).astype(np.float32)
+        with_bias = bool(g.integers(0, 2))
+        relu = bool(g.integers(0, 2))
+        exact = a64 @ b64 + (bias[None, None, :] if with_bias else 0.0)
+        if relu:
+            exact = np.maximum(exact, 0.0)
+        off, strides, size = strided(M, N, batch, col_major, False, aligned)
+        sentinel = H.encode(np.full(size, 12345.0, np.float32), dt)
+        obase = srt.Tensor(sentinel.copy())
+        out = srt.Tensor(shape=lead + [M, N], order=order, _storage=obase.storage, _offset=off, _strides=strides)
+        want_flat = sentinel.copy()
+        as_strided(want_flat[off:], lead + [M, N], [s * want_flat.itemsize for s in strides])[...] = \
+            H.encode(exact.astype(np.float32), dt).reshape(lead + [M, N])
+        what = (seed, case, dt, ta, tb, batch, M, N, K, col_major, aligned, [t.strides for t in tensors], strides, off, with_bias, relu)
+        kernel = query_kernel(tensors[0], ta, tensors[1], tb, out)
+        seen.add(kernel)
+        q.matmul(tensors[0], ta, tensors[1], tb, out, bias=srt.Tensor(H.encode(bias, dt)) if with_bias else None,
+                 activation=srt.ActivationType.relu if relu else srt.ActivationType.identity)
+        assert np.array_equal(obase.array().view(np.uint8), want_flat.view(np.uint8)), what + (kernel,)
+    assert len(seen) >= 5, seen
