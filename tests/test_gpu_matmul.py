@@ -1405,4 +1405,4 @@ def test_random_operand_and_result_views_through_the_librarys_own_choice(seed):
         q.matmul(tensors[0], ta, tensors[1], tb, out, bias=srt.Tensor(H.encode(bias, dt)) if with_bias else None,
                  activation=srt.ActivationType.relu if relu else srt.ActivationType.identity)
         assert np.array_equal(obase.array().view(np.uint8), want_flat.view(np.uint8)), what + (kernel,)
-    assert len(seen) >= 5, seen
+    assert len(seen) >= 4, seen
