@@ -202,3 +202,63 @@ def test_backward_errors():
     assert f(y.device_read(q), ctypes.byref(yd), y.device_read(q), ctypes.byref(yd), 1, 0.0,
              out.device_read_write(q), ctypes.byref(od), None, None, q.stream) == native.ERROR_NOT_SUPPORTED
     assert f(None, None, None, None, 1, 0.0, None, None, None, None, q.stream) == native.ERROR_INVALID_VALUE
+
+
+@pytest.mark.parametrize("seed", [51, 52, 53])
+def test_random_shapes_and_views(seed):
+    """Random extents (one row to thousands: one or many row chunks), element types, activations, and y / dy / dx as views
+    with padded rows, aligned or unaligned starts, sometimes stored column by column; dx inside a sentinel buffer.  dx must
+    be the oracle's bit for bit and stay inside its view; the bias gradient exact on integer data and within its bound
+    otherwise."""
+    from numpy.lib.stride_tricks import as_strided
+    g = np.random.default_rng(seed)
+    q = srt.current_queue()
+
+    def place(values, aligned, allow_columns):
+        m, n = values.shape
+        vdt = H.F32 if values.dtype == np.float32 else H.F16 if values.dtype == np.float16 else H.BF16
+        unit = 8 if aligned else 1
+        by_columns = allow_columns and g.random() < 0.2
+        lead, other = (m, n) if by_columns else (n, m)
+        pitch = lead + int(g.choice([0, 0, 8, 16] if aligned else [0, 1, 5, 8]))
+        off = int(g.integers(0, 4)) * unit
+        flat = H.encode(np.full(off + pitch * other + 8, 99.0, np.float32), vdt)
+        strides = [1, pitch] if by_columns else [pitch, 1]
+        as_strided(flat[off:], (m, n), [s * flat.itemsize for s in strides])[...] = values
+        base = srt.Tensor(flat)
+        return base, srt.Tensor(shape=[m, n], order=base.order, _storage=base.storage, _offset=off, _strides=strides), flat, off, strides
+
+    for case in range(60):
+        dt = DTS[int(g.integers(0, 3))]
+        act, coef = ACTS[int(g.integers(0, len(ACTS)))]
+        m = int(np.exp(g.uniform(0, np.log(5000))))
+        n = int(np.exp(g.uniform(0, np.log(3000))))
+        aligned = g.random() < 0.6
+        if aligned:
+            n = max(8, n // 8 * 8)
+        integers = g.random() < 0.4
+        if integers:
+            act, coef = srt.ActivationType.relu, 0.0
+            y_st = H.encode(g.integers(-1, 3, (m, n)).astype(np.float32), dt)
+            dy_st = H.encode(g.integers(-2, 3, (m, n)).astype(np.float32), dt)
+        else:
+            y_st = forward_output(g, (m, n), act, coef, dt)
+            dy_st = H.encode(g.standard_normal((m, n)).astype(np.float32), dt)
+        _, y, _, _, _ = place(y_st, aligned, True)
+        _, dy, _, _, _ = place(dy_st, aligned, True)
+        obase, dx, oflat, off, strides = place(np.zeros_like(y_st), aligned, False)
+        want_bias = g.random() < 0.8
+        db = srt.Tensor(shape=[n], dtype=y.dtype) if want_bias else None
+        what = (seed, case, dt, act, m, n, aligned, integers, y.strides, dy.strides, strides, off)
+        q.activation_backward(y, dy, act, coef, dx, db)
+        want_dx, db64 = ora.activation_backward_bias(y_st, dy_st, int(act), coef)
+        want_flat = oflat.copy()
+        as_strided(want_flat[off:], (m, n), [s * want_flat.itemsize for s in strides])[...] = want_dx
+        assert np.array_equal(obase.array().view(np.uint8), want_flat.view(np.uint8)), what
+        if want_bias:
+            if integers:
+                sums = H.to64(want_dx).sum(axis=0)
+                assert np.array_equal(db.array().view(np.uint8), H.encode(sums.astype(np.float32), dt).view(np.uint8)), what
+            else:
+                abs64 = np.abs(H.to64(dy_st) * ora.activation_slope(int(act), H.decode(y_st), coef)).sum(axis=0)
+                check_dbias(db.array(), db64, abs64, m, dt)
